@@ -1,0 +1,288 @@
+// context.hip — bridge lifecycle, device buffers, events, workspace, synthetic-data fills.
+// Interface style after the reference's C-ABI (bridge/ane_bridge.h:11-98, bridge/ane_bridge.m:33-57,
+// 233-251): idempotent init returning 0/-1, opaque handles, NULL-safe frees, one stderr line per error.
+#include "common.h"
+
+#include <stdarg.h>
+#include <stdlib.h>
+
+Mi355Ctx g_ctx = {};
+static char g_err[512] = "";
+
+int mi355_fail(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    fprintf(stderr, "mi355_bridge: %s\n", g_err);
+    return -1;
+}
+
+bool mi355_ready(const char *who) {
+    if (g_ctx.ready) return true;
+    if (mi355_init() == 0) return true;
+    mi355_fail("%s: no usable GPU (mi355_init failed)", who);
+    return false;
+}
+
+void *mi355_ws(size_t bytes) {
+    if (bytes <= g_ctx.ws_bytes && g_ctx.ws) return g_ctx.ws;
+    size_t want = (bytes + 0xFFFFF) & ~(size_t)0xFFFFF;   // 1 MiB granules
+    if (g_ctx.ws) {
+        (void)hipStreamSynchronize(g_ctx.stream);
+        (void)hipFree(g_ctx.ws);
+        g_ctx.ws = nullptr;
+        g_ctx.ws_bytes = 0;
+    }
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, want);
+    if (e != hipSuccess) {
+        mi355_fail("workspace hipMalloc(%zu): %s", want, hipGetErrorString(e));
+        return nullptr;
+    }
+    g_ctx.ws = p;
+    g_ctx.ws_bytes = want;
+    return p;
+}
+
+MI355_API int mi355_init(void) {
+    if (g_ctx.ready) return 0;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return mi355_fail("init: no HIP device (%s)", e == hipSuccess ? "count 0" : hipGetErrorString(e));
+    }
+    HIP_OK(hipSetDevice(0));
+    hipDeviceProp_t prop;
+    HIP_OK(hipGetDeviceProperties(&prop, 0));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return mi355_fail("init: device 0 is %s; this library holds gfx950 code only", prop.gcnArchName);
+    g_ctx.device = 0;
+    g_ctx.num_cu = prop.multiProcessorCount;
+    g_ctx.stream = nullptr;
+    g_ctx.ws = nullptr;
+    g_ctx.ws_bytes = 0;
+    g_ctx.ready = true;
+    g_err[0] = 0;
+    return 0;
+}
+
+void mi355_free_caches(void);   // rope tables, host drop-in staging (other translation units)
+
+MI355_API void mi355_shutdown(void) {
+    if (!g_ctx.ready) return;
+    (void)hipDeviceSynchronize();
+    mi355_free_caches();
+    if (g_ctx.ws) (void)hipFree(g_ctx.ws);
+    g_ctx = Mi355Ctx{};
+}
+
+MI355_API const char *mi355_last_error(void) { return g_err; }
+
+MI355_API int mi355_device_info(char *name, size_t name_len, double *peak_hbm_gbs, int *compute_units) {
+    if (!mi355_ready("device_info")) return -1;
+    hipDeviceProp_t prop;
+    HIP_OK(hipGetDeviceProperties(&prop, g_ctx.device));
+    if (name && name_len) {
+        snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+    }
+    if (peak_hbm_gbs) {
+        // memoryClockRate is in kHz, bus width in bits; HBM transfers twice per clock.
+        *peak_hbm_gbs = 2.0 * (double)prop.memoryClockRate * 1e3 * ((double)prop.memoryBusWidth / 8.0) / 1e9;
+    }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    return 0;
+}
+
+MI355_API int mi355_set_stream(void *hip_stream) {
+    if (!mi355_ready("set_stream")) return -1;
+    g_ctx.stream = (hipStream_t)hip_stream;
+    return 0;
+}
+
+MI355_API int mi355_sync(void) {
+    if (!mi355_ready("sync")) return -1;
+    HIP_OK(hipStreamSynchronize(g_ctx.stream));
+    return 0;
+}
+
+MI355_API int mi355_workspace_reserve(size_t bytes) {
+    if (!mi355_ready("workspace_reserve")) return -1;
+    return mi355_ws(bytes) ? 0 : -1;
+}
+
+MI355_API int mi355_tune_set(const char *key, int value) {
+    if (!key) return -1;
+    struct { const char *k; int *v; } tab[] = {
+        {"rms_lpr", &g_ctx.rms_lpr}, {"rms_threads", &g_ctx.rms_threads},
+        {"ew_unroll", &g_ctx.ew_unroll}, {"ew_threads", &g_ctx.ew_threads},
+        {"ce_rows", &g_ctx.ce_rows}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
+        {"gather_tile", &g_ctx.gather_tile}, {"nt_store", &g_ctx.nt_store},
+    };
+    for (auto &t : tab)
+        if (strcmp(t.k, key) == 0) { *t.v = value; return 0; }
+    return -1;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Buffers
+// ---------------------------------------------------------------------------------------------
+struct mi355_buf {
+    void *dev;
+    size_t bytes;
+};
+
+MI355_API mi355_buf *mi355_buf_alloc(size_t bytes) {
+    if (!mi355_ready("buf_alloc")) return nullptr;
+    if (bytes == 0) { mi355_fail("buf_alloc: zero bytes"); return nullptr; }
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) { mi355_fail("buf_alloc(%zu): %s", bytes, hipGetErrorString(e)); return nullptr; }
+    e = hipMemsetAsync(p, 0, bytes, g_ctx.stream);
+    if (e != hipSuccess) { (void)hipFree(p); mi355_fail("buf_alloc memset: %s", hipGetErrorString(e)); return nullptr; }
+    mi355_buf *b = (mi355_buf *)malloc(sizeof(mi355_buf));
+    if (!b) { (void)hipFree(p); return nullptr; }
+    b->dev = p;
+    b->bytes = bytes;
+    return b;
+}
+
+MI355_API void mi355_buf_free(mi355_buf *b) {
+    if (!b) return;
+    if (g_ctx.ready && b->dev) {
+        (void)hipStreamSynchronize(g_ctx.stream);
+        (void)hipFree(b->dev);
+    }
+    free(b);
+}
+
+MI355_API void *mi355_buf_devptr(mi355_buf *b) { return b ? b->dev : nullptr; }
+MI355_API size_t mi355_buf_bytes(mi355_buf *b) { return b ? b->bytes : 0; }
+
+MI355_API void mi355_buf_write(mi355_buf *b, size_t offset, const void *src, size_t bytes) {
+    if (!b || !src || !g_ctx.ready || offset > b->bytes || bytes > b->bytes - offset || bytes == 0) return;
+    hipError_t e = hipMemcpyAsync((char *)b->dev + offset, src, bytes, hipMemcpyHostToDevice, g_ctx.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(g_ctx.stream);
+    if (e != hipSuccess) mi355_fail("buf_write: %s", hipGetErrorString(e));
+}
+
+MI355_API void mi355_buf_read(mi355_buf *b, size_t offset, void *dst, size_t bytes) {
+    if (!b || !dst || !g_ctx.ready || offset > b->bytes || bytes > b->bytes - offset || bytes == 0) return;
+    hipError_t e = hipMemcpyAsync(dst, (const char *)b->dev + offset, bytes, hipMemcpyDeviceToHost, g_ctx.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(g_ctx.stream);
+    if (e != hipSuccess) mi355_fail("buf_read: %s", hipGetErrorString(e));
+}
+
+__global__ void fill_zero_kernel(v4f *p, size_t n4, char *tail, size_t ntail) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    v4f z = {0.f, 0.f, 0.f, 0.f};
+    for (; i < n4; i += stride) p[i] = z;
+    if (blockIdx.x == 0 && threadIdx.x < ntail) tail[threadIdx.x] = 0;
+}
+
+MI355_API int mi355_buf_zero(mi355_buf *b) {
+    if (!mi355_ready("buf_zero")) return -1;
+    if (!b) return mi355_fail("buf_zero: NULL buffer");
+    // a fill kernel rather than hipMemsetAsync, so the call is safe inside a captured graph
+    size_t n4 = b->bytes / 16, ntail = b->bytes % 16;
+    size_t blocks = ceil_div(n4 ? n4 : 1, 256);
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, g_ctx.stream,
+                       (v4f *)b->dev, n4, (char *)b->dev + n4 * 16, ntail);
+    LAUNCH_OK("buf_zero");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Events
+// ---------------------------------------------------------------------------------------------
+struct mi355_event {
+    hipEvent_t ev;
+};
+
+MI355_API mi355_event *mi355_event_create(void) {
+    if (!mi355_ready("event_create")) return nullptr;
+    mi355_event *e = (mi355_event *)malloc(sizeof(mi355_event));
+    if (!e) return nullptr;
+    if (hipEventCreate(&e->ev) != hipSuccess) { free(e); mi355_fail("event_create failed"); return nullptr; }
+    return e;
+}
+
+MI355_API void mi355_event_destroy(mi355_event *e) {
+    if (!e) return;
+    if (g_ctx.ready) (void)hipEventDestroy(e->ev);
+    free(e);
+}
+
+MI355_API int mi355_event_record(mi355_event *e) {
+    if (!mi355_ready("event_record")) return -1;
+    if (!e) return mi355_fail("event_record: NULL event");
+    HIP_OK(hipEventRecord(e->ev, g_ctx.stream));
+    return 0;
+}
+
+MI355_API float mi355_event_elapsed_ms(mi355_event *start, mi355_event *stop) {
+    if (!g_ctx.ready || !start || !stop) return -1.0f;
+    if (hipEventSynchronize(stop->ev) != hipSuccess) return -1.0f;
+    float ms = -1.0f;
+    if (hipEventElapsedTime(&ms, start->ev, stop->ev) != hipSuccess) return -1.0f;
+    return ms;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Synthetic data: element i of stream `seed` is a pure function of (seed, i).
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint64_t splitmix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+__global__ void fill_normal_kernel(float *p, size_t n, uint64_t seed, float mean, float std) {
+    size_t pair = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t npair = (n + 1) / 2;
+    for (; pair < npair; pair += stride) {
+        uint64_t r = splitmix64(seed * 0xD1342543DE82EF95ull + pair);
+        float u1 = ((float)(uint32_t)(r >> 40) + 1.0f) * (1.0f / 16777217.0f);   // (0,1)
+        float u2 = (float)(uint32_t)((r >> 8) & 0xFFFFFF) * (1.0f / 16777216.0f);
+        float rad = sqrtf(-2.0f * logf(u1));
+        float sn, cs;
+        sincosf(6.283185307179586f * u2, &sn, &cs);
+        p[2 * pair] = mean + std * rad * cs;
+        if (2 * pair + 1 < n) p[2 * pair + 1] = mean + std * rad * sn;
+    }
+}
+
+__global__ void fill_randint_kernel(int32_t *p, size_t n, uint64_t seed, int32_t lo, uint32_t span) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        uint64_t r = splitmix64(seed * 0xD1342543DE82EF95ull + i);
+        p[i] = lo + (int32_t)(((r >> 32) * (uint64_t)span) >> 32);
+    }
+}
+
+MI355_API int mi355_fill_normal_dev(float *p, size_t n, uint64_t seed, float mean, float std) {
+    if (!mi355_ready("fill_normal")) return -1;
+    if (!p || n == 0) return mi355_fail("fill_normal: NULL pointer or empty");
+    size_t blocks = ceil_div((n + 1) / 2, 256);
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(fill_normal_kernel, dim3((unsigned)blocks), dim3(256), 0, g_ctx.stream, p, n, seed, mean, std);
+    LAUNCH_OK("fill_normal");
+    return 0;
+}
+
+MI355_API int mi355_fill_randint_dev(int32_t *p, size_t n, uint64_t seed, int32_t lo, int32_t hi) {
+    if (!mi355_ready("fill_randint")) return -1;
+    if (!p || n == 0 || hi <= lo) return mi355_fail("fill_randint: bad arguments");
+    size_t blocks = ceil_div(n, 256);
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(fill_randint_kernel, dim3((unsigned)blocks), dim3(256), 0, g_ctx.stream, p, n, seed, lo,
+                       (uint32_t)(hi - lo));
+    LAUNCH_OK("fill_randint");
+    return 0;
+}

@@ -1,0 +1,546 @@
+// eltwise.hip — streaming elementwise ops: SwiGLU gate fwd/bwd, residual family, RoPE, INT8.
+//
+// All of these are pure HBM streams (<= ~30 flops per 12-20 bytes), so the design is the same
+// for each: 128-bit loads and stores, every load instruction of a wave covering one contiguous
+// 1 KiB run, UNROLL independent loads in flight per lane before the first use, and enough
+// workgroups (one pass, no grid-stride loop) to cover the 256 compute units many times over.
+#include "common.h"
+
+#include <math.h>
+
+namespace {
+
+constexpr int EW_THREADS = 256;
+
+__device__ __forceinline__ float sigmoid_ref(float h) {
+    // 1/(1+exp(-h)) with the library expf and an IEEE division, as the reference's
+    // vvexpf + vvrecf sequence (training/training_dynamic/train.m:541-544)
+    return 1.0f / (1.0f + expf(-h));
+}
+
+// ---- SwiGLU forward: out = (h1*sig(h1))*h3  (mil_dynamic.h:264-266) ----
+template <int UNROLL>
+__global__ __launch_bounds__(EW_THREADS) void swiglu_fwd_kernel(float *__restrict__ out, const float *__restrict__ h1,
+                                                                const float *__restrict__ h3, size_t n4) {
+    const size_t base = (size_t)blockIdx.x * (EW_THREADS * UNROLL) + threadIdx.x;
+    v4f a[UNROLL], b[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) {
+            a[u] = ld4_nt(h1 + 4 * i);
+            b[u] = ld4_nt(h3 + 4 * i);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) {
+            v4f o;
+#pragma unroll
+            for (int j = 0; j < 4; j++) o[j] = (a[u][j] * sigmoid_ref(a[u][j])) * b[u][j];
+            st4_nt(out + 4 * i, o);
+        }
+    }
+}
+
+__global__ void swiglu_fwd_scalar(float *out, const float *h1, const float *h3, size_t lo, size_t n) {
+    size_t i = lo + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = (h1[i] * sigmoid_ref(h1[i])) * h3[i];
+}
+
+// ---- SwiGLU backward (train.m:537-554) ----
+__device__ __forceinline__ void swiglu_bwd_elem(float d, float h, float g, float &dh1, float &dh3) {
+    float sig = sigmoid_ref(h);
+    dh3 = d * (h * sig);
+    float u = -(sig + -1.0f);
+    u = h * u;
+    u = u + 1.0f;
+    u = sig * u;
+    dh1 = (d * g) * u;
+}
+
+template <int UNROLL>
+__global__ __launch_bounds__(EW_THREADS) void swiglu_bwd_kernel(float *__restrict__ dh1, float *__restrict__ dh3,
+                                                                const float *__restrict__ ds,
+                                                                const float *__restrict__ h1,
+                                                                const float *__restrict__ h3, size_t n4) {
+    const size_t base = (size_t)blockIdx.x * (EW_THREADS * UNROLL) + threadIdx.x;
+    v4f a[UNROLL], b[UNROLL], d[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) {
+            d[u] = ld4_nt(ds + 4 * i);
+            a[u] = ld4_nt(h1 + 4 * i);
+            b[u] = ld4_nt(h3 + 4 * i);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) {
+            v4f o1, o3;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float x1, x3;
+                swiglu_bwd_elem(d[u][j], a[u][j], b[u][j], x1, x3);
+                o1[j] = x1;
+                o3[j] = x3;
+            }
+            st4_nt(dh1 + 4 * i, o1);
+            st4_nt(dh3 + 4 * i, o3);
+        }
+    }
+}
+
+__global__ void swiglu_bwd_scalar(float *dh1, float *dh3, const float *ds, const float *h1, const float *h3,
+                                  size_t lo, size_t n) {
+    size_t i = lo + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        float x1, x3;
+        swiglu_bwd_elem(ds[i], h1[i], h3[i], x1, x3);
+        dh1[i] = x1;
+        dh3[i] = x3;
+    }
+}
+
+// ---- residual family ----
+template <int MODE, int UNROLL>
+__global__ __launch_bounds__(EW_THREADS) void axpby_kernel(float *y, const float *a, const float *b, float alpha,
+                                                           size_t n4) {
+    const size_t base = (size_t)blockIdx.x * (EW_THREADS * UNROLL) + threadIdx.x;
+    v4f av[UNROLL], bv[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) {
+            av[u] = ld4(a + 4 * i);
+            if (MODE != 1) bv[u] = ld4(b + 4 * i);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) {
+            v4f o;
+            if (MODE == 0) o = bv[u] * alpha + av[u];
+            else if (MODE == 1) o = av[u] * alpha;
+            else o = av[u] + bv[u];
+            st4(y + 4 * i, o);
+        }
+    }
+}
+
+template <int MODE>
+__global__ void axpby_scalar(float *y, const float *a, const float *b, float alpha, size_t lo, size_t n) {
+    size_t i = lo + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        if (MODE == 0) y[i] = b[i] * alpha + a[i];
+        else if (MODE == 1) y[i] = a[i] * alpha;
+        else y[i] = a[i] + b[i];
+    }
+}
+
+// ---- RoPE on interleaved row pairs; one thread = one pair of rows x VEC columns ----
+// rows: all (batch, head, pair) triples of Q then of K; tables [hd/2][S].
+template <int VEC>
+__global__ __launch_bounds__(EW_THREADS) void rope_kernel(float *q_out, float *k_out, const float *q_in,
+                                                          const float *k_in, int heads, int kv_heads, int hd, int S,
+                                                          int batch, const float *__restrict__ cos_t,
+                                                          const float *__restrict__ sin_t, float sgn, size_t total) {
+    const int cols = (S + VEC - 1) / VEC;   // column groups per row
+    const size_t idx = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;
+    if (idx >= total) return;
+    const int cg = (int)(idx % cols);
+    size_t pr = idx / cols;   // pair-row index
+    const int half = hd >> 1;
+    const size_t q_rows = (size_t)batch * heads * half;
+    const float *in;
+    float *out;
+    int i;
+    size_t row;
+    if (pr < q_rows) {
+        i = (int)(pr % half);
+        row = (pr / half) * hd + 2 * i;   // (b*heads + h)*hd + 2i
+        in = q_in; out = q_out;
+    } else {
+        pr -= q_rows;
+        i = (int)(pr % half);
+        row = (pr / half) * hd + 2 * i;
+        in = k_in; out = k_out;
+    }
+    const int s = cg * VEC;
+    const size_t o0 = row * S + s, o1 = o0 + S;
+    const size_t t = (size_t)i * S + s;
+    if constexpr (VEC == 4) {
+        v4f v0 = ld4(in + o0), v1 = ld4(in + o1);
+        v4f c = ld4(cos_t + t), sn = ld4(sin_t + t) * sgn;
+        // forward (sgn=+1): x0*c - x1*s, x0*s + x1*c ; backward (sgn=-1): x0*c + x1*s, -x0*s + x1*c
+        v4f r0 = v0 * c - v1 * sn;
+        v4f r1 = v0 * sn + v1 * c;
+        st4(out + o0, r0);
+        st4(out + o1, r1);
+    } else {
+        float v0 = in[o0], v1 = in[o1];
+        float c = cos_t[t], sn = sin_t[t] * sgn;
+        out[o0] = v0 * c - v1 * sn;
+        out[o1] = v0 * sn + v1 * c;
+    }
+}
+
+// ---- INT8 ----
+// max|x| over the tensor; non-negative floats order like their bit patterns, so an integer
+// atomicMax gives an exact, order-independent result.
+__global__ __launch_bounds__(EW_THREADS) void absmax_kernel(unsigned int *out_bits, const float *__restrict__ x,
+                                                            size_t n, size_t n4) {
+    __shared__ float red[EW_THREADS / 64];
+    float m = 0.f;
+    const size_t stride = (size_t)gridDim.x * EW_THREADS;
+    for (size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n4; i += stride) {
+        v4f v = ld4(x + 4 * i);
+#pragma unroll
+        for (int j = 0; j < 4; j++) m = fmaxf(m, fabsf(v[j]));
+    }
+    if (blockIdx.x == 0)
+        for (size_t i = n4 * 4 + threadIdx.x; i < n; i += EW_THREADS) m = fmaxf(m, fabsf(x[i]));
+#pragma unroll
+    for (int k = 1; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 1; k < EW_THREADS / 64; k++) m = fmaxf(m, red[k]);
+        atomicMax(out_bits, __float_as_uint(m));
+    }
+}
+
+__global__ void absmax_scalar_kernel(unsigned int *out_bits, const float *x, size_t n) {
+    float m = 0.f;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        m = fmaxf(m, fabsf(x[i]));
+    atomicMax(out_bits, __float_as_uint(m));
+}
+
+__global__ void scale_from_absmax_kernel(float *scale) {
+    float s = *scale / 127.0f;        // *scale holds max|x| (bits written by atomicMax)
+    if (s == 0.0f) s = 1.0f;
+    *scale = s;
+}
+
+__device__ __forceinline__ int quant1(float x, float scale, int rounding) {
+    float v = x / scale;              // IEEE division, as the reference (bridge/ane_bridge.m:361)
+    v = fminf(v, 127.0f);
+    v = fmaxf(v, -128.0f);
+    if (rounding == 1) return (int)(v + (v >= 0 ? 0.5f : -0.5f));   // half away from zero, then truncate
+    return (int)rintf(v);                                            // half to even
+}
+
+template <int UNROLL>
+__global__ __launch_bounds__(EW_THREADS) void quant_kernel(int *__restrict__ q4, const float *__restrict__ x,
+                                                           const float *__restrict__ scale_p, size_t n4,
+                                                           int rounding) {
+    const float scale = *scale_p;
+    const size_t base = (size_t)blockIdx.x * (EW_THREADS * UNROLL) + threadIdx.x;
+    v4f a[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) a[u] = ld4(x + 4 * i);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) {
+            unsigned int pk = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) pk |= ((unsigned int)(quant1(a[u][j], scale, rounding) & 0xFF)) << (8 * j);
+            q4[i] = (int)pk;
+        }
+    }
+}
+
+__global__ void quant_scalar(int8_t *q, const float *x, const float *scale_p, size_t lo, size_t n, int rounding) {
+    size_t i = lo + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) q[i] = (int8_t)quant1(x[i], *scale_p, rounding);
+}
+
+template <int UNROLL>
+__global__ __launch_bounds__(EW_THREADS) void dequant_kernel(float *__restrict__ x, const int *__restrict__ q4,
+                                                             const float *__restrict__ scale_p, size_t n4) {
+    const float scale = *scale_p;
+    const size_t base = (size_t)blockIdx.x * (EW_THREADS * UNROLL) + threadIdx.x;
+    int a[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) a[u] = q4[i];
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) {
+            v4f o;
+#pragma unroll
+            for (int j = 0; j < 4; j++) o[j] = (float)(int)(signed char)((a[u] >> (8 * j)) & 0xFF) * scale;
+            st4(x + 4 * i, o);
+        }
+    }
+}
+
+__global__ void dequant_scalar(float *x, const int8_t *q, const float *scale_p, size_t lo, size_t n) {
+    size_t i = lo + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = (float)q[i] * *scale_p;
+}
+
+inline int pick_unroll(size_t n4, int deflt) {
+    int u = g_ctx.ew_unroll ? g_ctx.ew_unroll : deflt;
+    if (u != 1 && u != 2 && u != 4 && u != 8) u = deflt;
+    // small tensors: favour more workgroups over deeper unrolling
+    while (u > 1 && ceil_div(n4, (size_t)EW_THREADS * u) < 2048) u >>= 1;
+    return u;
+}
+
+#define EW_LAUNCH(KERNEL_T, unroll, n4, ...)                                                               \
+    do {                                                                                                   \
+        const unsigned _g1 = (unsigned)ceil_div(n4, (size_t)EW_THREADS * 1);                               \
+        switch (unroll) {                                                                                  \
+            case 8: hipLaunchKernelGGL((KERNEL_T<8>), dim3((unsigned)ceil_div(n4, (size_t)EW_THREADS * 8)), \
+                                       dim3(EW_THREADS), 0, g_ctx.stream, __VA_ARGS__); break;             \
+            case 4: hipLaunchKernelGGL((KERNEL_T<4>), dim3((unsigned)ceil_div(n4, (size_t)EW_THREADS * 4)), \
+                                       dim3(EW_THREADS), 0, g_ctx.stream, __VA_ARGS__); break;             \
+            case 2: hipLaunchKernelGGL((KERNEL_T<2>), dim3((unsigned)ceil_div(n4, (size_t)EW_THREADS * 2)), \
+                                       dim3(EW_THREADS), 0, g_ctx.stream, __VA_ARGS__); break;             \
+            default: hipLaunchKernelGGL((KERNEL_T<1>), dim3(_g1), dim3(EW_THREADS), 0, g_ctx.stream,       \
+                                        __VA_ARGS__); break;                                               \
+        }                                                                                                  \
+    } while (0)
+
+__global__ void fill_zero_u32(unsigned int *p) { *p = 0u; }
+
+}   // namespace
+
+// n4 vector part + scalar tail split used by every elementwise op
+static inline void split_vec(size_t n, bool vec_ok, size_t &n4, size_t &tail_lo) {
+    n4 = vec_ok ? n / 4 : 0;
+    tail_lo = n4 * 4;
+}
+
+MI355_API int mi355_swiglu_fwd_dev(float *out, const float *h1, const float *h3, size_t n) {
+    if (!mi355_ready("swiglu_fwd")) return -1;
+    if (!out || !h1 || !h3) return mi355_fail("swiglu_fwd: NULL pointer");
+    if (n == 0) return mi355_fail("swiglu_fwd: empty tensor");
+    size_t n4, lo;
+    split_vec(n, aligned16(out) && aligned16(h1) && aligned16(h3), n4, lo);
+    if (n4) {
+        const int u = pick_unroll(n4, 4);
+        EW_LAUNCH(swiglu_fwd_kernel, u, n4, out, h1, h3, n4);
+        LAUNCH_OK("swiglu_fwd");
+    }
+    if (lo < n) {
+        hipLaunchKernelGGL(swiglu_fwd_scalar, dim3((unsigned)ceil_div(n - lo, 256)), dim3(256), 0, g_ctx.stream, out,
+                           h1, h3, lo, n);
+        LAUNCH_OK("swiglu_fwd tail");
+    }
+    return 0;
+}
+
+MI355_API int mi355_swiglu_bwd_dev(float *dh1, float *dh3, const float *dsilu, const float *h1, const float *h3,
+                                   size_t n) {
+    if (!mi355_ready("swiglu_bwd")) return -1;
+    if (!dh1 || !dh3 || !dsilu || !h1 || !h3) return mi355_fail("swiglu_bwd: NULL pointer");
+    if (n == 0) return mi355_fail("swiglu_bwd: empty tensor");
+    size_t n4, lo;
+    split_vec(n, aligned16(dh1) && aligned16(dh3) && aligned16(dsilu) && aligned16(h1) && aligned16(h3), n4, lo);
+    if (n4) {
+        const int u = pick_unroll(n4, 2);
+        EW_LAUNCH(swiglu_bwd_kernel, u, n4, dh1, dh3, dsilu, h1, h3, n4);
+        LAUNCH_OK("swiglu_bwd");
+    }
+    if (lo < n) {
+        hipLaunchKernelGGL(swiglu_bwd_scalar, dim3((unsigned)ceil_div(n - lo, 256)), dim3(256), 0, g_ctx.stream, dh1,
+                           dh3, dsilu, h1, h3, lo, n);
+        LAUNCH_OK("swiglu_bwd tail");
+    }
+    return 0;
+}
+
+template <int MODE>
+static int axpby_run(float *y, const float *a, const float *b, float alpha, size_t n) {
+    size_t n4, lo;
+    split_vec(n, aligned16(y) && aligned16(a) && (MODE == 1 || aligned16(b)), n4, lo);
+    if (n4) {
+        const int u = pick_unroll(n4, 4);
+        switch (u) {
+            case 8: hipLaunchKernelGGL((axpby_kernel<MODE, 8>), dim3((unsigned)ceil_div(n4, (size_t)EW_THREADS * 8)), dim3(EW_THREADS), 0, g_ctx.stream, y, a, b, alpha, n4); break;
+            case 4: hipLaunchKernelGGL((axpby_kernel<MODE, 4>), dim3((unsigned)ceil_div(n4, (size_t)EW_THREADS * 4)), dim3(EW_THREADS), 0, g_ctx.stream, y, a, b, alpha, n4); break;
+            case 2: hipLaunchKernelGGL((axpby_kernel<MODE, 2>), dim3((unsigned)ceil_div(n4, (size_t)EW_THREADS * 2)), dim3(EW_THREADS), 0, g_ctx.stream, y, a, b, alpha, n4); break;
+            default: hipLaunchKernelGGL((axpby_kernel<MODE, 1>), dim3((unsigned)ceil_div(n4, (size_t)EW_THREADS)), dim3(EW_THREADS), 0, g_ctx.stream, y, a, b, alpha, n4); break;
+        }
+        LAUNCH_OK("axpby");
+    }
+    if (lo < n) {
+        hipLaunchKernelGGL((axpby_scalar<MODE>), dim3((unsigned)ceil_div(n - lo, 256)), dim3(256), 0, g_ctx.stream, y, a,
+                           b, alpha, lo, n);
+        LAUNCH_OK("axpby tail");
+    }
+    return 0;
+}
+
+MI355_API int mi355_axpby_dev(float *y, const float *a, const float *b, float alpha, size_t n, int mode) {
+    if (!mi355_ready("axpby")) return -1;
+    if (!y || !a || (mode != 1 && !b)) return mi355_fail("axpby: NULL pointer");
+    if (n == 0) return mi355_fail("axpby: empty tensor");
+    switch (mode) {
+        case 0: return axpby_run<0>(y, a, b, alpha, n);
+        case 1: return axpby_run<1>(y, a, b, alpha, n);
+        case 2: return axpby_run<2>(y, a, b, alpha, n);
+        default: return mi355_fail("axpby: mode must be 0, 1 or 2");
+    }
+}
+
+// ---- RoPE ----
+MI355_API int mi355_rope_tables(float *cos_host, float *sin_host, int S, int hd, float theta) {
+    if (!cos_host || !sin_host) return mi355_fail("rope_tables: NULL pointer");
+    if (S <= 0 || hd <= 0 || (hd & 1) || !(theta > 0.f)) return mi355_fail("rope_tables: bad S/hd/theta");
+    for (int i = 0; i < hd / 2; i++) {
+        // training/training_dynamic/cpu_ops.h:172-175
+        const float freq = 1.0f / powf(theta, 2.0f * i / (float)hd);
+        for (int p = 0; p < S; p++) {
+            const float ang = p * freq;
+            cos_host[(size_t)i * S + p] = cosf(ang);
+            sin_host[(size_t)i * S + p] = sinf(ang);
+        }
+    }
+    return 0;
+}
+
+struct RopeCache {
+    int S, hd;
+    float theta;
+    float *cos_d, *sin_d;
+};
+static RopeCache g_rope[8];
+static int g_rope_n = 0;
+
+void mi355_free_rope_cache(void) {
+    for (int i = 0; i < g_rope_n; i++) (void)hipFree(g_rope[i].cos_d);   // one allocation holds both
+    g_rope_n = 0;
+}
+
+MI355_API int mi355_rope_tables_dev(const float **cos_dev, const float **sin_dev, int S, int hd, float theta) {
+    if (!mi355_ready("rope_tables_dev")) return -1;
+    if (!cos_dev || !sin_dev) return mi355_fail("rope_tables_dev: NULL pointer");
+    for (int i = 0; i < g_rope_n; i++)
+        if (g_rope[i].S == S && g_rope[i].hd == hd && g_rope[i].theta == theta) {
+            *cos_dev = g_rope[i].cos_d;
+            *sin_dev = g_rope[i].sin_d;
+            return 0;
+        }
+    if (g_rope_n == 8) return mi355_fail("rope_tables_dev: table cache full (8 distinct (S,hd,theta))");
+    if (S <= 0 || hd <= 0 || (hd & 1) || !(theta > 0.f)) return mi355_fail("rope_tables_dev: bad S/hd/theta");
+    const size_t n = (size_t)(hd / 2) * S;
+    float *host = (float *)malloc(2 * n * sizeof(float));
+    if (!host) return mi355_fail("rope_tables_dev: out of host memory");
+    mi355_rope_tables(host, host + n, S, hd, theta);
+    float *dev = nullptr;
+    hipError_t e = hipMalloc((void **)&dev, 2 * n * sizeof(float));
+    if (e == hipSuccess) e = hipMemcpy(dev, host, 2 * n * sizeof(float), hipMemcpyHostToDevice);
+    free(host);
+    if (e != hipSuccess) {
+        if (dev) (void)hipFree(dev);
+        return mi355_fail("rope_tables_dev: %s", hipGetErrorString(e));
+    }
+    g_rope[g_rope_n++] = RopeCache{S, hd, theta, dev, dev + n};
+    *cos_dev = dev;
+    *sin_dev = dev + n;
+    return 0;
+}
+
+MI355_API int mi355_rope_dev(float *q_out, float *k_out, const float *q_in, const float *k_in, int heads, int kv_heads,
+                             int hd, int S, int batch, const float *cos_dev, const float *sin_dev, int dir) {
+    if (!mi355_ready("rope")) return -1;
+    if (!cos_dev || !sin_dev) return mi355_fail("rope: NULL table");
+    if (hd <= 0 || (hd & 1) || S <= 0 || batch <= 0 || heads < 0 || kv_heads < 0 || heads + kv_heads == 0)
+        return mi355_fail("rope: bad shape heads=%d kv_heads=%d hd=%d S=%d batch=%d", heads, kv_heads, hd, S, batch);
+    if ((heads > 0 && (!q_out || !q_in)) || (kv_heads > 0 && (!k_out || !k_in))) return mi355_fail("rope: NULL pointer");
+    if (dir != 1 && dir != -1) return mi355_fail("rope: dir must be +1 or -1");
+    const bool vec_ok = (S % 4 == 0) && aligned16(cos_dev) && aligned16(sin_dev) &&
+                        (heads == 0 || (aligned16(q_in) && aligned16(q_out))) &&
+                        (kv_heads == 0 || (aligned16(k_in) && aligned16(k_out)));
+    const size_t pair_rows = (size_t)batch * (heads + kv_heads) * (hd / 2);
+    if (vec_ok) {
+        const size_t total = pair_rows * (S / 4);
+        hipLaunchKernelGGL((rope_kernel<4>), dim3((unsigned)ceil_div(total, EW_THREADS)), dim3(EW_THREADS), 0,
+                           g_ctx.stream, q_out, k_out, q_in, k_in, heads, kv_heads, hd, S, batch, cos_dev, sin_dev,
+                           (float)dir, total);
+    } else {
+        const size_t total = pair_rows * S;
+        hipLaunchKernelGGL((rope_kernel<1>), dim3((unsigned)ceil_div(total, EW_THREADS)), dim3(EW_THREADS), 0,
+                           g_ctx.stream, q_out, k_out, q_in, k_in, heads, kv_heads, hd, S, batch, cos_dev, sin_dev,
+                           (float)dir, total);
+    }
+    LAUNCH_OK("rope");
+    return 0;
+}
+
+// ---- INT8 ----
+MI355_API int mi355_int8_scale_dev(float *scale_dev, const float *x, size_t n) {
+    if (!mi355_ready("int8_scale")) return -1;
+    if (!scale_dev || !x) return mi355_fail("int8_scale: NULL pointer");
+    if (n == 0) return mi355_fail("int8_scale: empty tensor");
+    hipLaunchKernelGGL(fill_zero_u32, dim3(1), dim3(1), 0, g_ctx.stream, (unsigned int *)scale_dev);
+    if (aligned16(x)) {
+        const size_t n4 = n / 4;
+        size_t blocks = ceil_div(n4 ? n4 : 1, (size_t)EW_THREADS * 4);
+        if (blocks > 2048) blocks = 2048;
+        hipLaunchKernelGGL(absmax_kernel, dim3((unsigned)blocks), dim3(EW_THREADS), 0, g_ctx.stream,
+                           (unsigned int *)scale_dev, x, n, n4);
+    } else {
+        size_t blocks = ceil_div(n, 256 * 16);
+        if (blocks > 2048) blocks = 2048;
+        hipLaunchKernelGGL(absmax_scalar_kernel, dim3((unsigned)blocks), dim3(256), 0, g_ctx.stream,
+                           (unsigned int *)scale_dev, x, n);
+    }
+    hipLaunchKernelGGL(scale_from_absmax_kernel, dim3(1), dim3(1), 0, g_ctx.stream, scale_dev);
+    LAUNCH_OK("int8_scale");
+    return 0;
+}
+
+MI355_API int mi355_int8_quant_dev(int8_t *q, const float *x, const float *scale_dev, size_t n, int rounding) {
+    if (!mi355_ready("int8_quant")) return -1;
+    if (!q || !x || !scale_dev) return mi355_fail("int8_quant: NULL pointer");
+    if (n == 0) return mi355_fail("int8_quant: empty tensor");
+    if (rounding != 0 && rounding != 1) return mi355_fail("int8_quant: rounding must be 0 or 1");
+    size_t n4, lo;
+    split_vec(n, aligned16(x) && ((uintptr_t)q & 3u) == 0, n4, lo);
+    if (n4) {
+        const int u = pick_unroll(n4, 4);
+        EW_LAUNCH(quant_kernel, u, n4, (int *)q, x, scale_dev, n4, rounding);
+        LAUNCH_OK("int8_quant");
+    }
+    if (lo < n) {
+        hipLaunchKernelGGL(quant_scalar, dim3((unsigned)ceil_div(n - lo, 256)), dim3(256), 0, g_ctx.stream, q, x,
+                           scale_dev, lo, n, rounding);
+        LAUNCH_OK("int8_quant tail");
+    }
+    return 0;
+}
+
+MI355_API int mi355_int8_dequant_dev(float *x, const int8_t *q, const float *scale_dev, size_t n) {
+    if (!mi355_ready("int8_dequant")) return -1;
+    if (!q || !x || !scale_dev) return mi355_fail("int8_dequant: NULL pointer");
+    if (n == 0) return mi355_fail("int8_dequant: empty tensor");
+    size_t n4, lo;
+    split_vec(n, aligned16(x) && ((uintptr_t)q & 3u) == 0, n4, lo);
+    if (n4) {
+        const int u = pick_unroll(n4, 4);
+        EW_LAUNCH(dequant_kernel, u, n4, x, (const int *)q, scale_dev, n4);
+        LAUNCH_OK("int8_dequant");
+    }
+    if (lo < n) {
+        hipLaunchKernelGGL(dequant_scalar, dim3((unsigned)ceil_div(n - lo, 256)), dim3(256), 0, g_ctx.stream, x, q,
+                           scale_dev, lo, n);
+        LAUNCH_OK("int8_dequant tail");
+    }
+    return 0;
+}

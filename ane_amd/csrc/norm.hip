@@ -1,0 +1,345 @@
+// norm.hip — RMSNorm forward / backward on channel-first [batch][C][S] tensors.
+//
+// Reference ops: rmsnorm (training/stories_cpu_ops.h:6-21) and rmsnorm_bwd
+// (training/stories_cpu_ops.h:23-53; twins in training/training_dynamic/cpu_ops.h:7-54).
+//
+// The reduction runs over the STRIDED axis c; columns s are contiguous.  A workgroup owns a
+// strip of W = LPR*VEC columns of one slab.  LPR adjacent lanes cover the strip with one
+// 128-bit load each, the remaining lane bits and the waves spread over rows, so every load
+// instruction of a wave reads (64/LPR) full row segments.  Each thread keeps its rows in
+// registers (one HBM pass), per-column partial sums are combined with cross-lane shuffles and a
+// small LDS exchange between waves, then the strip is normalised from registers and stored.
+// dw partials (one per workgroup and row) go to a workspace and are summed in a fixed order by
+// a second kernel, so the result is deterministic and needs no floating-point atomics.
+#include "common.h"
+#include "tile.h"
+
+namespace {
+
+// CAP > 0: rows are held in registers (C <= CAP * THREADS/LPR).  CAP == 0: rows are re-read
+// in the second pass (they come back from L2).
+template <int VEC, int LPR, int THREADS, int CAP>
+__global__ __launch_bounds__(THREADS) void rms_fwd_kernel(float *__restrict__ y, const float *__restrict__ x,
+                                                          const float *__restrict__ w, int C, int S, int strips,
+                                                          int nblk, float eps, float invC) {
+    constexpr int RPS = THREADS / LPR;
+    constexpr int W = LPR * VEC;
+    constexpr int NW = THREADS / 64;
+    __shared__ float lds[NW * 1 * (LPR < 64 ? LPR : 64) * VEC];
+    const int blk = xcd_remap(blockIdx.x, nblk);
+    const int slab = blk / strips, strip = blk - slab * strips;
+    const int lc = threadIdx.x % LPR, row0 = threadIdx.x / LPR;
+    const int col = strip * W + lc * VEC;
+    const bool col_ok = col < S;
+    const size_t base = (size_t)slab * C * S + col;
+    const float *xs = x + base;
+    float *ys = y + base;
+
+    float acc[1][VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc[0][j] = 0.f;
+
+    if constexpr (CAP > 0) {
+        float xv[CAP][VEC];
+        float wv[CAP];
+#pragma unroll
+        for (int k = 0; k < CAP; k++) {
+            const int c = row0 + k * RPS;
+            if (c < C && col_ok) {
+                ldv<VEC>(xv[k], xs + (size_t)c * S);
+                wv[k] = w[c];
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) xv[k][j] = 0.f;
+                wv[k] = 0.f;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < CAP; k++)
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc[0][j] += xv[k][j] * xv[k][j];
+        strip_reduce<VEC, LPR, THREADS, 1>(acc, lds);
+        float rr[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; j++) rr[j] = 1.0f / sqrtf(acc[0][j] * invC + eps);
+#pragma unroll
+        for (int k = 0; k < CAP; k++) {
+            const int c = row0 + k * RPS;
+            if (c < C && col_ok) {
+                float o[VEC];
+#pragma unroll
+                for (int j = 0; j < VEC; j++) o[j] = (xv[k][j] * rr[j]) * wv[k];
+                stv<VEC>(ys + (size_t)c * S, o);
+            }
+        }
+    } else {
+        if (col_ok)
+            for (int c = row0; c < C; c += RPS) {
+                float t[VEC];
+                ldv<VEC>(t, xs + (size_t)c * S);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) acc[0][j] += t[j] * t[j];
+            }
+        strip_reduce<VEC, LPR, THREADS, 1>(acc, lds);
+        float rr[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; j++) rr[j] = 1.0f / sqrtf(acc[0][j] * invC + eps);
+        if (col_ok)
+            for (int c = row0; c < C; c += RPS) {
+                float t[VEC], o[VEC];
+                ldv<VEC>(t, xs + (size_t)c * S);
+                const float wc = w[c];
+#pragma unroll
+                for (int j = 0; j < VEC; j++) o[j] = (t[j] * rr[j]) * wc;
+                stv<VEC>(ys + (size_t)c * S, o);
+            }
+    }
+}
+
+template <int VEC, int LPR, int THREADS, int CAP>
+__global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__restrict__ dw_part,
+                                                          const float *dy, const float *__restrict__ x,
+                                                          const float *__restrict__ w, int C, int S, int strips,
+                                                          int nblk, float eps, float invC, int variant) {
+    constexpr int RPS = THREADS / LPR;
+    constexpr int W = LPR * VEC;
+    constexpr int NW = THREADS / 64;
+    __shared__ float lds[NW * 2 * (LPR < 64 ? LPR : 64) * VEC];
+    const int blk = xcd_remap(blockIdx.x, nblk);
+    const int slab = blk / strips, strip = blk - slab * strips;
+    const int lc = threadIdx.x % LPR, row0 = threadIdx.x / LPR;
+    const int col = strip * W + lc * VEC;
+    const bool col_ok = col < S;
+    const size_t base = (size_t)slab * C * S + col;
+    const float *xs = x + base, *dys = dy + base;
+    float *dxs = dx + base;
+    float *part = dw_part + (size_t)blk * C;
+
+    float acc[2][VEC];   // [0] = sum x^2, [1] = sum (dy*x)*w
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc[0][j] = acc[1][j] = 0.f;
+
+    auto finish = [&](float (&rr)[VEC], float (&dotn)[VEC]) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            rr[j] = 1.0f / sqrtf(acc[0][j] * invC + eps);
+            dotn[j] = acc[1][j] * ((rr[j] * rr[j]) * invC);
+        }
+    };
+    auto row_out = [&](int c, const float (&xr)[VEC], const float (&dyr)[VEC], float wc, const float (&rr)[VEC],
+                       const float (&dotn)[VEC]) {
+        float o[VEC];
+        float p = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            if (variant == 0) o[j] = ((dyr[j] - xr[j] * dotn[j]) * rr[j]) * wc;
+            else o[j] = (dyr[j] * wc) * rr[j] - (xr[j] * dotn[j]) * rr[j];
+            p += (dyr[j] * xr[j]) * rr[j];
+        }
+        if (col_ok) stv<VEC>(dxs + (size_t)c * S, o);
+        p = group_sum<(LPR < 64 ? LPR : 64)>(p);
+        if (lc == 0) part[c] = p;
+    };
+
+    if constexpr (CAP > 0) {
+        float xv[CAP][VEC], dv[CAP][VEC], wv[CAP];
+#pragma unroll
+        for (int k = 0; k < CAP; k++) {
+            const int c = row0 + k * RPS;
+            if (c < C && col_ok) {
+                ldv<VEC>(xv[k], xs + (size_t)c * S);
+                ldv<VEC>(dv[k], dys + (size_t)c * S);
+                wv[k] = w[c];
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) xv[k][j] = dv[k][j] = 0.f;
+                wv[k] = 0.f;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < CAP; k++)
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                acc[0][j] += xv[k][j] * xv[k][j];
+                acc[1][j] += (dv[k][j] * xv[k][j]) * wv[k];
+            }
+        strip_reduce<VEC, LPR, THREADS, 2>(acc, lds);
+        float rr[VEC], dotn[VEC];
+        finish(rr, dotn);
+#pragma unroll
+        for (int k = 0; k < CAP; k++) {
+            const int c = row0 + k * RPS;
+            if (c < C) row_out(c, xv[k], dv[k], wv[k], rr, dotn);   // uniform per LPR lane group
+        }
+    } else {
+        if (col_ok)
+            for (int c = row0; c < C; c += RPS) {
+                float a[VEC], b[VEC];
+                ldv<VEC>(a, xs + (size_t)c * S);
+                ldv<VEC>(b, dys + (size_t)c * S);
+                const float wc = w[c];
+#pragma unroll
+                for (int j = 0; j < VEC; j++) {
+                    acc[0][j] += a[j] * a[j];
+                    acc[1][j] += (b[j] * a[j]) * wc;
+                }
+            }
+        strip_reduce<VEC, LPR, THREADS, 2>(acc, lds);
+        float rr[VEC], dotn[VEC];
+        finish(rr, dotn);
+        for (int c = row0; c < C; c += RPS) {
+            float a[VEC], b[VEC];
+            if (col_ok) {
+                ldv<VEC>(a, xs + (size_t)c * S);
+                ldv<VEC>(b, dys + (size_t)c * S);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) a[j] = b[j] = 0.f;
+            }
+            row_out(c, a, b, w[c], rr, dotn);
+        }
+    }
+}
+
+// out[c] += sum_r part[r][c], rows taken in a fixed order: 16 interleaved row groups, each
+// summed with four independent accumulators (so four loads are in flight), then combined in a
+// fixed order.  One workgroup handles 64 channels.
+__global__ __launch_bounds__(1024) void reduce_rows_kernel(float *__restrict__ out, const float *__restrict__ part,
+                                                           int nrows, int C) {
+    __shared__ float lds[16][64];
+    const int cl = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + cl;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (c < C) {
+        int r = g;
+        for (; r + 48 < nrows; r += 64) {
+            s0 += part[(size_t)r * C + c];
+            s1 += part[(size_t)(r + 16) * C + c];
+            s2 += part[(size_t)(r + 32) * C + c];
+            s3 += part[(size_t)(r + 48) * C + c];
+        }
+        for (; r < nrows; r += 16) s0 += part[(size_t)r * C + c];
+    }
+    lds[g][cl] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (g == 0 && c < C) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) t += lds[k][cl];
+        out[c] = out[c] + t;
+    }
+}
+
+struct NormCfg {
+    int vec, lpr, threads, cap;
+};
+
+// Picks the tile: registers when the rows fit, and the narrowest strip needed to give every
+// compute unit at least two workgroups.
+NormCfg pick_cfg(int C, int S, int batch, bool vec_ok, int max_cap, int lpr_knob, int thr_knob) {
+    NormCfg best{};
+    if (!vec_ok) return NormCfg{1, 64, 256, 0};
+    const int lprs[3] = {16, 8, 4};
+    const int thrs[2] = {256, 1024};
+    const int caps[2] = {8, 16};
+    long best_score = -1;
+    for (int lpr : lprs) {
+        if (lpr_knob && lpr != lpr_knob) continue;
+        for (int thr : thrs) {
+            if (thr_knob && thr != thr_knob) continue;
+            const int rps = thr / lpr;
+            int cap = 0;
+            for (int cp : caps)
+                if (cp <= max_cap && (long)cp * rps >= C) { cap = cp; break; }
+            if (thr == 1024 && cap > 8) cap = 0;   // 16 waves per CU leave 128 VGPRs per lane
+            const long strips = ceil_div((size_t)S, (size_t)lpr * 4);
+            const long nblk = strips * batch;
+            long score = (cap > 0 ? 1000000 : 0);
+            const long want = 2L * (g_ctx.num_cu > 0 ? g_ctx.num_cu : 256);
+            score += (nblk >= want ? want : nblk) * 100 / want * 1000;   // occupancy first
+            score += lpr;                                                // then the widest strip
+            score += (thr == 256 ? 1 : 0);
+            if (score > best_score) { best_score = score; best = NormCfg{4, lpr, thr, cap}; }
+        }
+    }
+    if (best_score < 0) best = NormCfg{4, 16, 256, 0};
+    return best;
+}
+
+template <int VEC, int LPR, int THREADS, int CAP>
+void launch_fwd(float *y, const float *x, const float *w, int C, int S, int batch, float eps) {
+    const int strips = (int)ceil_div((size_t)S, (size_t)LPR * VEC);
+    const int nblk = strips * batch;
+    hipLaunchKernelGGL((rms_fwd_kernel<VEC, LPR, THREADS, CAP>), dim3(nblk), dim3(THREADS), 0, g_ctx.stream, y, x, w,
+                       C, S, strips, nblk, eps, 1.0f / (float)C);
+}
+
+template <int VEC, int LPR, int THREADS, int CAP>
+void launch_bwd(float *dx, float *part, const float *dy, const float *x, const float *w, int C, int S, int batch,
+                float eps, int variant) {
+    const int strips = (int)ceil_div((size_t)S, (size_t)LPR * VEC);
+    const int nblk = strips * batch;
+    hipLaunchKernelGGL((rms_bwd_kernel<VEC, LPR, THREADS, CAP>), dim3(nblk), dim3(THREADS), 0, g_ctx.stream, dx, part,
+                       dy, x, w, C, S, strips, nblk, eps, 1.0f / (float)C, variant);
+}
+
+#define NORM_DISPATCH(FN, cfg, ...)                                                                   \
+    do {                                                                                              \
+        const int key = (cfg).vec * 1000000 + (cfg).lpr * 10000 + ((cfg).threads / 256) * 100 + (cfg).cap; \
+        switch (key) {                                                                                \
+            case 1640100: FN<1, 64, 256, 0>(__VA_ARGS__); break;                                      \
+            case 4160100: FN<4, 16, 256, 0>(__VA_ARGS__); break;                                      \
+            case 4160108: FN<4, 16, 256, 8>(__VA_ARGS__); break;                                      \
+            case 4160116: FN<4, 16, 256, 16>(__VA_ARGS__); break;                                     \
+            case 4160400: FN<4, 16, 1024, 0>(__VA_ARGS__); break;                                     \
+            case 4160408: FN<4, 16, 1024, 8>(__VA_ARGS__); break;                                     \
+            case 4080100: FN<4, 8, 256, 0>(__VA_ARGS__); break;                                       \
+            case 4080108: FN<4, 8, 256, 8>(__VA_ARGS__); break;                                       \
+            case 4080116: FN<4, 8, 256, 16>(__VA_ARGS__); break;                                      \
+            case 4080400: FN<4, 8, 1024, 0>(__VA_ARGS__); break;                                      \
+            case 4080408: FN<4, 8, 1024, 8>(__VA_ARGS__); break;                                      \
+            case 4040100: FN<4, 4, 256, 0>(__VA_ARGS__); break;                                       \
+            case 4040108: FN<4, 4, 256, 8>(__VA_ARGS__); break;                                       \
+            case 4040116: FN<4, 4, 256, 16>(__VA_ARGS__); break;                                      \
+            case 4040400: FN<4, 4, 1024, 0>(__VA_ARGS__); break;                                      \
+            case 4040408: FN<4, 4, 1024, 8>(__VA_ARGS__); break;                                      \
+            default: return mi355_fail("rmsnorm: no kernel for tile key %d", key);                    \
+        }                                                                                             \
+    } while (0)
+
+}   // namespace
+
+int mi355_reduce_rows(float *out, const float *part, int nrows, int C) {
+    hipLaunchKernelGGL(reduce_rows_kernel, dim3((unsigned)ceil_div((size_t)C, 64)), dim3(1024), 0, g_ctx.stream, out,
+                       part, nrows, C);
+    LAUNCH_OK("reduce_rows");
+    return 0;
+}
+
+MI355_API int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, int C, int S, int batch, float eps) {
+    if (!mi355_ready("rmsnorm_fwd")) return -1;
+    if (!y || !x || !w) return mi355_fail("rmsnorm_fwd: NULL pointer");
+    if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_fwd: bad shape C=%d S=%d batch=%d", C, S, batch);
+    const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(y);
+    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 16, g_ctx.rms_lpr, g_ctx.rms_threads);
+    NORM_DISPATCH(launch_fwd, cfg, y, x, w, C, S, batch, eps);
+    LAUNCH_OK("rmsnorm_fwd");
+    return 0;
+}
+
+MI355_API int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const float *x, const float *w, int C,
+                                    int S, int batch, float eps, int variant) {
+    if (!mi355_ready("rmsnorm_bwd")) return -1;
+    if (!dx || !dw || !dy || !x || !w) return mi355_fail("rmsnorm_bwd: NULL pointer");
+    if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_bwd: bad shape C=%d S=%d batch=%d", C, S, batch);
+    if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd: variant must be 0 or 1");
+    const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(dy) && aligned16(dx);
+    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 16, g_ctx.rms_lpr, g_ctx.rms_threads);
+    const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
+    const int nblk = strips * batch;
+    float *part = (float *)mi355_ws((size_t)nblk * C * sizeof(float));
+    if (!part) return -1;
+    NORM_DISPATCH(launch_bwd, cfg, dx, part, dy, x, w, C, S, batch, eps, variant);
+    LAUNCH_OK("rmsnorm_bwd");
+    return mi355_reduce_rows(dw, part, nblk, C);
+}

@@ -1,0 +1,255 @@
+// softmax_ce.hip — fused classifier softmax + cross-entropy forward/backward on logits [V][S].
+//
+// Reference op: cross_entropy_loss (training/training_dynamic/cpu_ops.h:68-93; transpose form
+// training/stories_cpu_ops.h:71-108) plus the loss-scale pass of training/training_dynamic/train.m:497.
+//
+// The softmax runs down the STRIDED axis v (columns t are contiguous), so a wave reads whole rows
+// with 128-bit loads and every lane owns four columns; no cross-lane traffic is needed until the
+// four waves of a workgroup are combined through LDS.
+//   pass 1  each workgroup reduces a block of rows to per-column (max, sum exp) partials
+//           (online rescaling between 64-row register tiles);
+//   combine per column, partials are merged in a fixed order, the target logit is read, the
+//           per-column loss term is formed and the mean is taken by a fixed tree;
+//   pass 2  dlogits = (exp(l - M) * (1/L) - onehot) * (1/S) * grad_scale.  Row blocks are visited
+//           in the reverse order of pass 1 so the most recently read rows are re-read first
+//           (they are the most likely to still sit in the last-level cache).
+#include "common.h"
+
+#include <math.h>
+
+namespace {
+
+constexpr int CE_THREADS = 256;
+constexpr int CE_WAVES = CE_THREADS / 64;
+constexpr int CE_CAP = 16;                       // register tile: 16 steps x 4 waves = 64 rows
+constexpr int CE_TILE_ROWS = CE_CAP * CE_WAVES;
+
+template <int VEC>
+__device__ __forceinline__ void ld_cols(float (&r)[VEC], const float *p) {
+    if constexpr (VEC == 4) {
+        v4f t = ld4(p);
+        r[0] = t.x; r[1] = t.y; r[2] = t.z; r[3] = t.w;
+    } else {
+        r[0] = *p;
+    }
+}
+
+// grid: (row blocks, column strips of 64*VEC)
+template <int VEC>
+__global__ __launch_bounds__(CE_THREADS) void ce_partial_kernel(float *__restrict__ pm, float *__restrict__ pl,
+                                                                const float *__restrict__ logits, int V, int S,
+                                                                int rows_per_block) {
+    __shared__ float sm[CE_WAVES][64 * VEC], sl[CE_WAVES][64 * VEC];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = (blockIdx.y * 64 + lane) * VEC;
+    const bool col_ok = col < S;
+    const int v_lo = blockIdx.x * rows_per_block;
+    const int v_hi = min(V, v_lo + rows_per_block);
+
+    float m[VEC], l[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) { m[j] = -INFINITY; l[j] = 0.f; }
+
+    for (int base = v_lo; base < v_hi; base += CE_TILE_ROWS) {
+        float x[CE_CAP][VEC];
+#pragma unroll
+        for (int k = 0; k < CE_CAP; k++) {
+            const int v = base + k * CE_WAVES + wave;
+            if (v < v_hi && col_ok) ld_cols<VEC>(x[k], logits + (size_t)v * S + col);
+            else {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) x[k][j] = -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            float tm = x[0][j];
+#pragma unroll
+            for (int k = 1; k < CE_CAP; k++) tm = fmaxf(tm, x[k][j]);
+            const float nm = fmaxf(m[j], tm);
+            if (nm > -INFINITY) {
+                float s = 0.f;
+#pragma unroll
+                for (int k = 0; k < CE_CAP; k++) s += exp_neg(x[k][j] - nm);   // exp(-inf) = 0 for masked rows
+                l[j] = l[j] * exp_neg(m[j] - nm) + s;
+                m[j] = nm;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; j++) { sm[wave][lane * VEC + j] = m[j]; sl[wave][lane * VEC + j] = l[j]; }
+    __syncthreads();
+    if (wave == 0 && col_ok) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            float M = sm[0][lane * VEC + j];
+#pragma unroll
+            for (int w = 1; w < CE_WAVES; w++) M = fmaxf(M, sm[w][lane * VEC + j]);
+            float L = 0.f;
+#pragma unroll
+            for (int w = 0; w < CE_WAVES; w++) {
+                const float mw = sm[w][lane * VEC + j];
+                if (mw > -INFINITY) L += sl[w][lane * VEC + j] * exp_neg(mw - M);
+            }
+            pm[(size_t)blockIdx.x * S + col + j] = M;
+            pl[(size_t)blockIdx.x * S + col + j] = L;
+        }
+    }
+}
+
+// One workgroup per 64 columns: 16 groups of threads each merge an interleaved subset of the row
+// blocks, then the 16 partial results are merged in order.
+__global__ __launch_bounds__(1024) void ce_combine_kernel(float *__restrict__ colM, float *__restrict__ colInv,
+                                                          float *__restrict__ colLoss, const float *__restrict__ pm,
+                                                          const float *__restrict__ pl,
+                                                          const float *__restrict__ logits,
+                                                          const int32_t *__restrict__ targets, int V, int S,
+                                                          int nblk) {
+    __shared__ float sm[16][64], sl[16][64];
+    const int cl = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int t = blockIdx.x * 64 + cl;
+    float m = -INFINITY, l = 0.f;
+    if (t < S)
+        for (int r = g; r < nblk; r += 16) {
+            const float mr = pm[(size_t)r * S + t], lr = pl[(size_t)r * S + t];
+            const float nm = fmaxf(m, mr);
+            if (nm > -INFINITY) {
+                l = l * exp_neg(m - nm) + lr * exp_neg(mr - nm);
+                m = nm;
+            }
+        }
+    sm[g][cl] = m;
+    sl[g][cl] = l;
+    __syncthreads();
+    if (g == 0 && t < S) {
+        float M = sm[0][cl];
+#pragma unroll
+        for (int k = 1; k < 16; k++) M = fmaxf(M, sm[k][cl]);
+        float L = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++)
+            if (sm[k][cl] > -INFINITY) L += sl[k][cl] * exp_neg(sm[k][cl] - M);
+        const float inv = 1.0f / L;
+        colM[t] = M;
+        colInv[t] = inv;
+        const int tgt = targets[t];
+        float loss = 0.f;
+        if (tgt >= 0 && tgt < V) {
+            const float p = exp_neg(logits[(size_t)tgt * S + t] - M) * inv;
+            loss = -logf(p + 1e-10f);
+        }
+        colLoss[t] = loss;
+    }
+}
+
+// loss = (sum_t colLoss[t]) / S with a fixed summation tree
+__global__ __launch_bounds__(256) void ce_loss_kernel(float *__restrict__ loss_out, const float *__restrict__ colLoss,
+                                                      int S) {
+    __shared__ float red[256];
+    float s = 0.f;
+    for (int t = threadIdx.x; t < S; t += 256) s += colLoss[t];
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+        if (threadIdx.x < off) red[threadIdx.x] += red[threadIdx.x + off];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *loss_out = red[0] / (float)S;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(CE_THREADS) void ce_grad_kernel(float *dlogits, const float *logits,
+                                                             const float *__restrict__ colM,
+                                                             const float *__restrict__ colInv,
+                                                             const int32_t *__restrict__ targets, int V, int S,
+                                                             int rows_per_block, float invS, float grad_scale) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = (blockIdx.y * 64 + lane) * VEC;
+    if (col >= S) return;
+    const int rb = gridDim.x - 1 - blockIdx.x;           // reverse order of pass 1
+    const int v_lo = rb * rows_per_block;
+    const int v_hi = min(V, v_lo + rows_per_block);
+    float M[VEC], inv[VEC], sc[VEC];
+    int tgt[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        M[j] = colM[col + j];
+        inv[j] = colInv[col + j];
+        const int tg = targets[col + j];
+        const bool ok = tg >= 0 && tg < V;
+        tgt[j] = ok ? tg : -1;
+        sc[j] = ok ? invS : 1.0f;      // an out-of-range target leaves the column unscaled (stories_cpu_ops.h:98)
+    }
+    for (int base = v_lo; base < v_hi; base += CE_TILE_ROWS) {
+        float x[CE_CAP][VEC];
+#pragma unroll
+        for (int k = 0; k < CE_CAP; k++) {
+            const int v = base + k * CE_WAVES + wave;
+            if (v < v_hi) ld_cols<VEC>(x[k], logits + (size_t)v * S + col);
+        }
+#pragma unroll
+        for (int k = 0; k < CE_CAP; k++) {
+            const int v = base + k * CE_WAVES + wave;
+            if (v < v_hi) {
+                float o[VEC];
+#pragma unroll
+                for (int j = 0; j < VEC; j++) {
+                    float p = exp_neg(x[k][j] - M[j]) * inv[j];
+                    if (v == tgt[j]) p -= 1.0f;
+                    p = p * sc[j];
+                    if (grad_scale != 1.0f) p = p * grad_scale;
+                    o[j] = p;
+                }
+                float *dst = dlogits + (size_t)v * S + col;
+                if constexpr (VEC == 4) {
+                    v4f t = {o[0], o[1], o[2], o[3]};
+                    st4_nt(dst, t);
+                } else {
+                    *dst = o[0];
+                }
+            }
+        }
+    }
+}
+
+}   // namespace
+
+MI355_API int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float *logits, const int32_t *targets, int V,
+                                   int S, float grad_scale) {
+    if (!mi355_ready("softmax_ce")) return -1;
+    if (!dlogits || !loss_dev || !logits || !targets) return mi355_fail("softmax_ce: NULL pointer");
+    if (V <= 0 || S <= 0) return mi355_fail("softmax_ce: bad shape V=%d S=%d", V, S);
+    int rpb = g_ctx.ce_rows > 0 ? g_ctx.ce_rows : 256;
+    rpb = (int)ceil_div((size_t)rpb, CE_TILE_ROWS) * CE_TILE_ROWS;
+    const int nblk = (int)ceil_div((size_t)V, (size_t)rpb);
+    const bool vec_ok = (S % 4 == 0) && aligned16(logits) && aligned16(dlogits);
+    const int vec = vec_ok ? 4 : 1;
+    const int strips = (int)ceil_div((size_t)S, (size_t)64 * vec);
+    if (strips > 65535) return mi355_fail("softmax_ce: S too large");
+
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const size_t part_b = al((size_t)nblk * S * sizeof(float)), col_b = al((size_t)S * sizeof(float));
+    char *ws = (char *)mi355_ws(2 * part_b + 3 * col_b);
+    if (!ws) return -1;
+    float *pm = (float *)ws, *pl = (float *)(ws + part_b);
+    float *colM = (float *)(ws + 2 * part_b), *colInv = (float *)(ws + 2 * part_b + col_b);
+    float *colLoss = (float *)(ws + 2 * part_b + 2 * col_b);
+
+    const dim3 grid((unsigned)nblk, (unsigned)strips);
+    if (vec_ok) hipLaunchKernelGGL((ce_partial_kernel<4>), grid, dim3(CE_THREADS), 0, g_ctx.stream, pm, pl, logits, V, S, rpb);
+    else hipLaunchKernelGGL((ce_partial_kernel<1>), grid, dim3(CE_THREADS), 0, g_ctx.stream, pm, pl, logits, V, S, rpb);
+    LAUNCH_OK("softmax_ce partial");
+    hipLaunchKernelGGL(ce_combine_kernel, dim3((unsigned)ceil_div((size_t)S, 64)), dim3(1024), 0, g_ctx.stream, colM,
+                       colInv, colLoss, pm, pl, logits, targets, V, S, nblk);
+    LAUNCH_OK("softmax_ce combine");
+    hipLaunchKernelGGL(ce_loss_kernel, dim3(1), dim3(256), 0, g_ctx.stream, loss_dev, colLoss, S);
+    LAUNCH_OK("softmax_ce loss");
+    if (vec_ok)
+        hipLaunchKernelGGL((ce_grad_kernel<4>), grid, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
+                           targets, V, S, rpb, 1.0f / (float)S, grad_scale);
+    else
+        hipLaunchKernelGGL((ce_grad_kernel<1>), grid, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
+                           targets, V, S, rpb, 1.0f / (float)S, grad_scale);
+    LAUNCH_OK("softmax_ce grad");
+    return 0;
+}

@@ -1,0 +1,58 @@
+// tile.h — register-tile helpers shared by the strided-axis reduction kernels.
+#pragma once
+#include "common.h"
+
+template <int VEC>
+__device__ __forceinline__ void ldv(float (&r)[VEC], const float *p) {
+    if constexpr (VEC == 4) {
+        v4f t = ld4(p);
+        r[0] = t.x; r[1] = t.y; r[2] = t.z; r[3] = t.w;
+    } else {
+        r[0] = *p;
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void stv(float *p, const float (&r)[VEC]) {
+    if constexpr (VEC == 4) {
+        v4f t = {r[0], r[1], r[2], r[3]};
+        st4(p, t);
+    } else {
+        *p = r[0];
+    }
+}
+
+// Sum acc[q][j] over all threads of the block that share the same lane column (tid % LPR).
+// Every thread ends with the full per-column totals.  lds: NW*NV*LPR*VEC floats.
+template <int VEC, int LPR, int THREADS, int NV>
+__device__ __forceinline__ void strip_reduce(float (&acc)[NV][VEC], float *lds) {
+    constexpr int NW = THREADS / 64;
+    constexpr int WLPR = LPR < 64 ? LPR : 64;
+#pragma unroll
+    for (int q = 0; q < NV; q++)
+#pragma unroll
+        for (int j = 0; j < VEC; j++) acc[q][j] = wave_sum_stride<WLPR>(acc[q][j]);
+    if constexpr (NW > 1) {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int lc = threadIdx.x % LPR;
+        if (lane < WLPR) {
+#pragma unroll
+            for (int q = 0; q < NV; q++)
+#pragma unroll
+                for (int j = 0; j < VEC; j++) lds[((wave * NV + q) * WLPR + lane) * VEC + j] = acc[q][j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < NV; q++)
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                float s = 0.f;
+#pragma unroll
+                for (int wv = 0; wv < NW; wv++) s += lds[((wv * NV + q) * WLPR + (lc & (WLPR - 1))) * VEC + j];
+                acc[q][j] = s;
+            }
+    }
+}
+
+
+// out[c] += sum over rows of part[rows][C] in a fixed order (norm.hip)
+int mi355_reduce_rows(float *out, const float *part, int nrows, int C);

@@ -1,0 +1,208 @@
+/*
+ * mi355_bridge.h — C-callable bridge to the MI355X (gfx950) implementations of the per-layer
+ * CPU ops of the maderix/ANE training loops.
+ *
+ * Pure C, includable from C, C++ and Objective-C.  The interface style follows the reference's
+ * own C-ABI, bridge/ane_bridge.h:11-98: an idempotent `int ..._init(void)` returning 0 / -1,
+ * opaque handles that are NULL on failure, NULL-safe `..._free`, `write`/`read` calls that
+ * silently ignore bad arguments, and one "mi355_bridge: ..." line on stderr per failure.
+ *
+ * All tensors are fp32 in the reference's channel-first layout x[c*S + s]
+ * (training/stories_cpu_ops.h:110-118).  "batch B" means B consecutive [C,S] slabs — the
+ * reference processes one sequence per call, so batch B equals B reference calls in slab order.
+ *
+ * Threading: one process-global context and one HIP stream; entry points are not re-entrant
+ * (the reference's ops share a global scratch buffer the same way,
+ * training/training_dynamic/cpu_ops.h:5).  Device-resident calls (`*_dev`) are asynchronous on
+ * the bridge stream until mi355_sync() / mi355_buf_read(); host-pointer drop-ins are synchronous.
+ *
+ * Device-resident calls return 0 on success and -1 on failure (bad shape, NULL pointer, no
+ * device); on failure no kernel is launched and the outputs are untouched.
+ */
+#ifndef MI355_BRIDGE_H
+#define MI355_BRIDGE_H
+
+#include <stddef.h>
+#include <stdint.h>
+#include <stdbool.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * Lifecycle.  Replaces ane_bridge_init (bridge/ane_bridge.h:20, bridge/ane_bridge.m:33-57).
+ * ---------------------------------------------------------------------------------------- */
+
+/* Select device 0, create the context.  Idempotent.  0 on success, -1 if no usable GPU. */
+int mi355_init(void);
+/* Release every cached device allocation and the context.  Safe to call twice. */
+void mi355_shutdown(void);
+/* Text of the most recent failure ("" if none).  Static storage, never NULL. */
+const char *mi355_last_error(void);
+/* Device name, its peak HBM bandwidth in GB/s as reported by the driver (memory clock x bus
+ * width; 0 when not reported), and the number of compute units.  Any pointer may be NULL. */
+int mi355_device_info(char *name, size_t name_len, double *peak_hbm_gbs, int *compute_units);
+/* Run every later device-resident call on the given hipStream_t (NULL = the default stream). */
+int mi355_set_stream(void *hip_stream);
+/* Wait for everything queued on the bridge stream.  0 / -1. */
+int mi355_sync(void);
+/* Grow the internal workspace (sort buffers, reduction partials) to at least `bytes` now, so
+ * that later calls of up to that need allocate nothing. */
+int mi355_workspace_reserve(size_t bytes);
+/* Tuning knob for experiments: named integer settings ("rms_lpr", "ew_unroll", ...); unknown
+ * names return -1.  Defaults are chosen per shape when a knob is 0. */
+int mi355_tune_set(const char *key, int value);
+
+/* ------------------------------------------------------------------------------------------
+ * Device buffers (opaque).  Replace the IOSurface-backed tensors behind
+ * ane_bridge_write_input / ane_bridge_read_output / ane_bridge_free
+ * (bridge/ane_bridge.h:54-62, bridge/ane_bridge.m:233-251).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct mi355_buf mi355_buf;
+
+mi355_buf *mi355_buf_alloc(size_t bytes);                 /* NULL on failure; contents zeroed */
+void mi355_buf_free(mi355_buf *b);                        /* NULL-safe */
+void *mi355_buf_devptr(mi355_buf *b);                     /* raw device address (NULL if b NULL) */
+size_t mi355_buf_bytes(mi355_buf *b);
+/* Synchronous copies; out-of-range or NULL arguments are ignored, as in the reference. */
+void mi355_buf_write(mi355_buf *b, size_t offset, const void *src, size_t bytes);
+void mi355_buf_read(mi355_buf *b, size_t offset, void *dst, size_t bytes);
+int mi355_buf_zero(mi355_buf *b);                         /* asynchronous fill on the bridge stream */
+
+/* Timing on the bridge stream (HIP events). */
+typedef struct mi355_event mi355_event;
+mi355_event *mi355_event_create(void);
+void mi355_event_destroy(mi355_event *e);
+int mi355_event_record(mi355_event *e);
+/* Waits for `stop`, returns milliseconds between the two records (-1 on failure). */
+float mi355_event_elapsed_ms(mi355_event *start, mi355_event *stop);
+
+/* Synthetic data, generated on the device (counter-based splitmix64 + Box-Muller). */
+int mi355_fill_normal_dev(float *p, size_t n, uint64_t seed, float mean, float std);
+int mi355_fill_randint_dev(int32_t *p, size_t n, uint64_t seed, int32_t lo, int32_t hi /*excl.*/);
+
+/* ------------------------------------------------------------------------------------------
+ * Device-resident ops (the measured path).  Every pointer is a device address.
+ * ---------------------------------------------------------------------------------------- */
+
+/* RMSNorm forward.  Replaces rmsnorm — training/stories_cpu_ops.h:6-21,
+ * training/training_dynamic/cpu_ops.h:7-22.  y = (x * rsqrt(mean_c x^2 + eps)) * w[c].
+ * x, y: [batch][C][S]; w: [C].  The reference hard-codes eps = 1e-5f. */
+int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, int C, int S, int batch,
+                          float eps);
+
+/* RMSNorm backward.  Replaces rmsnorm_bwd — training/stories_cpu_ops.h:23-53,
+ * training/training_dynamic/cpu_ops.h:24-54.  dx is assigned, dw[C] is accumulated (+=).
+ * variant 0 = the reference CPU op: dx = ((dy - x*dot)*rr)*w;
+ * variant 1 = the textbook gradient (training/backward.h:28-42, training/ane_rmsnorm_bwd.h:56-74):
+ * dx = (dy*w)*rr - (x*dot)*rr.  Both use dot = rr^2/C * sum_c dy*x*w. */
+int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const float *x, const float *w,
+                          int C, int S, int batch, float eps, int variant);
+
+/* SwiGLU gate forward: out = (h1*sigmoid(h1))*h3.  Replaces the MIL sigmoid/mul/mul of
+ * training/training_dynamic/mil_dynamic.h:264-266 and training/forward.h:101,149-151. */
+int mi355_swiglu_fwd_dev(float *out, const float *h1, const float *h3, size_t n);
+
+/* SwiGLU gate backward.  Replaces the 13 vDSP/vForce calls of
+ * training/training_dynamic/train.m:537-554: dh3 = dsilu*(h1*sig), dh1 = (dsilu*h3)*(sig*(1+h1*(1-sig))). */
+int mi355_swiglu_bwd_dev(float *dh1, float *dh3, const float *dsilu, const float *h1,
+                         const float *h3, size_t n);
+
+/* cos/sin tables [hd/2][S] (pair-major, positions contiguous), built on the host with libm from
+ * angle = p * (1/powf(theta, 2i/hd)) — the expression of training/training_dynamic/cpu_ops.h:172-175
+ * (theta is 10000 there).  Host pointers. */
+int mi355_rope_tables(float *cos_host, float *sin_host, int S, int hd, float theta);
+/* The same tables resident on the device, cached per (S, hd, theta). */
+int mi355_rope_tables_dev(const float **cos_dev, const float **sin_dev, int S, int hd, float theta);
+
+/* RoPE on Q [batch][heads*hd][S] and K [batch][kv_heads*hd][S], interleaved row pairs (2i,2i+1).
+ * dir = -1 replaces rope_backward_inplace — training/training_dynamic/cpu_ops.h:168-184, called at
+ * training/training_dynamic/train.m:659-660 for dQ (Q_DIM) and dK (KV_DIM); dir = +1 is the forward
+ * rotation (training/forward.h:55-70; training/training_dynamic/mil_dynamic.h:131-168).
+ * In place when q_out == q_in / k_out == k_in.  k_* may be NULL (kv_heads = 0). */
+int mi355_rope_dev(float *q_out, float *k_out, const float *q_in, const float *k_in, int heads,
+                   int kv_heads, int hd, int S, int batch, const float *cos_dev,
+                   const float *sin_dev, int dir);
+
+/* Qwen3 per-head QK-RMSNorm fused with RoPE (one HBM pass).  Not in the reference: equals rmsnorm
+ * (stories_cpu_ops.h:6-21) applied to each head's [hd,S] slab with a [hd] weight shared by the
+ * heads, followed by the forward RoPE above. */
+int mi355_qknorm_rope_fwd_dev(float *q_out, float *k_out, const float *q, const float *k,
+                              const float *wq, const float *wk, int heads, int kv_heads, int hd,
+                              int S, int batch, const float *cos_dev, const float *sin_dev,
+                              float eps);
+/* Backward of the above: inverse rotation (cpu_ops.h:168-184) then rmsnorm_bwd per head
+ * (stories_cpu_ops.h:23-53).  dq/dk assigned; dwq/dwk [hd] accumulated over heads and batch.
+ * q, k are the saved pre-norm inputs. */
+int mi355_qknorm_rope_bwd_dev(float *dq, float *dk, float *dwq, float *dwk, const float *dq_out,
+                              const float *dk_out, const float *q, const float *k, const float *wq,
+                              const float *wk, int heads, int kv_heads, int hd, int S, int batch,
+                              const float *cos_dev, const float *sin_dev, float eps, int variant);
+
+/* Residual family.  mode 0: y = a + alpha*b (vDSP_vsma, training/training_dynamic/train.m:460);
+ * mode 1: y = alpha*a (vDSP_vsmul, train.m:497,523,595); mode 2: y = a + b (vDSP_vadd,
+ * training/train_large.m:427,442; loops at train.m:590,714,721).  y may alias a or b. */
+int mi355_axpby_dev(float *y, const float *a, const float *b, float alpha, size_t n, int mode);
+
+/* Embedding gather.  Replaces embed_lookup — training/stories_cpu_ops.h:112-120,
+ * training/training_dynamic/cpu_ops.h:150-156.  x[b][d][t] = E[ids[b][t]][d]; an id outside
+ * [0,V) leaves its column untouched (the static loop's policy).  Bit-exact copy. */
+int mi355_embed_gather_dev(float *x, const float *E, const int32_t *ids, int V, int D, int S,
+                           int batch);
+
+/* Embedding backward.  Replaces embed_backward — training/stories_cpu_ops.h:123-131,
+ * training/training_dynamic/cpu_ops.h:158-164.  dE[ids[b][t]][d] += dx[b][d][t], each (row, d) sum
+ * taken in ascending (b, t) order starting from the value already in dE, so the result is
+ * bit-identical to the reference loop and run-to-run deterministic.  Ids outside [0,V) are skipped. */
+int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, int V, int D,
+                                int S, int batch);
+
+/* Fused softmax + cross-entropy forward/backward on logits [V][S].  Replaces cross_entropy_loss —
+ * training/training_dynamic/cpu_ops.h:68-93, training/stories_cpu_ops.h:71-108 — and the loss-scale
+ * pass at training/training_dynamic/train.m:497 (grad_scale; 1.0f = none).
+ * dlogits = (softmax - onehot) * (1/S) * grad_scale; *loss_dev = mean_t -logf(p[tgt]+1e-10f).
+ * A target outside [0,V) contributes no loss and leaves its column as the unscaled softmax
+ * (stories_cpu_ops.h:98).  dlogits may alias logits. */
+int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float *logits,
+                         const int32_t *targets, int V, int S, float grad_scale);
+
+/* Per-tensor symmetric INT8.  Replaces the quantizer of ane_bridge_build_weight_blob_quantized —
+ * bridge/ane_bridge.m:346-365 — and the MIL quantize/dequantize pair of ane_int8_bench.m:83-92.
+ * scale = max|x|/127 (1.0 when the tensor is all zero); q = clamp(x/scale, -128, 127) rounded
+ * half-to-even (rounding 0) or half away from zero (rounding 1, the reference's); x^ = q*scale. */
+int mi355_int8_scale_dev(float *scale_dev, const float *x, size_t n);
+int mi355_int8_quant_dev(int8_t *q, const float *x, const float *scale_dev, size_t n, int rounding);
+int mi355_int8_dequant_dev(float *x, const int8_t *q, const float *scale_dev, size_t n);
+
+/* ------------------------------------------------------------------------------------------
+ * Host-pointer drop-ins: the reference signatures verbatim (host float* in, host float* out),
+ * so a caller swaps the symbol only.  Each call stages through cached device buffers
+ * (H2D, kernel, D2H) and returns when the result is in host memory.  On failure they print one
+ * line to stderr and leave the outputs untouched.
+ * ---------------------------------------------------------------------------------------- */
+/* rmsnorm — training/stories_cpu_ops.h:6 */
+void mi355_rmsnorm(float *out, const float *x, const float *w, int d, int S);
+/* rmsnorm_bwd — training/stories_cpu_ops.h:23 */
+void mi355_rmsnorm_bwd(float *dx, float *dw, const float *dy, const float *x, const float *w,
+                       int d, int S);
+/* cross_entropy_loss — training/stories_cpu_ops.h:71, training/training_dynamic/cpu_ops.h:68 */
+float mi355_cross_entropy_loss(float *dlogits, const float *logits, const uint16_t *targets, int V,
+                               int S);
+/* embed_lookup — training/stories_cpu_ops.h:112.  The reference reads the vocabulary size from the
+ * compile-time VOCAB macro; it is an argument here.  The table is kept resident on the device, keyed
+ * by its host address, and re-uploaded after mi355_host_table_invalidate(embed). */
+void mi355_embed_lookup(float *x, const float *embed, const uint16_t *tokens, int vocab, int dim,
+                        int seq);
+void mi355_host_table_invalidate(const float *embed);
+/* embed_backward — training/stories_cpu_ops.h:123 */
+void mi355_embed_backward(float *d_embed, const float *dx, const uint16_t *tokens, int vocab,
+                          int dim, int seq);
+/* rope_backward_inplace — training/training_dynamic/cpu_ops.h:168 (theta = 10000) */
+void mi355_rope_backward_inplace(float *dx, int seq, int dim, int hd);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MI355_BRIDGE_H */

@@ -1,0 +1,557 @@
+/*
+ * oracle.c — CPU restatement of the reference's per-layer CPU ops.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file is the checker the HIP kernels are compared against.  Nothing in the shipped
+ * library links, loads or calls it; only the test-suite, the smoke check and the benchmark's
+ * CPU-baseline leg do.
+ *
+ * The reference implements these ops on top of Apple Accelerate (vDSP / vForce / cblas), a
+ * closed system library with no pinned version that is not part of the reference tree.  Each
+ * function below restates the reference's call sequence with every Accelerate call replaced by
+ * a scalar loop that rounds after every elementary operation (the file is compiled with
+ * -ffp-contract=off), in the same operation order as the reference.  Where Accelerate leaves the
+ * order of a reduction unpublished (vDSP_sve, vDSP_maxv) an 8-lane strided accumulation is used,
+ * which is what a vectorised loop does; the parity tests arbitrate with float64 closed forms.
+ *
+ * All citations are relative to the reference tree.
+ *
+ * Layout: channel-first x[c*S + s] (training/stories_cpu_ops.h:110-118).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <stdio.h>
+#include <time.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* ---------------------------------------------------------------------------------------------
+ * Scalar equivalents of the Accelerate primitives the hot path uses.
+ * ------------------------------------------------------------------------------------------- */
+
+/* vDSP_sve: sum of a vector.  Order unpublished; 8 strided lanes then a fixed horizontal add. */
+static float sve(const float *a, int n) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int i = 0;
+    for (; i + 8 <= n; i += 8)
+        for (int k = 0; k < 8; k++) acc[k] += a[i + k];
+    for (int k = 0; i < n; i++, k++) acc[k] += a[i];
+    float s01 = acc[0] + acc[1], s23 = acc[2] + acc[3], s45 = acc[4] + acc[5], s67 = acc[6] + acc[7];
+    return (s01 + s23) + (s45 + s67);
+}
+
+/* vDSP_maxv: maximum of a vector (exact whatever the order). */
+static float maxv(const float *a, int n) {
+    float m = -INFINITY;
+    for (int i = 0; i < n; i++) if (a[i] > m) m = a[i];
+    return m;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * RMSNorm forward — training/stories_cpu_ops.h:6-21 (twin: training/training_dynamic/cpu_ops.h:7-22)
+ *   ss[s]  = sum_c x[c,s]^2        (vDSP_vmul + vDSP_vadd, sequential over c)
+ *   ss     = ss*(1/d) + eps        (vDSP_vsmsa)
+ *   rr     = 1/sqrt(ss)            (vvrsqrtf)
+ *   out    = (x*rr)*w[c]           (vDSP_vmul then vDSP_vsmul)
+ * The reference hard-codes eps = 1e-5f; it is a parameter here so the per-head QK-norm can share it.
+ * ------------------------------------------------------------------------------------------- */
+static void rrms_columns(float *rr, const float *x, int d, int S, float eps) {
+    for (int s = 0; s < S; s++) rr[s] = 0.0f;
+    for (int i = 0; i < d; i++) {
+        const float *xr = x + (size_t)i * S;
+        for (int s = 0; s < S; s++) {
+            float t = xr[s] * xr[s];
+            rr[s] = t + rr[s];
+        }
+    }
+    float invd = 1.0f / (float)d;
+    for (int s = 0; s < S; s++) {
+        float v = rr[s] * invd;
+        v = v + eps;
+        rr[s] = 1.0f / sqrtf(v);
+    }
+}
+
+ORC_API void orc_rmsnorm(float *out, const float *x, const float *w, int d, int S, float eps) {
+    float *rr = (float *)malloc((size_t)S * sizeof(float));
+    rrms_columns(rr, x, d, S, eps);
+    for (int i = 0; i < d; i++) {
+        const float *xr = x + (size_t)i * S;
+        float *o = out + (size_t)i * S;
+        float wi = w[i];
+        for (int s = 0; s < S; s++) {
+            float t = xr[s] * rr[s];
+            o[s] = t * wi;
+        }
+    }
+    free(rr);
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * RMSNorm backward — training/stories_cpu_ops.h:23-53 (twin: cpu_ops.h:24-54)
+ *   variant 0 (the reference CPU op):
+ *     dot[s] = (sum_c (dy*x)*w[c]) * (rr^2 * (1/d))
+ *     dx     = ((dy - x*dot) * rr) * w[c]          (assigned)
+ *     dw[c] += sum_s (dy*x)*rr                     (accumulated)
+ *   variant 1 (the textbook gradient; training/backward.h:28-42, training/ane_rmsnorm_bwd.h:56-74):
+ *     dx     = (dy*w[c])*rr - x*dot      with the same dot
+ * The two agree when w == 1.
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_rmsnorm_bwd(float *dx, float *dw, const float *dy, const float *x, const float *w,
+                             int d, int S, float eps, int variant) {
+    float *rr = (float *)malloc((size_t)S * sizeof(float));
+    float *dot = (float *)calloc((size_t)S, sizeof(float));
+    float *tmp = (float *)malloc((size_t)S * sizeof(float));
+    rrms_columns(rr, x, d, S, eps);
+    float invd = 1.0f / (float)d;
+    for (int i = 0; i < d; i++) {
+        const float *xr = x + (size_t)i * S, *dyr = dy + (size_t)i * S;
+        float wi = w[i];
+        for (int s = 0; s < S; s++) {
+            float t = dyr[s] * xr[s];
+            float u = t * wi;            /* vDSP_vsma: D = A*b + C */
+            dot[s] = u + dot[s];
+        }
+    }
+    for (int s = 0; s < S; s++) {
+        float q = rr[s] * rr[s];
+        q = q * invd;
+        dot[s] = dot[s] * q;
+    }
+    for (int i = 0; i < d; i++) {
+        const float *xr = x + (size_t)i * S, *dyr = dy + (size_t)i * S;
+        float *dxr = dx + (size_t)i * S;
+        float wi = w[i];
+        if (variant == 0) {
+            for (int s = 0; s < S; s++) {
+                float t = xr[s] * dot[s];
+                t = dyr[s] - t;          /* vDSP_vsub(B,A,C): C = A - B */
+                t = t * rr[s];
+                dxr[s] = t * wi;
+            }
+        } else {
+            for (int s = 0; s < S; s++) {
+                float a = dyr[s] * wi;
+                a = a * rr[s];
+                float b = xr[s] * dot[s];
+                b = b * rr[s];
+                dxr[s] = a - b;
+            }
+        }
+        for (int s = 0; s < S; s++) {
+            float t = dyr[s] * xr[s];
+            tmp[s] = t * rr[s];
+        }
+        dw[i] += sve(tmp, S);
+    }
+    free(rr); free(dot); free(tmp);
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * SwiGLU forward — MIL order training/training_dynamic/mil_dynamic.h:264-266
+ * (sigmoid, mul, mul); scalar twin training/forward.h:101,149-151.
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_swiglu_fwd(float *out, const float *h1, const float *h3, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        float e = expf(-h1[i]);
+        float sig = 1.0f / (1.0f + e);
+        float silu = h1[i] * sig;
+        out[i] = silu * h3[i];
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * SwiGLU backward — the 13-call vDSP/vForce block at training/training_dynamic/train.m:537-554.
+ *   sig = 1/(1+exp(-h1));  dh3 = dsilu*(h1*sig);  dh1 = (dsilu*h3) * (sig*(1 + h1*(1-sig)))
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_swiglu_bwd(float *dh1, float *dh3, const float *dsilu, const float *h1,
+                            const float *h3, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        float t = h1[i] * -1.0f;         /* vsmul */
+        t = expf(t);                     /* vvexpf */
+        t = t + 1.0f;                    /* vsadd */
+        float sig = 1.0f / t;            /* vvrecf */
+        float a = h1[i] * sig;           /* vmul -> dh3 */
+        dh3[i] = dsilu[i] * a;           /* vmul */
+        float u = sig + -1.0f;           /* vsadd */
+        u = -u;                          /* vneg */
+        u = h1[i] * u;                   /* vmul */
+        u = u + 1.0f;                    /* vsadd */
+        u = sig * u;                     /* vmul */
+        float b = dsilu[i] * h3[i];      /* vmul -> dh1 */
+        dh1[i] = b * u;                  /* vmul */
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * RoPE — backward (in place) restates training/training_dynamic/cpu_ops.h:168-184 with theta as
+ * a parameter (the reference hard-codes 10000).  Pairs are interleaved rows (2i, 2i+1) of each
+ * head; angle = p * (1/powf(theta, 2i/hd)).  Forward is the transpose of that rotation, the
+ * convention of training/forward.h:55-70 and of the cos/sin tables at mil_dynamic.h:534-564.
+ * ------------------------------------------------------------------------------------------- */
+static inline float rope_freq(int i, int hd, float theta) {
+    return 1.0f / powf(theta, 2.0f * i / (float)hd);
+}
+
+/* cos/sin tables laid out [hd/2][S] (pair-major, positions contiguous). */
+ORC_API void orc_rope_tables(float *cos_t, float *sin_t, int S, int hd, float theta) {
+    for (int i = 0; i < hd / 2; i++) {
+        float freq = rope_freq(i, hd, theta);
+        for (int p = 0; p < S; p++) {
+            float ang = p * freq;
+            cos_t[(size_t)i * S + p] = cosf(ang);
+            sin_t[(size_t)i * S + p] = sinf(ang);
+        }
+    }
+}
+
+ORC_API void orc_rope_bwd(float *dx, int seq, int dim, int hd, float theta) {
+    int nheads = dim / hd;
+    for (int h = 0; h < nheads; h++)
+        for (int i = 0; i < hd / 2; i++) {
+            float freq = rope_freq(i, hd, theta);
+            for (int p = 0; p < seq; p++) {
+                float ang = p * freq;
+                float c = cosf(ang), s = sinf(ang);
+                size_t i0 = (size_t)(h * hd + 2 * i) * seq + p;
+                size_t i1 = (size_t)(h * hd + 2 * i + 1) * seq + p;
+                float v0 = dx[i0], v1 = dx[i1];
+                dx[i0] = v0 * c + v1 * s;
+                dx[i1] = -v0 * s + v1 * c;
+            }
+        }
+}
+
+ORC_API void orc_rope_fwd(float *x, int seq, int dim, int hd, float theta) {
+    int nheads = dim / hd;
+    for (int h = 0; h < nheads; h++)
+        for (int i = 0; i < hd / 2; i++) {
+            float freq = rope_freq(i, hd, theta);
+            for (int p = 0; p < seq; p++) {
+                float ang = p * freq;
+                float c = cosf(ang), s = sinf(ang);
+                size_t i0 = (size_t)(h * hd + 2 * i) * seq + p;
+                size_t i1 = (size_t)(h * hd + 2 * i + 1) * seq + p;
+                float v0 = x[i0], v1 = x[i1];
+                x[i0] = v0 * c - v1 * s;
+                x[i1] = v0 * s + v1 * c;
+            }
+        }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Qwen3 per-head QK-RMSNorm + RoPE.  Not in the reference: it is the reference rmsnorm applied
+ * to each head's [hd,S] slab with one [hd] weight shared by the heads, followed by the RoPE
+ * above; backward = RoPE backward, then rmsnorm_bwd per head (dw accumulates over heads).
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_qknorm_rope_fwd(float *out, const float *x, const float *w, int nheads, int hd,
+                                 int S, float theta, float eps) {
+    for (int h = 0; h < nheads; h++)
+        orc_rmsnorm(out + (size_t)h * hd * S, x + (size_t)h * hd * S, w, hd, S, eps);
+    orc_rope_fwd(out, S, nheads * hd, hd, theta);
+}
+
+ORC_API void orc_qknorm_rope_bwd(float *dx, float *dw, const float *dy, const float *x,
+                                 const float *w, int nheads, int hd, int S, float theta, float eps,
+                                 int variant) {
+    size_t n = (size_t)nheads * hd * S;
+    float *g = (float *)malloc(n * sizeof(float));
+    memcpy(g, dy, n * sizeof(float));
+    orc_rope_bwd(g, S, nheads * hd, hd, theta);
+    for (int h = 0; h < nheads; h++)
+        orc_rmsnorm_bwd(dx + (size_t)h * hd * S, dw, g + (size_t)h * hd * S,
+                        x + (size_t)h * hd * S, w, hd, S, eps, variant);
+    free(g);
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Residual family.
+ *   mode 0: y = a + alpha*b   vDSP_vsma(b,&alpha,a,y) training/training_dynamic/train.m:460
+ *   mode 1: y = alpha*a       vDSP_vsmul              train.m:497,523,595
+ *   mode 2: y = a + b         vDSP_vadd / scalar loops training/train_large.m:427,442; train.m:590,714,721
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_axpby(float *y, const float *a, const float *b, float alpha, size_t n, int mode) {
+    if (mode == 0) for (size_t i = 0; i < n; i++) { float t = b[i] * alpha; y[i] = t + a[i]; }
+    else if (mode == 1) for (size_t i = 0; i < n; i++) y[i] = a[i] * alpha;
+    else for (size_t i = 0; i < n; i++) y[i] = a[i] + b[i];
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Embedding lookup — training/stories_cpu_ops.h:112-120: x[d*seq+t] = embed[tok*dim+d]; an id
+ * outside [0,V) leaves column t untouched.  Returns the number of ids skipped.
+ * ------------------------------------------------------------------------------------------- */
+ORC_API int orc_embed_lookup(float *x, const float *embed, const int32_t *tokens, int V, int dim,
+                             int seq) {
+    int skipped = 0;
+    for (int t = 0; t < seq; t++) {
+        int tok = tokens[t];
+        if (tok < 0 || tok >= V) { skipped++; continue; }
+        for (int d = 0; d < dim; d++) x[(size_t)d * seq + t] = embed[(size_t)tok * dim + d];
+    }
+    return skipped;
+}
+
+/* Embedding backward — training/stories_cpu_ops.h:123-131: d_embed[tok*dim+d] += dx[d*seq+t]
+ * for t ascending; ids outside [0,V) are skipped. */
+ORC_API void orc_embed_backward(float *d_embed, const float *dx, const int32_t *tokens, int V,
+                                int dim, int seq) {
+    for (int t = 0; t < seq; t++) {
+        int tok = tokens[t];
+        if (tok < 0 || tok >= V) continue;
+        for (int d = 0; d < dim; d++) d_embed[(size_t)tok * dim + d] += dx[(size_t)d * seq + t];
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Softmax + cross-entropy on logits[V,S] — training/training_dynamic/cpu_ops.h:68-93 (column
+ * gather) and training/stories_cpu_ops.h:71-108 (transpose form, with the out-of-range-target
+ * skip at :98 that leaves that column as the unscaled softmax).
+ *   m = max_v; e = exp(l - m); p = e * (1/sum e); loss -= logf(p[tgt] + 1e-10f);
+ *   p[tgt] -= 1; dlogits[:,t] = p * (1/S); return loss/S.
+ * grad_scale folds the separate vDSP_vsmul(dlogits, loss_scale) pass of train.m:497 (1.0f = none).
+ * ------------------------------------------------------------------------------------------- */
+ORC_API float orc_cross_entropy(float *dlogits, const float *logits, const int32_t *targets, int V,
+                                int S, float grad_scale) {
+    float *col = (float *)malloc((size_t)V * sizeof(float));
+    float total = 0.0f, invS = 1.0f / (float)S;
+    for (int t = 0; t < S; t++) {
+        for (int v = 0; v < V; v++) col[v] = logits[(size_t)v * S + t];      /* cblas_scopy */
+        float neg_max = -maxv(col, V);
+        for (int v = 0; v < V; v++) col[v] = col[v] + neg_max;              /* vsadd */
+        for (int v = 0; v < V; v++) col[v] = expf(col[v]);                  /* vvexpf */
+        float inv_sum = 1.0f / sve(col, V);
+        for (int v = 0; v < V; v++) col[v] = col[v] * inv_sum;              /* vsmul */
+        int tgt = targets[t];
+        if (tgt >= 0 && tgt < V) {
+            total -= logf(col[tgt] + 1e-10f);
+            col[tgt] -= 1.0f;
+            for (int v = 0; v < V; v++) col[v] = col[v] * invS;             /* vsmul */
+        }
+        if (grad_scale != 1.0f)
+            for (int v = 0; v < V; v++) col[v] = col[v] * grad_scale;       /* train.m:497 */
+        for (int v = 0; v < V; v++) dlogits[(size_t)v * S + t] = col[v];
+    }
+    free(col);
+    return total / (float)S;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Per-tensor symmetric INT8 — bridge/ane_bridge.m:346-365: scale = max|x|/127 (0 -> 1),
+ * v = x/scale clamped to [-128,127]; rounding 1 = half away from zero (the reference's
+ * (int8_t)(v +- 0.5f)), rounding 0 = round-half-to-even.  Dequantize = q*scale, the MIL
+ * dequantize(scale) of ane_int8_bench.m:83-92.
+ * ------------------------------------------------------------------------------------------- */
+ORC_API float orc_int8_scale(const float *x, size_t n) {
+    float m = 0.0f;
+    for (size_t i = 0; i < n; i++) { float a = x[i] < 0 ? -x[i] : x[i]; if (a > m) m = a; }
+    float scale = m / 127.0f;
+    if (scale == 0.0f) scale = 1.0f;
+    return scale;
+}
+
+ORC_API void orc_int8_quant(int8_t *q, const float *x, size_t n, float scale, int rounding) {
+    for (size_t i = 0; i < n; i++) {
+        float v = x[i] / scale;
+        if (v > 127.0f) v = 127.0f;
+        if (v < -128.0f) v = -128.0f;
+        if (rounding == 1) q[i] = (int8_t)(v + (v >= 0 ? 0.5f : -0.5f));
+        else q[i] = (int8_t)nearbyintf(v);   /* default rounding mode: to nearest, ties to even */
+    }
+}
+
+ORC_API void orc_int8_dequant(float *x, const int8_t *q, size_t n, float scale) {
+    for (size_t i = 0; i < n; i++) x[i] = (float)q[i] * scale;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * GQA tile / reduce — training/training_dynamic/io.h:330-351.
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_gqa_tile(float *out, const float *in, int kv_heads, int ratio, int hd, int seq) {
+    size_t slab = (size_t)hd * seq;
+    for (int kv = 0; kv < kv_heads; kv++)
+        for (int r = 0; r < ratio; r++)
+            memcpy(out + (size_t)(kv * ratio + r) * slab, in + (size_t)kv * slab, slab * sizeof(float));
+}
+
+ORC_API void orc_gqa_reduce(float *out, const float *in, int kv_heads, int ratio, int hd, int seq) {
+    size_t slab = (size_t)hd * seq;
+    memset(out, 0, (size_t)kv_heads * slab * sizeof(float));
+    for (int kv = 0; kv < kv_heads; kv++)
+        for (int r = 0; r < ratio; r++) {
+            const float *src = in + (size_t)(kv * ratio + r) * slab;
+            float *dst = out + (size_t)kv * slab;
+            for (size_t i = 0; i < slab; i++) dst[i] += src[i];
+        }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Adam / AdamW — training/stories_cpu_ops.h:55-63 (wd = 0) and training_dynamic/cpu_ops.h:56-64.
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_adam_update(float *w, const float *g, float *m, float *v, size_t n, int t,
+                             float lr, float b1, float b2, float eps, float wd) {
+    float bc1 = 1.0f - powf(b1, (float)t), bc2 = 1.0f - powf(b2, (float)t);
+    for (size_t i = 0; i < n; i++) {
+        m[i] = b1 * m[i] + (1 - b1) * g[i];
+        v[i] = b2 * v[i] + (1 - b2) * g[i] * g[i];
+        float mh = m[i] / bc1, vh = v[i] / bc2;
+        w[i] -= lr * (mh / (sqrtf(vh) + eps) + wd * w[i]);
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Batched wrappers: the reference processes one [C,S] sequence per call; "batch B" is B calls
+ * on consecutive slabs (dw accumulates across the calls in slab order).  With threads > 1 the
+ * slabs are spread over OpenMP threads (only used for the multi-core CPU baseline; dw then
+ * accumulates per thread and is combined in thread order).
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_rmsnorm_batched(float *out, const float *x, const float *w, int d, int S,
+                                 int batch, float eps, int threads) {
+    size_t slab = (size_t)d * S;
+#pragma omp parallel for num_threads(threads) if (threads > 1)
+    for (int b = 0; b < batch; b++) orc_rmsnorm(out + b * slab, x + b * slab, w, d, S, eps);
+}
+
+ORC_API void orc_rmsnorm_bwd_batched(float *dx, float *dw, const float *dy, const float *x,
+                                     const float *w, int d, int S, int batch, float eps,
+                                     int variant, int threads) {
+    size_t slab = (size_t)d * S;
+    if (threads <= 1) {
+        for (int b = 0; b < batch; b++)
+            orc_rmsnorm_bwd(dx + b * slab, dw, dy + b * slab, x + b * slab, w, d, S, eps, variant);
+        return;
+    }
+    float *part = (float *)calloc((size_t)batch * d, sizeof(float));
+#pragma omp parallel for num_threads(threads)
+    for (int b = 0; b < batch; b++)
+        orc_rmsnorm_bwd(dx + b * slab, part + (size_t)b * d, dy + b * slab, x + b * slab, w, d, S,
+                        eps, variant);
+    for (int b = 0; b < batch; b++)
+        for (int i = 0; i < d; i++) dw[i] += part[(size_t)b * d + i];
+    free(part);
+}
+
+ORC_API void orc_qknorm_rope_fwd_batched(float *out, const float *x, const float *w, int nheads,
+                                         int hd, int S, int batch, float theta, float eps,
+                                         int threads) {
+    size_t slab = (size_t)nheads * hd * S;
+#pragma omp parallel for num_threads(threads) if (threads > 1)
+    for (int b = 0; b < batch; b++)
+        orc_qknorm_rope_fwd(out + b * slab, x + b * slab, w, nheads, hd, S, theta, eps);
+}
+
+ORC_API void orc_qknorm_rope_bwd_batched(float *dx, float *dw, const float *dy, const float *x,
+                                         const float *w, int nheads, int hd, int S, int batch,
+                                         float theta, float eps, int variant, int threads) {
+    size_t slab = (size_t)nheads * hd * S;
+    if (threads <= 1) {
+        for (int b = 0; b < batch; b++)
+            orc_qknorm_rope_bwd(dx + b * slab, dw, dy + b * slab, x + b * slab, w, nheads, hd, S,
+                                theta, eps, variant);
+        return;
+    }
+    float *part = (float *)calloc((size_t)batch * hd, sizeof(float));
+#pragma omp parallel for num_threads(threads)
+    for (int b = 0; b < batch; b++)
+        orc_qknorm_rope_bwd(dx + b * slab, part + (size_t)b * hd, dy + b * slab, x + b * slab, w,
+                            nheads, hd, S, theta, eps, variant);
+    for (int b = 0; b < batch; b++)
+        for (int i = 0; i < hd; i++) dw[i] += part[(size_t)b * hd + i];
+    free(part);
+}
+
+ORC_API void orc_rope_batched(float *x, int seq, int dim, int hd, int batch, float theta, int dir,
+                              int threads) {
+    size_t slab = (size_t)dim * seq;
+#pragma omp parallel for num_threads(threads) if (threads > 1)
+    for (int b = 0; b < batch; b++) {
+        if (dir > 0) orc_rope_fwd(x + b * slab, seq, dim, hd, theta);
+        else orc_rope_bwd(x + b * slab, seq, dim, hd, theta);
+    }
+}
+
+/* elementwise ops split into contiguous ranges per thread */
+ORC_API void orc_swiglu_fwd_mt(float *out, const float *h1, const float *h3, size_t n, int threads) {
+    if (threads <= 1) { orc_swiglu_fwd(out, h1, h3, n); return; }
+#pragma omp parallel for num_threads(threads)
+    for (int k = 0; k < threads; k++) {
+        size_t lo = n * k / threads, hi = n * (k + 1) / threads;
+        orc_swiglu_fwd(out + lo, h1 + lo, h3 + lo, hi - lo);
+    }
+}
+
+ORC_API void orc_swiglu_bwd_mt(float *dh1, float *dh3, const float *dsilu, const float *h1,
+                               const float *h3, size_t n, int threads) {
+    if (threads <= 1) { orc_swiglu_bwd(dh1, dh3, dsilu, h1, h3, n); return; }
+#pragma omp parallel for num_threads(threads)
+    for (int k = 0; k < threads; k++) {
+        size_t lo = n * k / threads, hi = n * (k + 1) / threads;
+        orc_swiglu_bwd(dh1 + lo, dh3 + lo, dsilu + lo, h1 + lo, h3 + lo, hi - lo);
+    }
+}
+
+ORC_API void orc_axpby_mt(float *y, const float *a, const float *b, float alpha, size_t n, int mode,
+                          int threads) {
+    if (threads <= 1) { orc_axpby(y, a, b, alpha, n, mode); return; }
+#pragma omp parallel for num_threads(threads)
+    for (int k = 0; k < threads; k++) {
+        size_t lo = n * k / threads, hi = n * (k + 1) / threads;
+        orc_axpby(y + lo, a + lo, b ? b + lo : NULL, alpha, hi - lo, mode);
+    }
+}
+
+/* batched embedding: sequences b = 0..batch-1 in order (ascending position order overall) */
+ORC_API int orc_embed_lookup_batched(float *x, const float *embed, const int32_t *tokens, int V,
+                                     int dim, int seq, int batch) {
+    int skipped = 0;
+    for (int b = 0; b < batch; b++)
+        skipped += orc_embed_lookup(x + (size_t)b * dim * seq, embed, tokens + (size_t)b * seq, V, dim, seq);
+    return skipped;
+}
+
+ORC_API void orc_embed_backward_batched(float *d_embed, const float *dx, const int32_t *tokens,
+                                        int V, int dim, int seq, int batch) {
+    for (int b = 0; b < batch; b++)
+        orc_embed_backward(d_embed, dx + (size_t)b * dim * seq, tokens + (size_t)b * seq, V, dim, seq);
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Input recipes of the reference's own tests: glibc and Darwin share the POSIX 48-bit LCG, so
+ * srand48(seed)+drand48() regenerate the same streams.
+ *   recipe 0: training/test_rmsnorm_bwd.m:26-33   x=(2u-1)*0.5, dy=(2u-1)*0.1 interleaved; w=0.5u+0.75
+ *   recipe 1: training/test_classifier.m:25-27    x=2u-1; w=0.5u+0.75   (dy untouched)
+ *   recipe 2: training/test_classifier.m:132-134  x=10u-5               (w, dy untouched)
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_recipe_drand48(int recipe, long seed, float *x, float *dy, float *w, size_t n,
+                                int d) {
+    srand48(seed);
+    if (recipe == 0) {
+        for (size_t i = 0; i < n; i++) {
+            x[i] = (float)(drand48() * 2 - 1) * 0.5f;
+            dy[i] = (float)(drand48() * 2 - 1) * 0.1f;
+        }
+        for (int i = 0; i < d; i++) w[i] = (float)(drand48() * 0.5 + 0.75);
+    } else if (recipe == 1) {
+        for (size_t i = 0; i < n; i++) x[i] = (float)(drand48() * 2 - 1);
+        for (int i = 0; i < d; i++) w[i] = (float)(drand48() * 0.5 + 0.75);
+    } else {
+        for (size_t i = 0; i < n; i++) x[i] = (float)(drand48() * 10 - 5);
+    }
+}
+
+ORC_API double orc_now_s(void) {
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+}
+
+ORC_API int orc_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
