@@ -1,0 +1,325 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+One "step" = one pass of the Qwen3-0.6B full-step fused-op sweep (BASELINE config 4) over one
+synthetic batch of 16 x 256 tokens, fp32, channel-first:
+    forward, layers 0..27 : rmsnorm(att) -> qknorm+rope -> residual -> rmsnorm(ffn) -> swiglu -> residual
+    classifier            : softmax + cross-entropy fwd/bwd on logits [151936, 256]
+    backward, layers 27..0: swiglu_bwd -> rmsnorm_bwd(ffn) -> residual -> qknorm+rope bwd -> rmsnorm_bwd(att) -> residual
+    INT8                  : per-tensor scale, quantize, dequantize on [1024, 4096]
+Every layer has its own activation buffers (as a training step has), so each op reads data that
+was last touched a whole sweep ago.  Inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` = tokens/s = 4096 / step time.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0      # MI355X published HBM3E peak
+
+# Qwen3-0.6B (training/training_dynamic/models/qwen3_06b.h:6-16), batch 16
+Q3 = dict(C=1024, H=3072, heads=16, kv_heads=8, hd=128, S=256, batch=16, layers=28, V=151936, theta=1e6,
+          int8_shape=(1024, 4096))
+
+
+def alg_bytes(cfg):
+    """Algorithmic bytes per launch of each op (fp32 = 4 B; St = batch*S columns)."""
+    C, H, S, B = cfg["C"], cfg["H"], cfg["S"], cfg["batch"]
+    St = B * S
+    qkd = (cfg["heads"] + cfg["kv_heads"]) * cfg["hd"]
+    V = cfg["V"]
+    n8 = cfg["int8_shape"][0] * cfg["int8_shape"][1]
+    return {
+        "rmsnorm_fwd": 8 * C * St + 4 * C,
+        "rmsnorm_bwd": 12 * C * St + 12 * C,
+        "qknorm_rope_fwd": 8 * qkd * St,
+        "qknorm_rope_bwd": 12 * qkd * St,
+        "swiglu_fwd": 12 * H * St,
+        "swiglu_bwd": 20 * H * St,
+        "residual": 12 * C * St,
+        "softmax_ce": 8 * V * S,
+        "int8_scale": 4 * n8,
+        "int8_quant": 5 * n8,
+        "int8_dequant": 5 * n8,
+    }
+
+
+class Workload:
+    def __init__(self, br, cfg, layers):
+        self.br, self.cfg, self.L = br, cfg, layers
+        C, H, S, B = cfg["C"], cfg["H"], cfg["S"], cfg["batch"]
+        qd, kd = cfg["heads"] * cfg["hd"], cfg["kv_heads"] * cfg["hd"]
+        A = br.DevArray
+        seed = [1]
+
+        def rnd(*shape, std=1.0, mean=0.0):
+            a = A(shape)
+            br.check(br.lib.mi355_fill_normal_dev(a.ptr, a.size, seed[0], mean, std))
+            seed[0] += 1
+            return a
+
+        self.lay = []
+        for _ in range(layers):
+            d = dict(
+                x=rnd(B, C, S), w_att=rnd(C, std=0.02, mean=1.0), xn=A((B, C, S)),
+                q=rnd(B, qd, S), k=rnd(B, kd, S), wq=rnd(cfg["hd"], std=0.02, mean=1.0),
+                wk=rnd(cfg["hd"], std=0.02, mean=1.0), q_rot=A((B, qd, S)), k_rot=A((B, kd, S)),
+                o=rnd(B, C, S), x2=A((B, C, S)), w_ffn=rnd(C, std=0.02, mean=1.0), x2n=A((B, C, S)),
+                h1=rnd(B, H, S), h3=rnd(B, H, S), gate=A((B, H, S)), f=rnd(B, C, S), x_next=A((B, C, S)),
+                # backward
+                dsilu=rnd(B, H, S), dh1=A((B, H, S)), dh3=A((B, H, S)),
+                dx_ffn=rnd(B, C, S), dx2=A((B, C, S)), dw_ffn=A(C), dy=rnd(B, C, S),
+                gq=rnd(B, qd, S), gk=rnd(B, kd, S), dq=A((B, qd, S)), dk=A((B, kd, S)), dwq=A(cfg["hd"]),
+                dwk=A(cfg["hd"]), dx_attn=rnd(B, C, S), dx1=A((B, C, S)), dw_att=A(C), dy_out=A((B, C, S)),
+            )
+            self.lay.append(d)
+        V = cfg["V"]
+        self.logits = rnd(V, S, std=2.0)
+        self.dlogits = A((V, S))
+        self.targets = A(S, np.int32)
+        br.check(br.lib.mi355_fill_randint_dev(self.targets.ptr, S, 999, 0, V))
+        self.loss = A(1)
+        n8 = cfg["int8_shape"][0] * cfg["int8_shape"][1]
+        self.x8 = rnd(n8)
+        self.q8 = A(n8, np.int8)
+        self.y8 = A(n8)
+        self.scale8 = A(1)
+        self.cos, self.sin = br.rope_tables_dev(S, cfg["hd"], cfg["theta"])
+        self.alpha = float(np.float32(1.0 / np.sqrt(2.0 * cfg["layers"])))   # training/training_dynamic/train.m:188
+        br.sync()
+
+    # ---- single ops on layer buffers d -------------------------------------------------------
+    def op(self, name, d):
+        lib, c, ck = self.br.lib, self.cfg, self.br.check
+        C, H, S, B, hd = c["C"], c["H"], c["S"], c["batch"], c["hd"]
+        n_c, n_h = B * C * S, B * H * S
+        if name == "rmsnorm_fwd":
+            ck(lib.mi355_rmsnorm_fwd_dev(d["xn"].ptr, d["x"].ptr, d["w_att"].ptr, C, S, B, 1e-5))
+        elif name == "rmsnorm_fwd2":
+            ck(lib.mi355_rmsnorm_fwd_dev(d["x2n"].ptr, d["x2"].ptr, d["w_ffn"].ptr, C, S, B, 1e-5))
+        elif name == "qknorm_rope_fwd":
+            ck(lib.mi355_qknorm_rope_fwd_dev(d["q_rot"].ptr, d["k_rot"].ptr, d["q"].ptr, d["k"].ptr, d["wq"].ptr,
+                                             d["wk"].ptr, c["heads"], c["kv_heads"], hd, S, B, self.cos, self.sin, 1e-5))
+        elif name == "residual1":
+            ck(lib.mi355_axpby_dev(d["x2"].ptr, d["x"].ptr, d["o"].ptr, self.alpha, n_c, 0))
+        elif name == "swiglu_fwd":
+            ck(lib.mi355_swiglu_fwd_dev(d["gate"].ptr, d["h1"].ptr, d["h3"].ptr, n_h))
+        elif name == "residual2":
+            ck(lib.mi355_axpby_dev(d["x_next"].ptr, d["x2"].ptr, d["f"].ptr, self.alpha, n_c, 0))
+        elif name == "swiglu_bwd":
+            ck(lib.mi355_swiglu_bwd_dev(d["dh1"].ptr, d["dh3"].ptr, d["dsilu"].ptr, d["h1"].ptr, d["h3"].ptr, n_h))
+        elif name == "rmsnorm_bwd2":
+            ck(lib.mi355_rmsnorm_bwd_dev(d["dx2"].ptr, d["dw_ffn"].ptr, d["dx_ffn"].ptr, d["x2"].ptr, d["w_ffn"].ptr,
+                                         C, S, B, 1e-5, 0))
+        elif name == "residual3":      # dx2 += dy (train.m:590)
+            ck(lib.mi355_axpby_dev(d["dx2"].ptr, d["dx2"].ptr, d["dy"].ptr, 0.0, n_c, 2))
+        elif name == "qknorm_rope_bwd":
+            ck(lib.mi355_qknorm_rope_bwd_dev(d["dq"].ptr, d["dk"].ptr, d["dwq"].ptr, d["dwk"].ptr, d["gq"].ptr,
+                                             d["gk"].ptr, d["q"].ptr, d["k"].ptr, d["wq"].ptr, d["wk"].ptr, c["heads"],
+                                             c["kv_heads"], hd, S, B, self.cos, self.sin, 1e-5, 0))
+        elif name == "rmsnorm_bwd":
+            ck(lib.mi355_rmsnorm_bwd_dev(d["dx1"].ptr, d["dw_att"].ptr, d["dx_attn"].ptr, d["x"].ptr, d["w_att"].ptr,
+                                         C, S, B, 1e-5, 0))
+        elif name == "residual4":      # dy = dx_rms1 + dx2 (train.m:721)
+            ck(lib.mi355_axpby_dev(d["dy_out"].ptr, d["dx1"].ptr, d["dx2"].ptr, 0.0, n_c, 2))
+        else:
+            raise KeyError(name)
+
+    FWD = ["rmsnorm_fwd", "qknorm_rope_fwd", "residual1", "rmsnorm_fwd2", "swiglu_fwd", "residual2"]
+    BWD = ["swiglu_bwd", "rmsnorm_bwd2", "residual3", "qknorm_rope_bwd", "rmsnorm_bwd", "residual4"]
+
+    def ce(self):
+        self.br.check(self.br.lib.mi355_softmax_ce_dev(self.dlogits.ptr, self.loss.ptr, self.logits.ptr,
+                                                       self.targets.ptr, self.cfg["V"], self.cfg["S"], 1.0))
+
+    def int8(self, which=("scale", "quant", "dequant")):
+        lib, n = self.br.lib, self.x8.size
+        if "scale" in which:
+            self.br.check(lib.mi355_int8_scale_dev(self.scale8.ptr, self.x8.ptr, n))
+        if "quant" in which:
+            self.br.check(lib.mi355_int8_quant_dev(self.q8.ptr, self.x8.ptr, self.scale8.ptr, n, 0))
+        if "dequant" in which:
+            self.br.check(lib.mi355_int8_dequant_dev(self.y8.ptr, self.q8.ptr, self.scale8.ptr, n))
+
+    def step(self):
+        for d in self.lay:
+            for name in self.FWD:
+                self.op(name, d)
+        self.ce()
+        for d in reversed(self.lay):
+            for name in self.BWD:
+                self.op(name, d)
+        self.int8()
+
+
+def time_region(br, fn, reps=1):
+    e0, e1 = br.Event(), br.Event()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    return e0.elapsed_ms(e1) / reps
+
+
+def per_op_table(br, wl, reps):
+    """Average launch time of each op over all layer buffers (cold operands), HIP events on the
+    bridge stream."""
+    ab = alg_bytes(wl.cfg)
+    names = {"rmsnorm_fwd": "rmsnorm_fwd", "rmsnorm_bwd": "rmsnorm_bwd", "qknorm_rope_fwd": "qknorm_rope_fwd",
+             "qknorm_rope_bwd": "qknorm_rope_bwd", "swiglu_fwd": "swiglu_fwd", "swiglu_bwd": "swiglu_bwd",
+             "residual1": "residual"}
+    table = []
+    for opname, key in names.items():
+        def run():
+            for d in wl.lay:
+                wl.op(opname, d)
+        run()
+        ms = time_region(br, run, reps) / len(wl.lay)
+        table.append(dict(op=key, ms=ms, alg_mb=ab[key] / 1e6, gbs=ab[key] / ms / 1e6, frac=ab[key] / ms / 1e6 / PEAK_HBM_GBS))
+    for key, fn in (("softmax_ce", wl.ce), ("int8_scale", lambda: wl.int8(("scale",))),
+                    ("int8_quant", lambda: wl.int8(("quant",))), ("int8_dequant", lambda: wl.int8(("dequant",)))):
+        fn()
+        ms = time_region(br, fn, max(reps, 3))
+        table.append(dict(op=key, ms=ms, alg_mb=ab[key] / 1e6, gbs=ab[key] / ms / 1e6, frac=ab[key] / ms / 1e6 / PEAK_HBM_GBS))
+    return table
+
+
+def cpu_baseline(br, wl, sample_layers, threads_mt):
+    """The CPU oracle (clean-room C port of the reference ops, one thread as the reference runs
+    them) timed on a bounded sample: `sample_layers` of the 28 layers plus the full classifier and
+    INT8 ops; the layer time is scaled to 28 layers.  Also returns GPU-vs-oracle parity on that sample."""
+    import oracle as O
+    c = wl.cfg
+    C, H, S, B, hd, L = c["C"], c["H"], c["S"], c["batch"], c["hd"], c["layers"]
+    now = time.perf_counter
+
+    def layer_time(d, threads):
+        h = {k: v.numpy() for k, v in d.items() if k in ("x", "w_att", "q", "k", "wq", "wk", "o", "w_ffn", "h1", "h3",
+                                                         "f", "dsilu", "dx_ffn", "dy", "gq", "gk", "dx_attn")}
+        out = {}
+        t0 = now()
+        out["xn"] = O.rmsnorm(h["x"], h["w_att"], threads=threads)
+        out["q_rot"] = O.qknorm_rope_fwd(h["q"], h["wq"], hd, c["theta"], threads=threads)
+        out["k_rot"] = O.qknorm_rope_fwd(h["k"], h["wk"], hd, c["theta"], threads=threads)
+        out["x2"] = O.axpby(h["x"], h["o"], wl.alpha, 0, threads=threads)
+        out["x2n"] = O.rmsnorm(out["x2"], h["w_ffn"], threads=threads)
+        out["gate"] = O.swiglu_fwd(h["h1"], h["h3"], threads=threads)
+        out["x_next"] = O.axpby(out["x2"], h["f"], wl.alpha, 0, threads=threads)
+        out["dh1"], out["dh3"] = O.swiglu_bwd(h["dsilu"], h["h1"], h["h3"], threads=threads)
+        out["dx2"], out["dw_ffn"] = O.rmsnorm_bwd(h["dx_ffn"], out["x2"], h["w_ffn"], threads=threads)
+        out["dx2"] = O.axpby(out["dx2"], h["dy"], 0.0, 2, threads=threads)
+        out["dq"], out["dwq"] = O.qknorm_rope_bwd(h["gq"], h["q"], h["wq"], hd, c["theta"], threads=threads)
+        out["dk"], out["dwk"] = O.qknorm_rope_bwd(h["gk"], h["k"], h["wk"], hd, c["theta"], threads=threads)
+        out["dx1"], out["dw_att"] = O.rmsnorm_bwd(h["dx_attn"], h["x"], h["w_att"], threads=threads)
+        out["dy_out"] = O.axpby(out["dx1"], out["dx2"], 0.0, 2, threads=threads)
+        return now() - t0, out
+
+    def rel(a, ref):
+        a = np.asarray(a, np.float64).ravel(); ref = np.asarray(ref, np.float64).ravel()
+        rms = float(np.sqrt(np.mean(ref * ref))) or 1.0
+        return float(np.max(np.abs(a - ref) / np.maximum(np.abs(ref), rms)))
+
+    t_layer = []
+    parity = 0.0
+    for i in range(sample_layers):
+        t, out = layer_time(wl.lay[i], 1)
+        t_layer.append(t)
+        if i == 0:
+            # dw buffers accumulate over steps on the GPU; compare the assigned tensors only
+            for k in ("xn", "q_rot", "k_rot", "x2", "x2n", "gate", "x_next", "dh1", "dh3", "dx2", "dq", "dk", "dx1",
+                      "dy_out"):
+                parity = max(parity, rel(wl.lay[0][k].numpy(), out[k]))
+    logits = wl.logits.numpy(); tg = wl.targets.numpy()
+    t0 = now(); loss, dl = O.cross_entropy(logits, tg); t_ce = now() - t0
+    parity = max(parity, rel(wl.dlogits.numpy(), dl), abs(float(wl.loss.numpy()[0]) - loss) / abs(loss))
+    del dl, logits
+    x8 = wl.x8.numpy()
+    t0 = now(); sc = O.int8_scale(x8); q = O.int8_quant(x8, sc, 0); y = O.int8_dequant(q, sc); t_i8 = now() - t0
+    int8_exact = bool(np.array_equal(q, wl.q8.numpy()) and np.array_equal(y, wl.y8.numpy()))
+    t1 = float(np.mean(t_layer)) * L + t_ce + t_i8
+    tokens = B * S
+    res = dict(value=tokens / t1, unit="tokens/s", cores=1, kind="port",
+               sample="%d of %d layers (all 12 layer ops, batch %dx%d) + full softmax-CE [%d,%d] + full INT8 %s; "
+                      "layer time scaled x%d; %.1f s of CPU work" % (sample_layers, L, B, S, c["V"], S,
+                                                                     list(c["int8_shape"]), L,
+                                                                     sum(t_layer) + t_ce + t_i8),
+               seconds_per_step_est=t1)
+    if threads_mt > 1:
+        tm, _ = layer_time(wl.lay[0], threads_mt)
+        res["multithread"] = dict(threads=threads_mt, layer_seconds=tm, layer_speedup=float(np.mean(t_layer)) / tm)
+    return res, parity, int8_exact
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=Q3["layers"], help="layers in the sweep (28 = the named workload)")
+    ap.add_argument("--cpu-layers", type=int, default=2, help="layers in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--op-reps", type=int, default=3)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the path needs no collectives); run with --gpus 1")
+
+    import ane_amd.bridge as br
+    br.init()
+    dev_name, drv_peak, cus = br.device_info()
+    cfg = dict(Q3)
+    wl = Workload(br, cfg, args.layers)
+
+    for _ in range(args.warmup):
+        wl.step()
+    br.sync()
+    t0 = time.perf_counter()
+    ms = time_region(br, wl.step, args.steps)
+    br.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    ab = alg_bytes(cfg)
+    per_layer = (2 * ab["rmsnorm_fwd"] + 2 * ab["rmsnorm_bwd"] + ab["qknorm_rope_fwd"] + ab["qknorm_rope_bwd"] +
+                 ab["swiglu_fwd"] + ab["swiglu_bwd"] + 4 * ab["residual"])
+    total_bytes = args.layers * per_layer + ab["softmax_ce"] + ab["int8_scale"] + ab["int8_quant"] + ab["int8_dequant"]
+    tokens = cfg["batch"] * cfg["S"]
+
+    table = per_op_table(br, wl, args.op_reps)
+    dom = max((r for r in table), key=lambda r: r["alg_mb"] * (args.layers if r["op"] not in
+                                                               ("softmax_ce", "int8_scale", "int8_quant", "int8_dequant") else 1))
+    roofline = dict(bound="hbm", kernel=dom["op"], achieved=dom["gbs"], peak=PEAK_HBM_GBS, unit="GB/s",
+                    frac=dom["gbs"] / PEAK_HBM_GBS, traffic=None, alg_bytes_per_launch=ab[dom["op"]],
+                    avg_launch_ms=dom["ms"])
+
+    out = {
+        "metric": "layer-op tokens/s at Qwen3-0.6B shape (fused-op HBM GB/s and % of peak in `ops`)",
+        "value": tokens / (ms / 1e3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "qwen3-0.6b full-step fused-op sweep (BASELINE config 4): %d layers x 12 fused ops "
+                               "(batch 16 x S 256, C 1024, H 3072, 16/8 heads x 128) + softmax-CE [151936,256] + "
+                               "INT8 [1024,4096]" % args.layers,
+                   "layers": args.layers, "tokens_per_step": tokens, "alg_gb_per_step": total_bytes / 1e9},
+        "aggregate_gbs": total_bytes / ms / 1e6, "aggregate_frac_of_peak": total_bytes / ms / 1e6 / PEAK_HBM_GBS,
+        "host_wall_ms_per_step": wall_ms,
+        "device": dev_name, "compute_units": cus, "driver_reported_peak_gbs": drv_peak,
+        "roofline": roofline,
+        "ops": [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()} for r in table],
+    }
+    if args.cpu_layers > 0:
+        threads = min(16, os.cpu_count() or 1)
+        cpu, parity, int8_exact = cpu_baseline(br, wl, min(args.cpu_layers, args.layers), threads)
+        out["cpu_baseline"] = cpu
+        out["parity_vs_oracle_on_sample"] = {"max_rel_err": parity, "int8_bit_exact": int8_exact}
+        out["gpu_over_cpu"] = out["value"] / cpu["value"]
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

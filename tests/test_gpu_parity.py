@@ -1,0 +1,501 @@
+"""Parity of the HIP path with the CPU oracle, called through the C-ABI (ctypes) on a real MI355X.
+
+Bars: bit-exact for id/byte work (gather, scatter-add, INT8, the residual family); for fp32 ops
+max_i |gpu_i - ref_i| / max(|ref_i|, rms(ref)) <= 1e-5 (helpers.rel_err, TOL_F32)."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import helpers as H
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = H.TOL_F32
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "kat_small.npz"))
+
+
+def dev(br, a):
+    return br.DevArray.from_numpy(a)
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+
+
+# ---------------------------------------------------------------------------------------------
+# RMSNorm
+# ---------------------------------------------------------------------------------------------
+RMS_SHAPES = [
+    (1, 768, 256),      # BASELINE config 0
+    (16, 1024, 256),    # Qwen3-0.6B layer shape
+    (3, 48, 20),        # golden-sized, S % 4 == 0 but narrow
+    (2, 100, 37),       # S % 4 != 0 -> scalar columns
+    (2, 5000, 64),      # C too large for the register tile -> streaming variant
+    (5, 128, 256),      # head-sized C
+    (1, 1, 4),          # degenerate
+]
+
+
+@pytest.mark.parametrize("B,Cc,S", RMS_SHAPES)
+def test_rmsnorm_fwd_bwd(br, B, Cc, S):
+    say("rmsnorm B=%d C=%d S=%d" % (B, Cc, S))
+    x = H.normal(0, (B, Cc, S)); w = H.normal(1, Cc, 1.0, 0.02); dy = H.normal(2, (B, Cc, S))
+    dw0 = H.normal(3, Cc)
+    xd, wd, dyd = dev(br, x), dev(br, w), dev(br, dy)
+    yd = br.DevArray(x.shape); dxd = br.DevArray(x.shape)
+    br.check(br.lib.mi355_rmsnorm_fwd_dev(yd.ptr, xd.ptr, wd.ptr, Cc, S, B, 1e-5))
+    assert H.rel_err(yd.numpy(), O.rmsnorm(x, w)) <= TOL
+    assert H.rel_err(yd.numpy(), H.np_rmsnorm(x, w)) <= TOL
+    for variant in (0, 1):
+        dwd = dev(br, dw0)
+        dxd.upload(np.full(x.shape, 7.0, np.float32))          # dx is assigned, not accumulated
+        br.check(br.lib.mi355_rmsnorm_bwd_dev(dxd.ptr, dwd.ptr, dyd.ptr, xd.ptr, wd.ptr, Cc, S, B, 1e-5, variant))
+        rdx, rdw = O.rmsnorm_bwd(dy, x, w, variant=variant, dw=dw0)
+        assert H.rel_err(dxd.numpy(), rdx) <= TOL
+        assert H.rel_err(dwd.numpy(), rdw) <= TOL
+        if Cc >= 16:        # with a handful of channels dy - x*dot cancels almost exactly: fp32 itself is off by > 1e-5
+            t64dx, t64dw = H.np_rmsnorm_bwd(dy, x, w, variant=variant)
+            assert H.rel_err(dxd.numpy(), t64dx) <= TOL
+            assert H.rel_err(dwd.numpy(), dw0 + t64dw) <= TOL
+
+
+def test_rmsnorm_golden_reference_recipe(br):
+    x, dy, w = GOLD["rms_x"], GOLD["rms_dy"], GOLD["rms_w"]
+    Cc, S = x.shape
+    xd, wd, dyd = dev(br, x), dev(br, w), dev(br, dy)
+    yd = br.DevArray(x.shape); dxd = br.DevArray(x.shape); dwd = br.DevArray(Cc)
+    br.check(br.lib.mi355_rmsnorm_fwd_dev(yd.ptr, xd.ptr, wd.ptr, Cc, S, 1, 1e-5))
+    br.check(br.lib.mi355_rmsnorm_bwd_dev(dxd.ptr, dwd.ptr, dyd.ptr, xd.ptr, wd.ptr, Cc, S, 1, 1e-5, 0))
+    assert H.rel_err(yd.numpy(), GOLD["rms_y"]) <= TOL
+    assert H.rel_err(dxd.numpy(), GOLD["rms_dx_v0"]) <= TOL
+    assert H.rel_err(dwd.numpy(), GOLD["rms_dw"]) <= TOL
+    # the full-size recipe of training/test_rmsnorm_bwd.m:26-33 (DIM 768, SEQ 256, srand48(42))
+    xr, dyr, wr = O.recipe_drand48(0, 42, 768 * 256, 768)
+    xr = xr.reshape(768, 256); dyr = dyr.reshape(768, 256)
+    xd, wd, dyd = dev(br, xr), dev(br, wr), dev(br, dyr)
+    dxd = br.DevArray(xr.shape); dwd = br.DevArray(768)
+    br.check(br.lib.mi355_rmsnorm_bwd_dev(dxd.ptr, dwd.ptr, dyd.ptr, xd.ptr, wd.ptr, 768, 256, 1, 1e-5, 0))
+    rdx, rdw = O.rmsnorm_bwd(dyr, xr, wr)
+    assert H.rel_err(dxd.numpy(), rdx) <= TOL and H.rel_err(dwd.numpy(), rdw) <= TOL
+
+
+def test_rmsnorm_unaligned_pointers_and_every_tile(br):
+    """A tensor that starts 4 bytes into an allocation takes the scalar-column kernel; every
+    register-tile configuration gives the same answer."""
+    B, Cc, S = 2, 96, 64
+    x = H.normal(4, (B, Cc, S)); w = H.normal(5, Cc, 1.0, 0.02); dy = H.normal(6, (B, Cc, S))
+    big = br.DevArray(x.size + 1); bigy = br.DevArray(x.size + 1)
+    br.lib.mi355_buf_write(big.handle, 4, x.ctypes.data, x.nbytes)
+    wd = dev(br, w)
+    br.check(br.lib.mi355_rmsnorm_fwd_dev(bigy.ptr + 4, big.ptr + 4, wd.ptr, Cc, S, B, 1e-5))
+    out = np.empty_like(x)
+    br.lib.mi355_buf_read(bigy.handle, 4, out.ctypes.data, out.nbytes)
+    ref = O.rmsnorm(x, w)
+    assert H.rel_err(out, ref) <= TOL
+    xd, dyd = dev(br, x), dev(br, dy)
+    rdx, rdw = O.rmsnorm_bwd(dy, x, w)
+    try:
+        for lpr in (4, 8, 16):
+            for thr in (256, 1024):
+                say("rmsnorm tile lpr=%d threads=%d" % (lpr, thr))
+                br.tune("rms_lpr", lpr); br.tune("rms_threads", thr)
+                yd = br.DevArray(x.shape); dxd = br.DevArray(x.shape); dwd = br.DevArray(Cc)
+                br.check(br.lib.mi355_rmsnorm_fwd_dev(yd.ptr, xd.ptr, wd.ptr, Cc, S, B, 1e-5))
+                br.check(br.lib.mi355_rmsnorm_bwd_dev(dxd.ptr, dwd.ptr, dyd.ptr, xd.ptr, wd.ptr, Cc, S, B, 1e-5, 0))
+                assert H.rel_err(yd.numpy(), ref) <= TOL
+                assert H.rel_err(dxd.numpy(), rdx) <= TOL and H.rel_err(dwd.numpy(), rdw) <= TOL
+    finally:
+        br.tune("rms_lpr", 0); br.tune("rms_threads", 0)
+
+
+# ---------------------------------------------------------------------------------------------
+# SwiGLU
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [2048 * 256, 3072 * 256 * 16, 1003, 3, 4 * 256 * 8 + 1])
+def test_swiglu_fwd_bwd(br, n):
+    say("swiglu n=%d" % n)
+    h1 = H.normal(10, n); h3 = H.normal(11, n); d = H.normal(12, n)
+    special = np.array([0.0, 30.0, -30.0, 88.0, -88.0, 1e-8, -100.0, 100.0], np.float32)
+    h1[:min(8, n)] = special[:min(8, n)]             # saturating and tiny gate inputs
+    h1d, h3d, dd = dev(br, h1), dev(br, h3), dev(br, d)
+    od = br.DevArray(n); d1 = br.DevArray(n); d3 = br.DevArray(n)
+    br.check(br.lib.mi355_swiglu_fwd_dev(od.ptr, h1d.ptr, h3d.ptr, n))
+    br.check(br.lib.mi355_swiglu_bwd_dev(d1.ptr, d3.ptr, dd.ptr, h1d.ptr, h3d.ptr, n))
+    assert H.rel_err(od.numpy(), O.swiglu_fwd(h1, h3)) <= TOL
+    r1, r3 = O.swiglu_bwd(d, h1, h3)
+    assert H.rel_err(d1.numpy(), r1) <= TOL and H.rel_err(d3.numpy(), r3) <= TOL
+    assert H.rel_err(od.numpy(), H.np_swiglu_fwd(h1, h3)) <= TOL
+    t1, t3 = H.np_swiglu_bwd(d, h1, h3)
+    assert H.rel_err(d1.numpy(), t1) <= TOL and H.rel_err(d3.numpy(), t3) <= TOL
+    assert np.all(np.isfinite(od.numpy())) and np.all(np.isfinite(d1.numpy()))
+
+
+def test_swiglu_golden(br):
+    h1, h3, d = GOLD["sw_h1"], GOLD["sw_h3"], GOLD["sw_d"]
+    n = h1.size
+    h1d, h3d, dd = dev(br, h1), dev(br, h3), dev(br, d)
+    od = br.DevArray(n); d1 = br.DevArray(n); d3 = br.DevArray(n)
+    br.check(br.lib.mi355_swiglu_fwd_dev(od.ptr, h1d.ptr, h3d.ptr, n))
+    br.check(br.lib.mi355_swiglu_bwd_dev(d1.ptr, d3.ptr, dd.ptr, h1d.ptr, h3d.ptr, n))
+    assert H.rel_err(od.numpy(), GOLD["sw_out"]) <= TOL
+    assert H.rel_err(d1.numpy(), GOLD["sw_dh1"]) <= TOL and H.rel_err(d3.numpy(), GOLD["sw_dh3"]) <= TOL
+
+
+# ---------------------------------------------------------------------------------------------
+# residual family: bit-exact
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [768 * 256, 1024 * 256 * 16, 1001, 2])
+def test_axpby_bit_exact(br, n):
+    a = H.normal(20, n); b = H.normal(21, n)
+    ad, bd = dev(br, a), dev(br, b)
+    yd = br.DevArray(n)
+    for alpha in (np.float32(24 ** 0.25), np.float32(1 / np.sqrt(2 * 28))):
+        br.check(br.lib.mi355_axpby_dev(yd.ptr, ad.ptr, bd.ptr, alpha, n, 0))
+        assert np.array_equal(yd.numpy(), O.axpby(a, b, alpha, 0))
+        br.check(br.lib.mi355_axpby_dev(yd.ptr, ad.ptr, None, alpha, n, 1))
+        assert np.array_equal(yd.numpy(), O.axpby(a, None, alpha, 1))
+    br.check(br.lib.mi355_axpby_dev(yd.ptr, ad.ptr, bd.ptr, 0.0, n, 2))
+    assert np.array_equal(yd.numpy(), O.axpby(a, b, 0.0, 2))
+    # in place on a (the dx2 += dy pattern of training/training_dynamic/train.m:590)
+    br.check(br.lib.mi355_axpby_dev(ad.ptr, ad.ptr, bd.ptr, 0.0, n, 2))
+    assert np.array_equal(ad.numpy(), a + b)
+
+
+# ---------------------------------------------------------------------------------------------
+# RoPE
+# ---------------------------------------------------------------------------------------------
+ROPE_CASES = [
+    (1, 12, 12, 64, 256, 10000.0),    # Stories110M, BASELINE config 1
+    (16, 16, 8, 128, 256, 1e6),       # Qwen3-0.6B, GQA 16/8
+    (2, 3, 1, 8, 10, 10000.0),        # S % 4 != 0
+    (1, 4, 0, 16, 8, 1e6),            # Q only
+]
+
+
+@pytest.mark.parametrize("B,h,kvh,hd,S,theta", ROPE_CASES)
+def test_rope_fwd_bwd(br, B, h, kvh, hd, S, theta):
+    say("rope B=%d heads=%d/%d hd=%d S=%d theta=%g" % (B, h, kvh, hd, S, theta))
+    q = H.normal(30, (B, h * hd, S)); k = H.normal(31, (B, max(kvh, 1) * hd, S))
+    cd, sd = br.rope_tables_dev(S, hd, theta)
+    # the host table builder equals the oracle's table bit for bit (same libm, same expression)
+    ch = np.empty((hd // 2, S), np.float32); sh = np.empty((hd // 2, S), np.float32)
+    br.check(br.lib.mi355_rope_tables(ch.ctypes.data, sh.ctypes.data, S, hd, theta))
+    oc, os_ = O.rope_tables(S, hd, theta)
+    assert np.array_equal(ch, oc) and np.array_equal(sh, os_)
+    for direction in (+1, -1):
+        qd, kd = dev(br, q), dev(br, k)
+        qo = br.DevArray(q.shape); ko = br.DevArray(k.shape)
+        br.check(br.lib.mi355_rope_dev(qo.ptr, ko.ptr if kvh else None, qd.ptr, kd.ptr if kvh else None, h, kvh, hd, S,
+                                       B, cd, sd, direction))
+        rq = O.rope(q, hd, theta, direction)
+        assert H.rel_err(qo.numpy(), rq) <= TOL
+        assert np.array_equal(qo.numpy(), rq)          # same table, same operation order: bit-identical
+        if kvh:
+            assert np.array_equal(ko.numpy(), O.rope(k, hd, theta, direction))
+        # in place, as rope_backward_inplace is used (training/training_dynamic/train.m:659-660)
+        br.check(br.lib.mi355_rope_dev(qd.ptr, kd.ptr if kvh else None, qd.ptr, kd.ptr if kvh else None, h, kvh, hd, S,
+                                       B, cd, sd, direction))
+        assert np.array_equal(qd.numpy(), rq)
+        # sanity against float64 angles: the reference's float32 angle p*(1/powf(..)) is itself off by up to
+        # ~|angle| * 2^-23 (angles reach 255 rad), which is what separates the two here
+        assert H.rel_err(qo.numpy(), H.np_rope(q, hd, theta, direction)) <= 2e-4
+
+
+def test_rope_golden(br):
+    x = GOLD["rope_x"]; hd = 16; S = x.shape[1]
+    for theta, tag in ((10000.0, "1e4"), (1e6, "1e6")):
+        cd, sd = br.rope_tables_dev(S, hd, theta)
+        xd = dev(br, x); od = br.DevArray(x.shape)
+        br.check(br.lib.mi355_rope_dev(od.ptr, None, xd.ptr, None, 4, 0, hd, S, 1, cd, sd, +1))
+        assert H.rel_err(od.numpy(), GOLD["rope_fwd_" + tag]) <= TOL
+        br.check(br.lib.mi355_rope_dev(od.ptr, None, xd.ptr, None, 4, 0, hd, S, 1, cd, sd, -1))
+        assert H.rel_err(od.numpy(), GOLD["rope_bwd_" + tag]) <= TOL
+
+
+# ---------------------------------------------------------------------------------------------
+# fused QK-RMSNorm + RoPE
+# ---------------------------------------------------------------------------------------------
+QK_CASES = [
+    (16, 16, 8, 128, 256, 1e6),     # Qwen3-0.6B
+    (2, 12, 12, 64, 256, 10000.0),
+    (2, 3, 2, 16, 24, 1e6),         # narrow strips
+    (1, 2, 1, 8, 10, 1e6),          # S % 4 != 0 -> unfused composition
+    (1, 1, 1, 2048, 16, 1e6),       # head_dim beyond the widest register tile -> unfused composition
+]
+
+
+@pytest.mark.parametrize("B,h,kvh,hd,S,theta", QK_CASES)
+def test_qknorm_rope_fwd_bwd(br, B, h, kvh, hd, S, theta):
+    say("qknorm_rope B=%d heads=%d/%d hd=%d S=%d" % (B, h, kvh, hd, S))
+    q = H.normal(40, (B, h * hd, S)); k = H.normal(41, (B, kvh * hd, S))
+    wq = H.normal(42, hd, 1.0, 0.02); wk = H.normal(43, hd, 1.0, 0.02)
+    gq = H.normal(44, q.shape); gk = H.normal(45, k.shape)
+    dwq0 = H.normal(46, hd); dwk0 = H.normal(47, hd)
+    cd, sd = br.rope_tables_dev(S, hd, theta)
+    qd, kd, wqd, wkd, gqd, gkd = (dev(br, a) for a in (q, k, wq, wk, gq, gk))
+    qo = br.DevArray(q.shape); ko = br.DevArray(k.shape)
+    br.check(br.lib.mi355_qknorm_rope_fwd_dev(qo.ptr, ko.ptr, qd.ptr, kd.ptr, wqd.ptr, wkd.ptr, h, kvh, hd, S, B, cd, sd,
+                                              1e-5))
+    assert H.rel_err(qo.numpy(), O.qknorm_rope_fwd(q, wq, hd, theta)) <= TOL
+    assert H.rel_err(ko.numpy(), O.qknorm_rope_fwd(k, wk, hd, theta)) <= TOL
+    for variant in (0, 1):
+        dq = br.DevArray(q.shape); dk = br.DevArray(k.shape)
+        dwq = dev(br, dwq0); dwk = dev(br, dwk0)
+        br.check(br.lib.mi355_qknorm_rope_bwd_dev(dq.ptr, dk.ptr, dwq.ptr, dwk.ptr, gqd.ptr, gkd.ptr, qd.ptr, kd.ptr,
+                                                  wqd.ptr, wkd.ptr, h, kvh, hd, S, B, cd, sd, 1e-5, variant))
+        rdq, rdwq = O.qknorm_rope_bwd(gq, q, wq, hd, theta, variant=variant, dw=dwq0)
+        rdk, rdwk = O.qknorm_rope_bwd(gk, k, wk, hd, theta, variant=variant, dw=dwk0)
+        assert H.rel_err(dq.numpy(), rdq) <= TOL and H.rel_err(dk.numpy(), rdk) <= TOL
+        assert H.rel_err(dwq.numpy(), rdwq) <= TOL and H.rel_err(dwk.numpy(), rdwk) <= TOL
+
+
+def test_qknorm_rope_golden(br):
+    x, w, dy = GOLD["rope_x"], GOLD["qk_w"], GOLD["qk_dy"]
+    S = x.shape[1]
+    cd, sd = br.rope_tables_dev(S, 16, 1e6)
+    xd, wd, gd = dev(br, x), dev(br, w), dev(br, dy)
+    od = br.DevArray(x.shape); dxd = br.DevArray(x.shape); dwd = br.DevArray(16)
+    br.check(br.lib.mi355_qknorm_rope_fwd_dev(od.ptr, None, xd.ptr, None, wd.ptr, None, 4, 0, 16, S, 1, cd, sd, 1e-5))
+    assert H.rel_err(od.numpy(), GOLD["qk_fwd"]) <= TOL
+    br.check(br.lib.mi355_qknorm_rope_bwd_dev(dxd.ptr, None, dwd.ptr, None, gd.ptr, None, xd.ptr, None, wd.ptr, None, 4,
+                                              0, 16, S, 1, cd, sd, 1e-5, 0))
+    assert H.rel_err(dxd.numpy(), GOLD["qk_dx_v0"]) <= TOL and H.rel_err(dwd.numpy(), GOLD["qk_dw"]) <= TOL
+
+
+# ---------------------------------------------------------------------------------------------
+# embedding
+# ---------------------------------------------------------------------------------------------
+def _embed_case(seed, V, D, B, S, oob=0):
+    E = H.normal(seed, (V, D), 0, 0.02)
+    ids = H.zipf_ids(seed + 1, B * S, V).reshape(B, S)
+    rng = np.random.default_rng(seed + 2)
+    for _ in range(oob):
+        ids[rng.integers(B), rng.integers(S)] = V + int(rng.integers(0, 3)) if rng.random() < 0.5 else -1
+    return E, ids
+
+
+@pytest.mark.parametrize("V,D,B,S,oob", [
+    (32000, 768, 64, 256, 0),     # BASELINE config 2
+    (500, 50, 3, 37, 4),          # ragged D and S, out-of-range ids
+    (70, 4, 1, 1, 0),
+    (1000, 1024, 2, 256, 2),
+])
+def test_embed_gather_bit_exact(br, V, D, B, S, oob):
+    say("gather V=%d D=%d B=%d S=%d" % (V, D, B, S))
+    E, ids = _embed_case(50, V, D, B, S, oob)
+    pre = H.normal(53, (B, D, S))
+    Ed, idd, xd = dev(br, E), dev(br, ids), dev(br, pre)
+    br.check(br.lib.mi355_embed_gather_dev(xd.ptr, Ed.ptr, idd.ptr, V, D, S, B))
+    ref, skipped = O.embed_lookup(E, ids, out=pre)
+    got = xd.numpy()
+    assert got.tobytes() == ref.tobytes()
+    assert skipped == int(((ids < 0) | (ids >= V)).sum())
+
+
+@pytest.mark.parametrize("V,D,B,S,oob", [
+    (32000, 768, 64, 256, 0),     # BASELINE config 2: Zipf(1.1), heavy duplicates
+    (500, 50, 3, 37, 4),
+    (64, 768, 8, 256, 0),         # tiny vocabulary: every segment is long
+    (70, 4, 1, 1, 0),
+    (40, 130, 2, 100, 1),
+])
+def test_embed_scatter_add_bit_exact_and_deterministic(br, V, D, B, S, oob):
+    say("scatter_add V=%d D=%d B=%d S=%d" % (V, D, B, S))
+    _, ids = _embed_case(60, V, D, B, S, oob)
+    dx = H.normal(63, (B, D, S))
+    dE0 = H.normal(64, (V, D), 0, 0.5)
+    idd, dxd = dev(br, ids), dev(br, dx)
+    outs = []
+    for _ in range(2):
+        dEd = dev(br, dE0)
+        br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, idd.ptr, V, D, S, B))
+        outs.append(dEd.numpy())
+    assert outs[0].tobytes() == outs[1].tobytes()                      # run-to-run deterministic
+    ref = O.embed_backward(dE0, dx, ids)
+    assert outs[0].tobytes() == ref.tobytes()                          # the ordered fp32 sum of the reference loop
+
+
+def test_embed_scatter_add_single_hot_token(br):
+    V, D, B, S = 10, 192, 4, 256
+    ids = np.full((B, S), 7, np.int32)
+    dx = H.normal(65, (B, D, S)) * np.float32(100)
+    dE0 = np.zeros((V, D), np.float32)
+    idd, dxd, dEd = dev(br, ids), dev(br, dx), dev(br, dE0)
+    br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, idd.ptr, V, D, S, B))
+    assert dEd.numpy().tobytes() == O.embed_backward(dE0, dx, ids).tobytes()
+
+
+# ---------------------------------------------------------------------------------------------
+# softmax + cross-entropy
+# ---------------------------------------------------------------------------------------------
+def _ce_check(br, logits, tgt, grad_scale=1.0, inplace=False):
+    V, S = logits.shape
+    ld, td = dev(br, logits), dev(br, tgt)
+    dd = ld if inplace else br.DevArray(logits.shape)
+    lossd = br.DevArray(1)
+    br.check(br.lib.mi355_softmax_ce_dev(dd.ptr, lossd.ptr, ld.ptr, td.ptr, V, S, grad_scale))
+    loss = float(lossd.numpy()[0]); dl = dd.numpy()
+    rl, rd = O.cross_entropy(logits, tgt, grad_scale)
+    assert abs(loss - rl) <= TOL * abs(rl) + 1e-12
+    assert H.rel_err(dl, rd) <= TOL
+    tl, td64 = H.np_cross_entropy(logits, tgt, grad_scale)
+    assert abs(loss - tl) <= TOL * abs(tl) + 1e-12
+    assert H.rel_err(dl, td64) <= TOL
+    return loss, dl
+
+
+@pytest.mark.parametrize("V,S", [(32000, 256), (37, 12), (1000, 5), (151936, 256), (300, 1024)])
+def test_softmax_ce(br, V, S):
+    say("softmax_ce V=%d S=%d" % (V, S))
+    logits = H.normal(70, (V, S), 0, 2.0)
+    tgt = np.random.default_rng(71).integers(0, V, S).astype(np.int32)
+    loss, dl = _ce_check(br, logits, tgt)
+    assert np.max(np.abs(dl.astype(np.float64).sum(axis=0))) < 1e-6     # sum_v (p - onehot)/S = 0
+
+
+def test_softmax_ce_golden_policy_scale_inplace(br):
+    logits, tgt = GOLD["ce_logits"], GOLD["ce_targets"]
+    loss, dl = _ce_check(br, logits, tgt)
+    assert abs(loss - float(GOLD["ce_loss"])) <= TOL * float(GOLD["ce_loss"])
+    assert H.rel_err(dl, GOLD["ce_dlogits"]) <= TOL
+    V, S = 4099, 64
+    big = H.normal(72, (V, S), 0, 2.0)
+    t2 = np.random.default_rng(73).integers(0, V, S).astype(np.int32)
+    t2[3] = V; t2[10] = -1; t2[63] = 70000                              # out-of-range targets are skipped
+    _ce_check(br, big, t2)
+    _ce_check(br, big, t2, grad_scale=256.0)                            # loss scaling of train.m:497 fused
+    _ce_check(br, big, t2, inplace=True)
+    # extreme logits: one dominant entry per column, and a constant column
+    ext = H.normal(74, (V, S), 0, 30.0); ext[:, 5] = 3.25
+    _ce_check(br, ext, t2)
+    # the recipe of training/test_classifier.m:132-134 at its own size
+    x, _, _ = O.recipe_drand48(2, 999, 32000 * 256, 0)
+    _ce_check(br, x.reshape(32000, 256), (np.arange(256, dtype=np.int32) * 7 + 13) % 256 + 1)
+
+
+def test_softmax_ce_deterministic(br):
+    V, S = 32000, 256
+    logits = H.normal(75, (V, S), 0, 2.0)
+    tgt = np.random.default_rng(76).integers(0, V, S).astype(np.int32)
+    ld, td = dev(br, logits), dev(br, tgt)
+    res = []
+    for _ in range(2):
+        dd = br.DevArray(logits.shape); lossd = br.DevArray(1)
+        br.check(br.lib.mi355_softmax_ce_dev(dd.ptr, lossd.ptr, ld.ptr, td.ptr, V, S, 1.0))
+        res.append((lossd.numpy().tobytes(), dd.numpy().tobytes()))
+    assert res[0] == res[1]
+
+
+# ---------------------------------------------------------------------------------------------
+# INT8: bit-exact
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [1024 * 4096, 13, 4099])
+def test_int8_bit_exact(br, n):
+    say("int8 n=%d" % n)
+    x = H.normal(80, n) * 3
+    if n > 100:                       # plant exact ties for scale = max|x|/127 = 1/8... use a power-of-two max
+        x = np.clip(x, -15.0, 15.0); x[0] = 15.875        # scale = 15.875/127 = 0.125
+        x[1:9] = [0.0625, 0.1875, 0.3125, -0.0625, -0.1875, -0.3125, 15.8125, -15.8125]   # k + 0.5 after /0.125
+    xd = dev(br, x)
+    sd = br.DevArray(1)
+    br.check(br.lib.mi355_int8_scale_dev(sd.ptr, xd.ptr, n))
+    scale = sd.numpy()[0]
+    assert scale == np.float32(O.int8_scale(x))
+    for mode in (0, 1):
+        qd = br.DevArray(n, np.int8)
+        br.check(br.lib.mi355_int8_quant_dev(qd.ptr, xd.ptr, sd.ptr, n, mode))
+        q = qd.numpy()
+        assert np.array_equal(q, O.int8_quant(x, scale, mode))
+        yd = br.DevArray(n)
+        br.check(br.lib.mi355_int8_dequant_dev(yd.ptr, qd.ptr, sd.ptr, n))
+        assert np.array_equal(yd.numpy(), O.int8_dequant(q, scale))
+        assert np.max(np.abs(yd.numpy().astype(np.float64) - x)) <= scale / 2 * (1 + 1e-6)
+    if n > 100:
+        assert not np.array_equal(O.int8_quant(x, scale, 0)[:9], O.int8_quant(x, scale, 1)[:9])   # ties differ
+
+
+def test_int8_golden_and_zero_tensor(br):
+    x = GOLD["i8_x"]
+    xd = dev(br, x); sd = br.DevArray(1)
+    br.check(br.lib.mi355_int8_scale_dev(sd.ptr, xd.ptr, x.size))
+    assert sd.numpy()[0] == 1.0
+    for mode, key in ((0, "i8_rne"), (1, "i8_away")):
+        qd = br.DevArray(x.size, np.int8)
+        br.check(br.lib.mi355_int8_quant_dev(qd.ptr, xd.ptr, sd.ptr, x.size, mode))
+        assert np.array_equal(qd.numpy(), GOLD[key])
+    zd = dev(br, np.zeros(100, np.float32))
+    br.check(br.lib.mi355_int8_scale_dev(sd.ptr, zd.ptr, 100))
+    assert sd.numpy()[0] == 1.0
+
+
+# ---------------------------------------------------------------------------------------------
+# host-pointer drop-ins (reference signatures) and error behaviour
+# ---------------------------------------------------------------------------------------------
+def _p(a):
+    return a.ctypes.data
+
+
+def test_host_dropins_match_oracle(br):
+    Cc, S = 768, 256
+    x = H.normal(90, (Cc, S)); w = H.normal(91, Cc, 1.0, 0.02); dy = H.normal(92, (Cc, S))
+    out = np.empty_like(x)
+    br.lib.mi355_rmsnorm(_p(out), _p(x), _p(w), Cc, S)
+    assert H.rel_err(out, O.rmsnorm(x, w)) <= TOL
+    dx = np.zeros_like(x); dw = H.normal(93, Cc); dw_in = dw.copy()
+    br.lib.mi355_rmsnorm_bwd(_p(dx), _p(dw), _p(dy), _p(x), _p(w), Cc, S)
+    rdx, rdw = O.rmsnorm_bwd(dy, x, w, dw=dw_in)
+    assert H.rel_err(dx, rdx) <= TOL and H.rel_err(dw, rdw) <= TOL
+
+    V = 5000
+    logits = H.normal(94, (V, S), 0, 2.0)
+    tg = np.random.default_rng(95).integers(0, V, S).astype(np.uint16)
+    dl = np.empty_like(logits)
+    loss = br.lib.mi355_cross_entropy_loss(_p(dl), _p(logits), _p(tg), V, S)
+    rl, rd = O.cross_entropy(logits, tg.astype(np.int32))
+    assert abs(loss - rl) <= TOL * abs(rl) and H.rel_err(dl, rd) <= TOL
+
+    D = 96
+    E = H.normal(96, (V, D), 0, 0.02)
+    tok = H.zipf_ids(97, S, V).astype(np.uint16)
+    xo = np.zeros((D, S), np.float32)
+    br.lib.mi355_embed_lookup(_p(xo), _p(E), _p(tok), V, D, S)
+    assert xo.tobytes() == O.embed_lookup(E, tok.astype(np.int32))[0][0].tobytes()
+    E2 = E.copy(); E2[tok[0]] += 1                                     # the optimizer changed the table
+    E[...] = E2
+    br.lib.mi355_host_table_invalidate(_p(E))
+    br.lib.mi355_embed_lookup(_p(xo), _p(E), _p(tok), V, D, S)
+    assert xo.tobytes() == O.embed_lookup(E, tok.astype(np.int32))[0][0].tobytes()
+    g = H.normal(98, (D, S)); dE = H.normal(99, (V, D)); dE_in = dE.copy()
+    br.lib.mi355_embed_backward(_p(dE), _p(g), _p(tok), V, D, S)
+    assert dE.tobytes() == O.embed_backward(dE_in, g[None], tok.astype(np.int32)[None]).tobytes()
+
+    dq = H.normal(100, (12 * 64, S)); dq_in = dq.copy()
+    br.lib.mi355_rope_backward_inplace(_p(dq), S, 12 * 64, 64)
+    assert np.array_equal(dq, O.rope(dq_in, 64, 10000.0, -1))
+
+
+def test_bad_arguments_fail_cleanly(br):
+    x = dev(br, np.ones((4, 8), np.float32)); y = dev(br, np.full((4, 8), 5.0, np.float32))
+    w = dev(br, np.ones(4, np.float32))
+    assert br.lib.mi355_rmsnorm_fwd_dev(y.ptr, None, w.ptr, 4, 8, 1, 1e-5) == -1
+    assert "NULL" in br.last_error()
+    assert br.lib.mi355_rmsnorm_fwd_dev(y.ptr, x.ptr, w.ptr, 0, 8, 1, 1e-5) == -1
+    assert br.lib.mi355_rmsnorm_bwd_dev(y.ptr, w.ptr, x.ptr, x.ptr, w.ptr, 4, 8, 1, 1e-5, 2) == -1
+    assert br.lib.mi355_swiglu_fwd_dev(y.ptr, x.ptr, x.ptr, 0) == -1
+    assert br.lib.mi355_axpby_dev(y.ptr, x.ptr, None, 1.0, 32, 0) == -1
+    assert br.lib.mi355_axpby_dev(y.ptr, x.ptr, x.ptr, 1.0, 32, 5) == -1
+    assert br.lib.mi355_softmax_ce_dev(y.ptr, None, x.ptr, x.ptr, 4, 8, 1.0) == -1
+    assert br.lib.mi355_int8_quant_dev(y.ptr, x.ptr, w.ptr, 32, 3) == -1
+    assert br.lib.mi355_rope_dev(y.ptr, None, x.ptr, None, 1, 0, 3, 8, 1, x.ptr, x.ptr, 1) == -1     # odd head_dim
+    assert br.lib.mi355_embed_gather_dev(y.ptr, x.ptr, None, 4, 8, 1, 1) == -1
+    assert np.array_equal(y.numpy(), np.full((4, 8), 5.0, np.float32))   # outputs untouched
+    assert br.lib.mi355_tune_set(b"no_such_knob", 1) == -1
+    # buffer accessors ignore bad ranges, as the reference's write_input/read_output do
+    junk = np.zeros(4, np.float32)
+    br.lib.mi355_buf_write(y.handle, 10 ** 9, junk.ctypes.data, 16)
+    br.lib.mi355_buf_read(None, 0, junk.ctypes.data, 16)
+    br.lib.mi355_buf_free(None)
+    assert np.array_equal(y.numpy(), np.full((4, 8), 5.0, np.float32))
