@@ -100,3 +100,9 @@ __device__ __forceinline__ float exp_neg(float d) {
     float e = __builtin_amdgcn_exp2f(hi);
     return __builtin_fmaf(e, lo * 0.693147180559945f, e);
 }
+
+// exp(d) for d <= 0 with a single-float product: relative error up to |d| * 6e-8.  Used where the
+// values are only summed (terms with large |d| are negligible there).
+__device__ __forceinline__ float exp_neg_fast(float d) {
+    return __builtin_amdgcn_exp2f(fmaxf(d, -200.0f) * 1.44269502162933349609375f);
+}

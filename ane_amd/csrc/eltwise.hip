@@ -115,8 +115,8 @@ __global__ __launch_bounds__(EW_THREADS) void axpby_kernel(float *y, const float
     for (int u = 0; u < UNROLL; u++) {
         const size_t i = base + (size_t)u * EW_THREADS;
         if (i < n4) {
-            av[u] = ld4(a + 4 * i);
-            if (MODE != 1) bv[u] = ld4(b + 4 * i);
+            av[u] = ld4_nt(a + 4 * i);
+            if (MODE != 1) bv[u] = ld4_nt(b + 4 * i);
         }
     }
 #pragma unroll
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(EW_THREADS) void axpby_kernel(float *y, const float
             if (MODE == 0) o = bv[u] * alpha + av[u];
             else if (MODE == 1) o = av[u] * alpha;
             else o = av[u] + bv[u];
-            st4(y + 4 * i, o);
+            st4_nt(y + 4 * i, o);
         }
     }
 }
@@ -190,41 +190,50 @@ __global__ __launch_bounds__(EW_THREADS) void rope_kernel(float *q_out, float *k
 }
 
 // ---- INT8 ----
-// max|x| over the tensor; non-negative floats order like their bit patterns, so an integer
-// atomicMax gives an exact, order-independent result.
-__global__ __launch_bounds__(EW_THREADS) void absmax_kernel(unsigned int *out_bits, const float *__restrict__ x,
-                                                            size_t n, size_t n4) {
+// max|x| over the tensor in two launches: per-workgroup maxima, then one workgroup folds them and
+// writes scale = max/127 (1.0 for an all-zero tensor).  max is exact whatever the order.
+__global__ __launch_bounds__(EW_THREADS) void absmax_kernel(float *__restrict__ part, const float *__restrict__ x,
+                                                            size_t n, size_t n4, bool vec) {
     __shared__ float red[EW_THREADS / 64];
     float m = 0.f;
     const size_t stride = (size_t)gridDim.x * EW_THREADS;
-    for (size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x; i < n4; i += stride) {
-        v4f v = ld4(x + 4 * i);
+    const size_t tid = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;
+    if (vec) {
+        for (size_t i = tid; i < n4; i += stride) {
+            v4f v = ld4(x + 4 * i);
 #pragma unroll
-        for (int j = 0; j < 4; j++) m = fmaxf(m, fabsf(v[j]));
+            for (int j = 0; j < 4; j++) m = fmaxf(m, fabsf(v[j]));
+        }
+        if (blockIdx.x == 0)
+            for (size_t i = n4 * 4 + threadIdx.x; i < n; i += EW_THREADS) m = fmaxf(m, fabsf(x[i]));
+    } else {
+        for (size_t i = tid; i < n; i += stride) m = fmaxf(m, fabsf(x[i]));
     }
-    if (blockIdx.x == 0)
-        for (size_t i = n4 * 4 + threadIdx.x; i < n; i += EW_THREADS) m = fmaxf(m, fabsf(x[i]));
 #pragma unroll
     for (int k = 1; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int k = 1; k < EW_THREADS / 64; k++) m = fmaxf(m, red[k]);
-        atomicMax(out_bits, __float_as_uint(m));
+        part[blockIdx.x] = m;
     }
 }
 
-__global__ void absmax_scalar_kernel(unsigned int *out_bits, const float *x, size_t n) {
+__global__ __launch_bounds__(1024) void scale_from_partials_kernel(float *scale, const float *__restrict__ part,
+                                                                   int nblk) {
+    __shared__ float red[16];
     float m = 0.f;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-        m = fmaxf(m, fabsf(x[i]));
-    atomicMax(out_bits, __float_as_uint(m));
-}
-
-__global__ void scale_from_absmax_kernel(float *scale) {
-    float s = *scale / 127.0f;        // *scale holds max|x| (bits written by atomicMax)
-    if (s == 0.0f) s = 1.0f;
-    *scale = s;
+    for (int i = threadIdx.x; i < nblk; i += 1024) m = fmaxf(m, part[i]);
+#pragma unroll
+    for (int k = 1; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 1; k < 16; k++) m = fmaxf(m, red[k]);
+        float s = m / 127.0f;
+        if (s == 0.0f) s = 1.0f;
+        *scale = s;
+    }
 }
 
 __device__ __forceinline__ int quant1(float x, float scale, int rounding) {
@@ -292,6 +301,8 @@ __global__ void dequant_scalar(float *x, const int8_t *q, const float *scale_p, 
     if (i < n) x[i] = (float)q[i] * *scale_p;
 }
 
+// One 128-bit access per lane and as many workgroups as that takes measured fastest on MI355X
+// (75-77 % of peak for the SwiGLU streams against 68-70 % with four accesses per lane).
 inline int pick_unroll(size_t n4, int deflt) {
     int u = g_ctx.ew_unroll ? g_ctx.ew_unroll : deflt;
     if (u != 1 && u != 2 && u != 4 && u != 8) u = deflt;
@@ -315,8 +326,6 @@ inline int pick_unroll(size_t n4, int deflt) {
         }                                                                                                  \
     } while (0)
 
-__global__ void fill_zero_u32(unsigned int *p) { *p = 0u; }
-
 }   // namespace
 
 // n4 vector part + scalar tail split used by every elementwise op
@@ -332,7 +341,7 @@ MI355_API int mi355_swiglu_fwd_dev(float *out, const float *h1, const float *h3,
     size_t n4, lo;
     split_vec(n, aligned16(out) && aligned16(h1) && aligned16(h3), n4, lo);
     if (n4) {
-        const int u = pick_unroll(n4, 4);
+        const int u = pick_unroll(n4, 1);
         EW_LAUNCH(swiglu_fwd_kernel, u, n4, out, h1, h3, n4);
         LAUNCH_OK("swiglu_fwd");
     }
@@ -352,7 +361,7 @@ MI355_API int mi355_swiglu_bwd_dev(float *dh1, float *dh3, const float *dsilu, c
     size_t n4, lo;
     split_vec(n, aligned16(dh1) && aligned16(dh3) && aligned16(dsilu) && aligned16(h1) && aligned16(h3), n4, lo);
     if (n4) {
-        const int u = pick_unroll(n4, 2);
+        const int u = pick_unroll(n4, 1);
         EW_LAUNCH(swiglu_bwd_kernel, u, n4, dh1, dh3, dsilu, h1, h3, n4);
         LAUNCH_OK("swiglu_bwd");
     }
@@ -369,7 +378,7 @@ static int axpby_run(float *y, const float *a, const float *b, float alpha, size
     size_t n4, lo;
     split_vec(n, aligned16(y) && aligned16(a) && (MODE == 1 || aligned16(b)), n4, lo);
     if (n4) {
-        const int u = pick_unroll(n4, 4);
+        const int u = pick_unroll(n4, 1);
         switch (u) {
             case 8: hipLaunchKernelGGL((axpby_kernel<MODE, 8>), dim3((unsigned)ceil_div(n4, (size_t)EW_THREADS * 8)), dim3(EW_THREADS), 0, g_ctx.stream, y, a, b, alpha, n4); break;
             case 4: hipLaunchKernelGGL((axpby_kernel<MODE, 4>), dim3((unsigned)ceil_div(n4, (size_t)EW_THREADS * 4)), dim3(EW_THREADS), 0, g_ctx.stream, y, a, b, alpha, n4); break;
@@ -488,20 +497,14 @@ MI355_API int mi355_int8_scale_dev(float *scale_dev, const float *x, size_t n) {
     if (!mi355_ready("int8_scale")) return -1;
     if (!scale_dev || !x) return mi355_fail("int8_scale: NULL pointer");
     if (n == 0) return mi355_fail("int8_scale: empty tensor");
-    hipLaunchKernelGGL(fill_zero_u32, dim3(1), dim3(1), 0, g_ctx.stream, (unsigned int *)scale_dev);
-    if (aligned16(x)) {
-        const size_t n4 = n / 4;
-        size_t blocks = ceil_div(n4 ? n4 : 1, (size_t)EW_THREADS * 4);
-        if (blocks > 2048) blocks = 2048;
-        hipLaunchKernelGGL(absmax_kernel, dim3((unsigned)blocks), dim3(EW_THREADS), 0, g_ctx.stream,
-                           (unsigned int *)scale_dev, x, n, n4);
-    } else {
-        size_t blocks = ceil_div(n, 256 * 16);
-        if (blocks > 2048) blocks = 2048;
-        hipLaunchKernelGGL(absmax_scalar_kernel, dim3((unsigned)blocks), dim3(256), 0, g_ctx.stream,
-                           (unsigned int *)scale_dev, x, n);
-    }
-    hipLaunchKernelGGL(scale_from_absmax_kernel, dim3(1), dim3(1), 0, g_ctx.stream, scale_dev);
+    const bool vec = aligned16(x);
+    const size_t n4 = vec ? n / 4 : 0;
+    size_t blocks = ceil_div(vec ? (n4 ? n4 : 1) : n, (size_t)EW_THREADS);
+    if (blocks > 4096) blocks = 4096;
+    float *part = (float *)mi355_ws(blocks * sizeof(float));
+    if (!part) return -1;
+    hipLaunchKernelGGL(absmax_kernel, dim3((unsigned)blocks), dim3(EW_THREADS), 0, g_ctx.stream, part, x, n, n4, vec);
+    hipLaunchKernelGGL(scale_from_partials_kernel, dim3(1), dim3(1024), 0, g_ctx.stream, scale_dev, part, (int)blocks);
     LAUNCH_OK("int8_scale");
     return 0;
 }
@@ -514,7 +517,7 @@ MI355_API int mi355_int8_quant_dev(int8_t *q, const float *x, const float *scale
     size_t n4, lo;
     split_vec(n, aligned16(x) && ((uintptr_t)q & 3u) == 0, n4, lo);
     if (n4) {
-        const int u = pick_unroll(n4, 4);
+        const int u = pick_unroll(n4, 1);
         EW_LAUNCH(quant_kernel, u, n4, (int *)q, x, scale_dev, n4, rounding);
         LAUNCH_OK("int8_quant");
     }
@@ -533,7 +536,7 @@ MI355_API int mi355_int8_dequant_dev(float *x, const int8_t *q, const float *sca
     size_t n4, lo;
     split_vec(n, aligned16(x) && ((uintptr_t)q & 3u) == 0, n4, lo);
     if (n4) {
-        const int u = pick_unroll(n4, 4);
+        const int u = pick_unroll(n4, 1);
         EW_LAUNCH(dequant_kernel, u, n4, x, (const int *)q, scale_dev, n4);
         LAUNCH_OK("int8_dequant");
     }

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(THREADS) void rms_fwd_kernel(float *__restrict__ y,
         for (int k = 0; k < CAP; k++) {
             const int c = row0 + k * RPS;
             if (c < C && col_ok) {
-                ldv<VEC>(xv[k], xs + (size_t)c * S);
+                ldv_nt<VEC>(xv[k], xs + (size_t)c * S);
                 wv[k] = w[c];
             } else {
 #pragma unroll
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(THREADS) void rms_fwd_kernel(float *__restrict__ y,
                 float o[VEC];
 #pragma unroll
                 for (int j = 0; j < VEC; j++) o[j] = (xv[k][j] * rr[j]) * wv[k];
-                stv<VEC>(ys + (size_t)c * S, o);
+                stv_nt<VEC>(ys + (size_t)c * S, o);
             }
         }
     } else {
@@ -87,11 +87,11 @@ __global__ __launch_bounds__(THREADS) void rms_fwd_kernel(float *__restrict__ y,
         if (col_ok)
             for (int c = row0; c < C; c += RPS) {
                 float t[VEC], o[VEC];
-                ldv<VEC>(t, xs + (size_t)c * S);
+                ldv_nt<VEC>(t, xs + (size_t)c * S);
                 const float wc = w[c];
 #pragma unroll
                 for (int j = 0; j < VEC; j++) o[j] = (t[j] * rr[j]) * wc;
-                stv<VEC>(ys + (size_t)c * S, o);
+                stv_nt<VEC>(ys + (size_t)c * S, o);
             }
     }
 }
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
             else o[j] = (dyr[j] * wc) * rr[j] - (xr[j] * dotn[j]) * rr[j];
             p += (dyr[j] * xr[j]) * rr[j];
         }
-        if (col_ok) stv<VEC>(dxs + (size_t)c * S, o);
+        if (col_ok) stv_nt<VEC>(dxs + (size_t)c * S, o);
         p = group_sum<(LPR < 64 ? LPR : 64)>(p);
         if (lc == 0) part[c] = p;
     };
@@ -147,8 +147,8 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
         for (int k = 0; k < CAP; k++) {
             const int c = row0 + k * RPS;
             if (c < C && col_ok) {
-                ldv<VEC>(xv[k], xs + (size_t)c * S);
-                ldv<VEC>(dv[k], dys + (size_t)c * S);
+                ldv_nt<VEC>(xv[k], xs + (size_t)c * S);
+                ldv_nt<VEC>(dv[k], dys + (size_t)c * S);
                 wv[k] = w[c];
             } else {
 #pragma unroll
@@ -190,8 +190,8 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
         for (int c = row0; c < C; c += RPS) {
             float a[VEC], b[VEC];
             if (col_ok) {
-                ldv<VEC>(a, xs + (size_t)c * S);
-                ldv<VEC>(b, dys + (size_t)c * S);
+                ldv_nt<VEC>(a, xs + (size_t)c * S);
+                ldv_nt<VEC>(b, dys + (size_t)c * S);
             } else {
 #pragma unroll
                 for (int j = 0; j < VEC; j++) a[j] = b[j] = 0.f;
@@ -201,32 +201,132 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
     }
 }
 
-// out[c] += sum_r part[r][c], rows taken in a fixed order: 16 interleaved row groups, each
+
+// y = a + alpha*b ; yn = (y * rsqrt(mean_c y^2 + eps)) * w — the residual add and the RMSNorm that
+// follows it (training/training_dynamic/train.m:460-461) in one launch.
+template <int VEC, int LPR, int THREADS, int CAP>
+__global__ __launch_bounds__(THREADS) void res_rms_fwd_kernel(float *y, float *__restrict__ yn, const float *a,
+                                                              const float *b, float alpha,
+                                                              const float *__restrict__ w, int C, int S, int strips,
+                                                              int nblk, float eps, float invC) {
+    constexpr int RPS = THREADS / LPR;
+    constexpr int W = LPR * VEC;
+    constexpr int NW = THREADS / 64;
+    __shared__ float lds[NW * 1 * (LPR < 64 ? LPR : 64) * VEC];
+    const int blk = xcd_remap(blockIdx.x, nblk);
+    const int slab = blk / strips, strip = blk - slab * strips;
+    const int lc = threadIdx.x % LPR, row0 = threadIdx.x / LPR;
+    const int col = strip * W + lc * VEC;
+    const bool col_ok = col < S;
+    const size_t base = (size_t)slab * C * S + col;
+    float acc[1][VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc[0][j] = 0.f;
+    if constexpr (CAP > 0) {
+        // y stays in registers between the two stores
+        float yv[CAP][VEC], wv[CAP];
+#pragma unroll
+        for (int k = 0; k < CAP; k++) {
+            const int c = row0 + k * RPS;
+            if (c < C && col_ok) {
+                float bv[VEC];
+                ldv_nt<VEC>(yv[k], a + base + (size_t)c * S);
+                ldv_nt<VEC>(bv, b + base + (size_t)c * S);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) yv[k][j] = bv[j] * alpha + yv[k][j];
+                wv[k] = w[c];
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) yv[k][j] = 0.f;
+                wv[k] = 0.f;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < CAP; k++) {
+            const int c = row0 + k * RPS;
+            if (c < C && col_ok) stv_nt<VEC>(y + base + (size_t)c * S, yv[k]);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc[0][j] += yv[k][j] * yv[k][j];
+        }
+        strip_reduce<VEC, LPR, THREADS, 1>(acc, lds);
+        float rr[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; j++) rr[j] = 1.0f / sqrtf(acc[0][j] * invC + eps);
+#pragma unroll
+        for (int k = 0; k < CAP; k++) {
+            const int c = row0 + k * RPS;
+            if (c < C && col_ok) {
+                float o[VEC];
+#pragma unroll
+                for (int j = 0; j < VEC; j++) o[j] = (yv[k][j] * rr[j]) * wv[k];
+                stv_nt<VEC>(yn + base + (size_t)c * S, o);
+            }
+        }
+    } else {
+        // y is stored in the first sweep and read back by the same lane in the second
+        if (col_ok)
+            for (int c = row0; c < C; c += RPS) {
+                float av[VEC], bv[VEC], t[VEC];
+                ldv_nt<VEC>(av, a + base + (size_t)c * S);
+                ldv_nt<VEC>(bv, b + base + (size_t)c * S);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) {
+                    t[j] = bv[j] * alpha + av[j];
+                    acc[0][j] += t[j] * t[j];
+                }
+                stv<VEC>(y + base + (size_t)c * S, t);
+            }
+        strip_reduce<VEC, LPR, THREADS, 1>(acc, lds);
+        float rr[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; j++) rr[j] = 1.0f / sqrtf(acc[0][j] * invC + eps);
+        if (col_ok)
+            for (int c = row0; c < C; c += RPS) {
+                float t[VEC], o[VEC];
+                ldv<VEC>(t, y + base + (size_t)c * S);
+                const float wc = w[c];
+#pragma unroll
+                for (int j = 0; j < VEC; j++) o[j] = (t[j] * rr[j]) * wc;
+                stv_nt<VEC>(yn + base + (size_t)c * S, o);
+            }
+    }
+}
+
+// out[c] += sum_r part[r][c], rows taken in a fixed order: 32 interleaved row groups, each
 // summed with four independent accumulators (so four loads are in flight), then combined in a
-// fixed order.  One workgroup handles 64 channels.
-__global__ __launch_bounds__(1024) void reduce_rows_kernel(float *__restrict__ out, const float *__restrict__ part,
-                                                           int nrows, int C) {
-    __shared__ float lds[16][64];
-    const int cl = threadIdx.x & 63, g = threadIdx.x >> 6;
-    const int c = blockIdx.x * 64 + cl;
+// fixed order.  One workgroup handles 32 channels; blockIdx.y selects one of two jobs so that
+// two reductions (dwq and dwk) share a launch.
+struct ReduceJob {
+    float *out;
+    const float *part;
+    int nrows;
+};
+
+__global__ __launch_bounds__(1024) void reduce_rows_kernel(ReduceJob j0, ReduceJob j1, int C) {
+    __shared__ float lds[32][33];
+    const ReduceJob job = blockIdx.y == 0 ? j0 : j1;
+    const int cl = threadIdx.x & 31, g = threadIdx.x >> 5;
+    const int c = blockIdx.x * 32 + cl;
+    const float *__restrict__ part = job.part;
+    const int nrows = job.nrows;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     if (c < C) {
         int r = g;
-        for (; r + 48 < nrows; r += 64) {
+        for (; r + 96 < nrows; r += 128) {
             s0 += part[(size_t)r * C + c];
-            s1 += part[(size_t)(r + 16) * C + c];
-            s2 += part[(size_t)(r + 32) * C + c];
-            s3 += part[(size_t)(r + 48) * C + c];
+            s1 += part[(size_t)(r + 32) * C + c];
+            s2 += part[(size_t)(r + 64) * C + c];
+            s3 += part[(size_t)(r + 96) * C + c];
         }
-        for (; r < nrows; r += 16) s0 += part[(size_t)r * C + c];
+        for (; r < nrows; r += 32) s0 += part[(size_t)r * C + c];
     }
     lds[g][cl] = (s0 + s1) + (s2 + s3);
     __syncthreads();
     if (g == 0 && c < C) {
         float t = 0.f;
 #pragma unroll
-        for (int k = 0; k < 16; k++) t += lds[k][cl];
-        out[c] = out[c] + t;
+        for (int k = 0; k < 32; k++) t += lds[k][cl];
+        job.out[c] = job.out[c] + t;
     }
 }
 
@@ -236,9 +336,18 @@ struct NormCfg {
 
 // Picks the tile: registers when the rows fit, and the narrowest strip needed to give every
 // compute unit at least two workgroups.
-NormCfg pick_cfg(int C, int S, int batch, bool vec_ok, int max_cap, int lpr_knob, int thr_knob) {
+NormCfg pick_cfg(int C, int S, int batch, bool vec_ok, int max_cap, int max_cap_1024, int lpr_knob, int thr_knob,
+                 bool backward) {
     NormCfg best{};
     if (!vec_ok) return NormCfg{1, 64, 256, 0};
+    if (!lpr_knob && !thr_knob && C >= 512) {
+        // Tall tensors, measured on MI355X at C=1024 and 16x256 columns: 16 waves per workgroup win.
+        // forward: 64-byte strips held in registers, 9.6 us; backward: 128-byte strips read twice
+        // (second read from L2), 17.7 us against 20.9 us for the single-pass register tile.
+        if (!backward) return NormCfg{4, 4, 1024, C <= 2048 ? 8 : 0};
+        const long strips8 = (long)ceil_div((size_t)S, 32);
+        return NormCfg{4, strips8 * batch >= 128 ? 8 : 4, 1024, 0};
+    }
     const int lprs[3] = {16, 8, 4};
     const int thrs[2] = {256, 1024};
     const int caps[2] = {8, 16};
@@ -251,7 +360,7 @@ NormCfg pick_cfg(int C, int S, int batch, bool vec_ok, int max_cap, int lpr_knob
             int cap = 0;
             for (int cp : caps)
                 if (cp <= max_cap && (long)cp * rps >= C) { cap = cp; break; }
-            if (thr == 1024 && cap > 8) cap = 0;   // 16 waves per CU leave 128 VGPRs per lane
+            if (thr == 1024 && cap > max_cap_1024) cap = 0;   // 16 waves per CU leave 128 VGPRs per lane
             const long strips = ceil_div((size_t)S, (size_t)lpr * 4);
             const long nblk = strips * batch;
             long score = (cap > 0 ? 1000000 : 0);
@@ -309,11 +418,17 @@ void launch_bwd(float *dx, float *part, const float *dy, const float *x, const f
 
 }   // namespace
 
-int mi355_reduce_rows(float *out, const float *part, int nrows, int C) {
-    hipLaunchKernelGGL(reduce_rows_kernel, dim3((unsigned)ceil_div((size_t)C, 64)), dim3(1024), 0, g_ctx.stream, out,
-                       part, nrows, C);
+int mi355_reduce_rows2(float *out0, const float *part0, int nrows0, float *out1, const float *part1, int nrows1,
+                       int C) {
+    const int jobs = (out1 && nrows1 > 0) ? 2 : 1;
+    hipLaunchKernelGGL(reduce_rows_kernel, dim3((unsigned)ceil_div((size_t)C, 32), jobs), dim3(1024), 0, g_ctx.stream,
+                       ReduceJob{out0, part0, nrows0}, ReduceJob{out1, part1, nrows1}, C);
     LAUNCH_OK("reduce_rows");
     return 0;
+}
+
+int mi355_reduce_rows(float *out, const float *part, int nrows, int C) {
+    return mi355_reduce_rows2(out, part, nrows, nullptr, nullptr, 0, C);
 }
 
 MI355_API int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, int C, int S, int batch, float eps) {
@@ -321,7 +436,7 @@ MI355_API int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, in
     if (!y || !x || !w) return mi355_fail("rmsnorm_fwd: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_fwd: bad shape C=%d S=%d batch=%d", C, S, batch);
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(y);
-    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 16, g_ctx.rms_lpr, g_ctx.rms_threads);
+    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 16, 8, g_ctx.rms_lpr, g_ctx.rms_threads, false);
     NORM_DISPATCH(launch_fwd, cfg, y, x, w, C, S, batch, eps);
     LAUNCH_OK("rmsnorm_fwd");
     return 0;
@@ -334,7 +449,7 @@ MI355_API int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_bwd: bad shape C=%d S=%d batch=%d", C, S, batch);
     if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd: variant must be 0 or 1");
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(dy) && aligned16(dx);
-    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 16, g_ctx.rms_lpr, g_ctx.rms_threads);
+    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 16, 0, g_ctx.rms_lpr, g_ctx.rms_threads, true);
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
     float *part = (float *)mi355_ws((size_t)nblk * C * sizeof(float));
@@ -342,4 +457,30 @@ MI355_API int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const
     NORM_DISPATCH(launch_bwd, cfg, dx, part, dy, x, w, C, S, batch, eps, variant);
     LAUNCH_OK("rmsnorm_bwd");
     return mi355_reduce_rows(dw, part, nblk, C);
+}
+
+MI355_API int mi355_residual_rmsnorm_fwd_dev(float *y, float *yn, const float *a, const float *b, float alpha,
+                                             const float *w, int C, int S, int batch, float eps) {
+    if (!mi355_ready("residual_rmsnorm_fwd")) return -1;
+    if (!y || !yn || !a || !b || !w) return mi355_fail("residual_rmsnorm_fwd: NULL pointer");
+    if (C <= 0 || S <= 0 || batch <= 0)
+        return mi355_fail("residual_rmsnorm_fwd: bad shape C=%d S=%d batch=%d", C, S, batch);
+    if (yn == y || yn == a || yn == b) return mi355_fail("residual_rmsnorm_fwd: yn must not alias y, a or b");
+    const bool vec_ok = (S % 4 == 0) && aligned16(y) && aligned16(yn) && aligned16(a) && aligned16(b);
+    const float invC = 1.0f / (float)C;
+#define RES_RMS(VEC, LPR, THR, CAP)                                                                              \
+    do {                                                                                                         \
+        const int strips = (int)ceil_div((size_t)S, (size_t)(LPR) * (VEC));                                      \
+        hipLaunchKernelGGL((res_rms_fwd_kernel<VEC, LPR, THR, CAP>), dim3(strips * batch), dim3(THR), 0,         \
+                           g_ctx.stream, y, yn, a, b, alpha, w, C, S, strips, strips * batch, eps, invC);        \
+    } while (0)
+    if (!vec_ok) RES_RMS(1, 64, 256, 0);
+    else if (C <= 128) RES_RMS(4, 16, 256, 8);
+    else if (C <= 512 && g_ctx.rms_threads != 1024) RES_RMS(4, 4, 256, 8);
+    else if (C <= 2048 && g_ctx.rms_threads != 256) RES_RMS(4, 4, 1024, 8);
+    else if (C <= 1024) RES_RMS(4, 4, 256, 16);
+    else RES_RMS(4, 8, 1024, 0);
+#undef RES_RMS
+    LAUNCH_OK("residual_rmsnorm_fwd");
+    return 0;
 }

@@ -43,8 +43,8 @@ __global__ __launch_bounds__(THREADS) void qknorm_rope_fwd_kernel(
         const int rp = p0 + kk * PPS;
         if (rp < half && col_ok) {
             const float *px = in + base + (size_t)(2 * rp) * S;
-            x0[kk] = ld4(px);
-            x1[kk] = ld4(px + S);
+            x0[kk] = ld4_nt(px);
+            x1[kk] = ld4_nt(px + S);
             cs[kk] = ld4(cos_t + (size_t)rp * S + col);
             sn[kk] = ld4(sin_t + (size_t)rp * S + col);
             w0[kk] = w[2 * rp];
@@ -73,8 +73,8 @@ __global__ __launch_bounds__(THREADS) void qknorm_rope_fwd_kernel(
             const v4f y0 = (x0[kk] * rr) * w0[kk];
             const v4f y1 = (x1[kk] * rr) * w1[kk];
             float *po = out + base + (size_t)(2 * rp) * S;
-            st4(po, y0 * cs[kk] - y1 * sn[kk]);
-            st4(po + S, y0 * sn[kk] + y1 * cs[kk]);
+            st4_nt(po, y0 * cs[kk] - y1 * sn[kk]);
+            st4_nt(po + S, y0 * sn[kk] + y1 * cs[kk]);
         }
     }
 }
@@ -110,9 +110,9 @@ __global__ __launch_bounds__(THREADS) void qknorm_rope_bwd_kernel(
         const int rp = p0 + kk * PPS;
         if (rp < half && col_ok) {
             const size_t o = base + (size_t)(2 * rp) * S;
-            x0[kk] = ld4(xin + o);
-            x1[kk] = ld4(xin + o + S);
-            const v4f g0 = ld4(gin + o), g1 = ld4(gin + o + S);
+            x0[kk] = ld4_nt(xin + o);
+            x1[kk] = ld4_nt(xin + o + S);
+            const v4f g0 = ld4_nt(gin + o), g1 = ld4_nt(gin + o + S);
             const v4f c = ld4(cos_t + (size_t)rp * S + col), s = ld4(sin_t + (size_t)rp * S + col);
             d0[kk] = g0 * c + g1 * s;        // inverse rotation (cpu_ops.h:179-180)
             d1[kk] = (-g0) * s + g1 * c;
@@ -154,8 +154,8 @@ __global__ __launch_bounds__(THREADS) void qknorm_rope_bwd_kernel(
             }
             if (col_ok) {
                 float *po = out + base + (size_t)(2 * rp) * S;
-                st4(po, o0);
-                st4(po + S, o1);
+                st4_nt(po, o0);
+                st4_nt(po + S, o1);
             }
             const v4f t0 = (d0[kk] * x0[kk]) * rr, t1 = (d1[kk] * x1[kk]) * rr;
             float s0 = ((t0[0] + t0[1]) + t0[2]) + t0[3];
@@ -181,7 +181,7 @@ bool pick_qk(int hd, QkCfg &cfg) {
     for (int lpr : lprs) {
         if (g_ctx.qk_lpr && g_ctx.qk_lpr != lpr) continue;
         const int pps = 256 / lpr;
-        const int caps[3] = {2, 4, 8};
+        const int caps[2] = {2, 4};   // 8 pairs per thread would spill
         for (int cap : caps)
             if (cap * pps >= half) { cfg = QkCfg{lpr, 256, cap}; return true; }
     }
@@ -194,13 +194,10 @@ bool pick_qk(int hd, QkCfg &cfg) {
         switch (key) {                                                                                        \
             case 1602: hipLaunchKernelGGL((KERNEL<16, 256, 2>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break; \
             case 1604: hipLaunchKernelGGL((KERNEL<16, 256, 4>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break; \
-            case 1608: hipLaunchKernelGGL((KERNEL<16, 256, 8>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break; \
             case 802: hipLaunchKernelGGL((KERNEL<8, 256, 2>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;   \
             case 804: hipLaunchKernelGGL((KERNEL<8, 256, 4>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;   \
-            case 808: hipLaunchKernelGGL((KERNEL<8, 256, 8>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;   \
             case 402: hipLaunchKernelGGL((KERNEL<4, 256, 2>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;   \
             case 404: hipLaunchKernelGGL((KERNEL<4, 256, 4>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;   \
-            case 408: hipLaunchKernelGGL((KERNEL<4, 256, 8>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;   \
             default: return mi355_fail("qknorm_rope: no kernel for tile key %d", key);                        \
         }                                                                                                     \
     } while (0)
@@ -266,7 +263,6 @@ MI355_API int mi355_qknorm_rope_bwd_dev(float *dq, float *dk, float *dwq, float 
     QK_DISPATCH(qknorm_rope_bwd_kernel, cfg, dim3(nq + nk), dq, dk, part, dq_out, dk_out, q, k, wq, wk, hd, S, strips,
                 nq, cos_dev, sin_dev, eps, 1.0f / (float)hd, variant);
     LAUNCH_OK("qknorm_rope_bwd");
-    if (nq > 0 && mi355_reduce_rows(dwq, part, nq, hd)) return -1;
-    if (nk > 0 && mi355_reduce_rows(dwk, part + (size_t)nq * hd, nk, hd)) return -1;
-    return 0;
+    if (nq > 0) return mi355_reduce_rows2(dwq, part, nq, dwk, part + (size_t)nq * hd, nk, hd);
+    return mi355_reduce_rows(dwk, part, nk, hd);
 }

@@ -34,6 +34,16 @@ __device__ __forceinline__ void ld_cols(float (&r)[VEC], const float *p) {
     }
 }
 
+template <int VEC>
+__device__ __forceinline__ void ld_cols_nt(float (&r)[VEC], const float *p) {
+    if constexpr (VEC == 4) {
+        v4f t = ld4_nt(p);
+        r[0] = t.x; r[1] = t.y; r[2] = t.z; r[3] = t.w;
+    } else {
+        r[0] = __builtin_nontemporal_load(p);
+    }
+}
+
 // grid: (row blocks, column strips of 64*VEC)
 template <int VEC>
 __global__ __launch_bounds__(CE_THREADS) void ce_partial_kernel(float *__restrict__ pm, float *__restrict__ pl,
@@ -70,7 +80,7 @@ __global__ __launch_bounds__(CE_THREADS) void ce_partial_kernel(float *__restric
             if (nm > -INFINITY) {
                 float s = 0.f;
 #pragma unroll
-                for (int k = 0; k < CE_CAP; k++) s += exp_neg(x[k][j] - nm);   // exp(-inf) = 0 for masked rows
+                for (int k = 0; k < CE_CAP; k++) s += exp_neg_fast(x[k][j] - nm);   // exp(-inf) = 0 for masked rows
                 l[j] = l[j] * exp_neg(m[j] - nm) + s;
                 m[j] = nm;
             }
@@ -110,12 +120,21 @@ __global__ __launch_bounds__(1024) void ce_combine_kernel(float *__restrict__ co
     const int t = blockIdx.x * 64 + cl;
     float m = -INFINITY, l = 0.f;
     if (t < S)
-        for (int r = g; r < nblk; r += 16) {
-            const float mr = pm[(size_t)r * S + t], lr = pl[(size_t)r * S + t];
-            const float nm = fmaxf(m, mr);
-            if (nm > -INFINITY) {
-                l = l * exp_neg(m - nm) + lr * exp_neg(mr - nm);
-                m = nm;
+        for (int r0 = g; r0 < nblk; r0 += 16 * 8) {
+            float mr[8], lr[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {     // eight independent loads in flight
+                const int r = r0 + 16 * u;
+                mr[u] = r < nblk ? pm[(size_t)r * S + t] : -INFINITY;
+                lr[u] = r < nblk ? pl[(size_t)r * S + t] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const float nm = fmaxf(m, mr[u]);
+                if (nm > -INFINITY) {
+                    l = l * exp_neg(m - nm) + lr[u] * exp_neg(mr[u] - nm);
+                    m = nm;
+                }
             }
         }
     sm[g][cl] = m;
@@ -185,7 +204,7 @@ __global__ __launch_bounds__(CE_THREADS) void ce_grad_kernel(float *dlogits, con
 #pragma unroll
         for (int k = 0; k < CE_CAP; k++) {
             const int v = base + k * CE_WAVES + wave;
-            if (v < v_hi) ld_cols<VEC>(x[k], logits + (size_t)v * S + col);
+            if (v < v_hi) ld_cols_nt<VEC>(x[k], logits + (size_t)v * S + col);
         }
 #pragma unroll
         for (int k = 0; k < CE_CAP; k++) {

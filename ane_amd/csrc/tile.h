@@ -11,6 +11,25 @@ __device__ __forceinline__ void ldv(float (&r)[VEC], const float *p) {
         r[0] = *p;
     }
 }
+// streaming variants: the operand is touched once by this kernel
+template <int VEC>
+__device__ __forceinline__ void ldv_nt(float (&r)[VEC], const float *p) {
+    if constexpr (VEC == 4) {
+        v4f t = ld4_nt(p);
+        r[0] = t.x; r[1] = t.y; r[2] = t.z; r[3] = t.w;
+    } else {
+        r[0] = __builtin_nontemporal_load(p);
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void stv_nt(float *p, const float (&r)[VEC]) {
+    if constexpr (VEC == 4) {
+        v4f t = {r[0], r[1], r[2], r[3]};
+        st4_nt(p, t);
+    } else {
+        __builtin_nontemporal_store(r[0], p);
+    }
+}
 template <int VEC>
 __device__ __forceinline__ void stv(float *p, const float (&r)[VEC]) {
     if constexpr (VEC == 4) {
@@ -56,3 +75,6 @@ __device__ __forceinline__ void strip_reduce(float (&acc)[NV][VEC], float *lds) 
 
 // out[c] += sum over rows of part[rows][C] in a fixed order (norm.hip)
 int mi355_reduce_rows(float *out, const float *part, int nrows, int C);
+// two such reductions in one launch (the second is skipped when out1 is NULL or nrows1 == 0)
+int mi355_reduce_rows2(float *out0, const float *part0, int nrows0, float *out1, const float *part1, int nrows1,
+                       int C);

@@ -4,8 +4,10 @@
 One "step" = one pass of the Qwen3-0.6B full-step fused-op sweep (BASELINE config 4) over one
 synthetic batch of 16 x 256 tokens, fp32, channel-first:
     forward, layers 0..27 : rmsnorm(att) -> qknorm+rope -> residual -> rmsnorm(ffn) -> swiglu -> residual
+                            (--fuse runs each residual and the RMSNorm that consumes its result as ONE launch,
+                             as they sit at training/training_dynamic/train.m:460-461)
     classifier            : softmax + cross-entropy fwd/bwd on logits [151936, 256]
-    backward, layers 27..0: swiglu_bwd -> rmsnorm_bwd(ffn) -> residual -> qknorm+rope bwd -> rmsnorm_bwd(att) -> residual
+    backward, layers 27..0: swiglu_bwd -> rmsnorm_bwd(ffn) -> qknorm+rope bwd -> rmsnorm_bwd(att)
     INT8                  : per-tensor scale, quantize, dequantize on [1024, 4096]
 Every layer has its own activation buffers (as a training step has), so each op reads data that
 was last touched a whole sweep ago.  Inputs are resident in HBM before the timed region.
@@ -45,6 +47,9 @@ def alg_bytes(cfg):
         "swiglu_fwd": 12 * H * St,
         "swiglu_bwd": 20 * H * St,
         "residual": 12 * C * St,
+        "scale_copy": 8 * H * St,        # y = alpha*a over an [H,St] tensor: a plain copy-shaped stream (train.m:523,595)
+        # residual + the RMSNorm after it in one launch; as two ops the same work is 12CSt + 8CSt + 4C
+        "residual_rmsnorm_fwd": 16 * C * St + 4 * C,
         "softmax_ce": 8 * V * S,
         "int8_scale": 4 * n8,
         "int8_quant": 5 * n8,
@@ -53,8 +58,8 @@ def alg_bytes(cfg):
 
 
 class Workload:
-    def __init__(self, br, cfg, layers):
-        self.br, self.cfg, self.L = br, cfg, layers
+    def __init__(self, br, cfg, layers, fuse=False):
+        self.br, self.cfg, self.L, self.fuse = br, cfg, layers, fuse
         C, H, S, B = cfg["C"], cfg["H"], cfg["S"], cfg["batch"]
         qd, kd = cfg["heads"] * cfg["hd"], cfg["kv_heads"] * cfg["hd"]
         A = br.DevArray
@@ -74,6 +79,7 @@ class Workload:
                 wk=rnd(cfg["hd"], std=0.02, mean=1.0), q_rot=A((B, qd, S)), k_rot=A((B, kd, S)),
                 o=rnd(B, C, S), x2=A((B, C, S)), w_ffn=rnd(C, std=0.02, mean=1.0), x2n=A((B, C, S)),
                 h1=rnd(B, H, S), h3=rnd(B, H, S), gate=A((B, H, S)), f=rnd(B, C, S), x_next=A((B, C, S)),
+                xn_next=A((B, C, S)),
                 # backward
                 dsilu=rnd(B, H, S), dh1=A((B, H, S)), dh3=A((B, H, S)),
                 dx_ffn=rnd(B, C, S), dx2=A((B, C, S)), dw_ffn=A(C), dy=rnd(B, C, S),
@@ -110,6 +116,14 @@ class Workload:
                                              d["wk"].ptr, c["heads"], c["kv_heads"], hd, S, B, self.cos, self.sin, 1e-5))
         elif name == "residual1":
             ck(lib.mi355_axpby_dev(d["x2"].ptr, d["x"].ptr, d["o"].ptr, self.alpha, n_c, 0))
+        elif name == "res_rms1":       # x2 = x + alpha*o ; x2n = rmsnorm(x2)   (train.m:460-461)
+            ck(lib.mi355_residual_rmsnorm_fwd_dev(d["x2"].ptr, d["x2n"].ptr, d["x"].ptr, d["o"].ptr, self.alpha,
+                                                  d["w_ffn"].ptr, C, S, B, 1e-5))
+        elif name == "res_rms2":       # x_next = x2 + alpha*f ; next layer's (or the final) rmsnorm of it
+            ck(lib.mi355_residual_rmsnorm_fwd_dev(d["x_next"].ptr, d["xn_next"].ptr, d["x2"].ptr, d["f"].ptr,
+                                                  self.alpha, d["w_att"].ptr, C, S, B, 1e-5))
+        elif name == "scale_copy":     # dffn = alpha*dy shaped stream over the SwiGLU-sized buffers
+            ck(lib.mi355_axpby_dev(d["dh1"].ptr, d["dsilu"].ptr, None, self.alpha, n_h, 1))
         elif name == "swiglu_fwd":
             ck(lib.mi355_swiglu_fwd_dev(d["gate"].ptr, d["h1"].ptr, d["h3"].ptr, n_h))
         elif name == "residual2":
@@ -133,8 +147,13 @@ class Workload:
         else:
             raise KeyError(name)
 
-    FWD = ["rmsnorm_fwd", "qknorm_rope_fwd", "residual1", "rmsnorm_fwd2", "swiglu_fwd", "residual2"]
-    BWD = ["swiglu_bwd", "rmsnorm_bwd2", "residual3", "qknorm_rope_bwd", "rmsnorm_bwd", "residual4"]
+    # 2 RMSNorm fwd + 2 residual + QK-norm/RoPE + SwiGLU per layer, forward; their backward (no residual adds:
+    # the named workload has two residuals per layer)
+    FWD_UNFUSED = ["rmsnorm_fwd", "qknorm_rope_fwd", "residual1", "rmsnorm_fwd2", "swiglu_fwd", "residual2"]
+    # fused: layer 0's first norm stands alone (its input comes from the embedding); every other norm is
+    # produced by the residual before it, the last one being the final norm (train.m:487)
+    FWD_FUSED = ["qknorm_rope_fwd", "res_rms1", "swiglu_fwd", "res_rms2"]
+    BWD = ["swiglu_bwd", "rmsnorm_bwd2", "qknorm_rope_bwd", "rmsnorm_bwd"]
 
     def ce(self):
         self.br.check(self.br.lib.mi355_softmax_ce_dev(self.dlogits.ptr, self.loss.ptr, self.logits.ptr,
@@ -150,8 +169,10 @@ class Workload:
             self.br.check(lib.mi355_int8_dequant_dev(self.y8.ptr, self.q8.ptr, self.scale8.ptr, n))
 
     def step(self):
+        if self.fuse:
+            self.op("rmsnorm_fwd", self.lay[0])
         for d in self.lay:
-            for name in self.FWD:
+            for name in (self.FWD_FUSED if self.fuse else self.FWD_UNFUSED):
                 self.op(name, d)
         self.ce()
         for d in reversed(self.lay):
@@ -175,7 +196,7 @@ def per_op_table(br, wl, reps):
     ab = alg_bytes(wl.cfg)
     names = {"rmsnorm_fwd": "rmsnorm_fwd", "rmsnorm_bwd": "rmsnorm_bwd", "qknorm_rope_fwd": "qknorm_rope_fwd",
              "qknorm_rope_bwd": "qknorm_rope_bwd", "swiglu_fwd": "swiglu_fwd", "swiglu_bwd": "swiglu_bwd",
-             "residual1": "residual"}
+             "residual1": "residual", "res_rms1": "residual_rmsnorm_fwd", "scale_copy": "scale_copy"}
     table = []
     for opname, key in names.items():
         def run():
@@ -213,13 +234,13 @@ def cpu_baseline(br, wl, sample_layers, threads_mt):
         out["x2n"] = O.rmsnorm(out["x2"], h["w_ffn"], threads=threads)
         out["gate"] = O.swiglu_fwd(h["h1"], h["h3"], threads=threads)
         out["x_next"] = O.axpby(out["x2"], h["f"], wl.alpha, 0, threads=threads)
+        if wl.fuse:
+            out["xn_next"] = O.rmsnorm(out["x_next"], h["w_att"], threads=threads)
         out["dh1"], out["dh3"] = O.swiglu_bwd(h["dsilu"], h["h1"], h["h3"], threads=threads)
         out["dx2"], out["dw_ffn"] = O.rmsnorm_bwd(h["dx_ffn"], out["x2"], h["w_ffn"], threads=threads)
-        out["dx2"] = O.axpby(out["dx2"], h["dy"], 0.0, 2, threads=threads)
         out["dq"], out["dwq"] = O.qknorm_rope_bwd(h["gq"], h["q"], h["wq"], hd, c["theta"], threads=threads)
         out["dk"], out["dwk"] = O.qknorm_rope_bwd(h["gk"], h["k"], h["wk"], hd, c["theta"], threads=threads)
         out["dx1"], out["dw_att"] = O.rmsnorm_bwd(h["dx_attn"], h["x"], h["w_att"], threads=threads)
-        out["dy_out"] = O.axpby(out["dx1"], out["dx2"], 0.0, 2, threads=threads)
         return now() - t0, out
 
     def rel(a, ref):
@@ -234,8 +255,7 @@ def cpu_baseline(br, wl, sample_layers, threads_mt):
         t_layer.append(t)
         if i == 0:
             # dw buffers accumulate over steps on the GPU; compare the assigned tensors only
-            for k in ("xn", "q_rot", "k_rot", "x2", "x2n", "gate", "x_next", "dh1", "dh3", "dx2", "dq", "dk", "dx1",
-                      "dy_out"):
+            for k in ("xn", "q_rot", "k_rot", "x2", "x2n", "gate", "x_next", "dh1", "dh3", "dx2", "dq", "dk", "dx1"):
                 parity = max(parity, rel(wl.lay[0][k].numpy(), out[k]))
     logits = wl.logits.numpy(); tg = wl.targets.numpy()
     t0 = now(); loss, dl = O.cross_entropy(logits, tg); t_ce = now() - t0
@@ -247,7 +267,7 @@ def cpu_baseline(br, wl, sample_layers, threads_mt):
     t1 = float(np.mean(t_layer)) * L + t_ce + t_i8
     tokens = B * S
     res = dict(value=tokens / t1, unit="tokens/s", cores=1, kind="port",
-               sample="%d of %d layers (all 12 layer ops, batch %dx%d) + full softmax-CE [%d,%d] + full INT8 %s; "
+               sample="%d of %d layers (all 10 layer ops, batch %dx%d) + full softmax-CE [%d,%d] + full INT8 %s; "
                       "layer time scaled x%d; %.1f s of CPU work" % (sample_layers, L, B, S, c["V"], S,
                                                                      list(c["int8_shape"]), L,
                                                                      sum(t_layer) + t_ce + t_i8),
@@ -264,7 +284,9 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=Q3["layers"], help="layers in the sweep (28 = the named workload)")
-    ap.add_argument("--cpu-layers", type=int, default=2, help="layers in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--cpu-layers", type=int, default=28, help="layers in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--fuse", action="store_true",
+                    help="run each residual and the RMSNorm after it as one launch (mi355_residual_rmsnorm_fwd_dev)")
     ap.add_argument("--op-reps", type=int, default=3)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -274,7 +296,7 @@ def main():
     br.init()
     dev_name, drv_peak, cus = br.device_info()
     cfg = dict(Q3)
-    wl = Workload(br, cfg, args.layers)
+    wl = Workload(br, cfg, args.layers, fuse=args.fuse)
 
     for _ in range(args.warmup):
         wl.step()
@@ -285,9 +307,12 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
     ab = alg_bytes(cfg)
+    # algorithmic bytes of the work done, op by op as the unfused definitions count it
     per_layer = (2 * ab["rmsnorm_fwd"] + 2 * ab["rmsnorm_bwd"] + ab["qknorm_rope_fwd"] + ab["qknorm_rope_bwd"] +
-                 ab["swiglu_fwd"] + ab["swiglu_bwd"] + 4 * ab["residual"])
+                 ab["swiglu_fwd"] + ab["swiglu_bwd"] + 2 * ab["residual"])
     total_bytes = args.layers * per_layer + ab["softmax_ce"] + ab["int8_scale"] + ab["int8_quant"] + ab["int8_dequant"]
+    if wl.fuse:
+        total_bytes += ab["rmsnorm_fwd"]      # 2L+1 norms: layer 0's own plus one per residual
     tokens = cfg["batch"] * cfg["S"]
 
     table = per_op_table(br, wl, args.op_reps)
@@ -302,10 +327,11 @@ def main():
         "value": tokens / (ms / 1e3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "qwen3-0.6b full-step fused-op sweep (BASELINE config 4): %d layers x 12 fused ops "
+        "config": {"workload": "qwen3-0.6b full-step fused-op sweep (BASELINE config 4): %d layers x 10 ops "
                                "(batch 16 x S 256, C 1024, H 3072, 16/8 heads x 128) + softmax-CE [151936,256] + "
                                "INT8 [1024,4096]" % args.layers,
-                   "layers": args.layers, "tokens_per_step": tokens, "alg_gb_per_step": total_bytes / 1e9},
+                   "layers": args.layers, "tokens_per_step": tokens, "alg_gb_per_step": total_bytes / 1e9,
+                   "residual_fused_into_next_rmsnorm": wl.fuse},
         "aggregate_gbs": total_bytes / ms / 1e6, "aggregate_frac_of_peak": total_bytes / ms / 1e6 / PEAK_HBM_GBS,
         "host_wall_ms_per_step": wall_ms,
         "device": dev_name, "compute_units": cus, "driver_reported_peak_gbs": drv_peak,

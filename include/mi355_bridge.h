@@ -100,6 +100,13 @@ int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, int C, int S
 int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const float *x, const float *w,
                           int C, int S, int batch, float eps, int variant);
 
+/* Residual add fused with the RMSNorm that follows it in the loops: vDSP_vsma + rmsnorm at
+ * training/training_dynamic/train.m:460-461 (and a layer's x_next feeding the next rmsnorm at :417).
+ * y = a + alpha*b (as mode 0 of mi355_axpby_dev); yn = rmsnorm(y, w).  One launch instead of two; the
+ * results are bit-identical to the two separate calls.  y may alias a or b; yn must not alias anything. */
+int mi355_residual_rmsnorm_fwd_dev(float *y, float *yn, const float *a, const float *b, float alpha,
+                                   const float *w, int C, int S, int batch, float eps);
+
 /* SwiGLU gate forward: out = (h1*sigmoid(h1))*h3.  Replaces the MIL sigmoid/mul/mul of
  * training/training_dynamic/mil_dynamic.h:264-266 and training/forward.h:101,149-151. */
 int mi355_swiglu_fwd_dev(float *out, const float *h1, const float *h3, size_t n);

@@ -111,6 +111,27 @@ def test_rmsnorm_unaligned_pointers_and_every_tile(br):
         br.tune("rms_lpr", 0); br.tune("rms_threads", 0)
 
 
+@pytest.mark.parametrize("B,Cc,S", [(16, 1024, 256), (1, 768, 256), (2, 100, 37), (3, 48, 20), (2, 300, 64)])
+def test_residual_rmsnorm_fused_equals_two_calls(br, B, Cc, S):
+    say("residual_rmsnorm B=%d C=%d S=%d" % (B, Cc, S))
+    a = H.normal(7, (B, Cc, S)); b = H.normal(8, (B, Cc, S)); w = H.normal(9, Cc, 1.0, 0.02)
+    alpha = np.float32(1 / np.sqrt(2 * 28))                     # training/training_dynamic/train.m:188
+    ad, bd, wd = dev(br, a), dev(br, b), dev(br, w)
+    y = br.DevArray(a.shape); yn = br.DevArray(a.shape)
+    br.check(br.lib.mi355_residual_rmsnorm_fwd_dev(y.ptr, yn.ptr, ad.ptr, bd.ptr, alpha, wd.ptr, Cc, S, B, 1e-5))
+    ry = O.axpby(a, b, alpha, 0)
+    assert np.array_equal(y.numpy(), ry)                        # the residual is exact fp32 arithmetic
+    assert H.rel_err(yn.numpy(), O.rmsnorm(ry, w)) <= TOL
+    y2 = br.DevArray(a.shape); yn2 = br.DevArray(a.shape)
+    br.check(br.lib.mi355_axpby_dev(y2.ptr, ad.ptr, bd.ptr, alpha, a.size, 0))
+    br.check(br.lib.mi355_rmsnorm_fwd_dev(yn2.ptr, y2.ptr, wd.ptr, Cc, S, B, 1e-5))
+    assert H.rel_err(yn.numpy(), yn2.numpy()) <= 2e-6           # same math, different summation tree
+    # in place on a (x_cur updated to x2)
+    br.check(br.lib.mi355_residual_rmsnorm_fwd_dev(ad.ptr, yn2.ptr, ad.ptr, bd.ptr, alpha, wd.ptr, Cc, S, B, 1e-5))
+    assert np.array_equal(ad.numpy(), ry) and np.array_equal(yn2.numpy(), yn.numpy())
+    assert br.lib.mi355_residual_rmsnorm_fwd_dev(y.ptr, y.ptr, ad.ptr, bd.ptr, alpha, wd.ptr, Cc, S, B, 1e-5) == -1
+
+
 # ---------------------------------------------------------------------------------------------
 # SwiGLU
 # ---------------------------------------------------------------------------------------------
