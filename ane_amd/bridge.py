@@ -74,6 +74,9 @@ SIGNATURES = {
     "mi355_host_table_invalidate": (None, [_p]),
     "mi355_embed_backward": (None, [_p, _p, _p, _i, _i, _i]),
     "mi355_rope_backward_inplace": (None, [_p, _i, _i, _i]),
+    "mi355_swiglu_bwd": (None, [_p, _p, _p, _p, _p, _z]),
+    "mi355_swiglu_fwd": (None, [_p, _p, _p, _z]),
+    "mi355_axpby": (None, [_p, _p, _p, _f, _z, _i]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():

@@ -51,5 +51,22 @@ def build(verbose=False, jobs=7):
     return LIB
 
 
+HOST_SRC = os.path.join(HERE, "host", "train_step_mirror.c")
+HOST_BIN = os.path.join(HERE, "host", "train_step_mirror")
+
+
+def build_host_mirror():
+    """Compile the C mirror of the reference's training-step op sequence against the library (gcc)."""
+    inc = os.path.join(os.path.dirname(HERE), "include")
+    cmd = ["gcc", "-O2", "-std=c99", "-ffp-contract=off", "-Wall", "-I", inc, HOST_SRC, "-L", HERE, "-lmi355_ops",
+           "-Wl,-rpath,$ORIGIN/..", "-lm", "-o", HOST_BIN]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        sys.stderr.write(r.stdout + r.stderr)
+        raise RuntimeError("gcc failed on train_step_mirror.c")
+    return HOST_BIN
+
+
 if __name__ == "__main__":
     print(build(verbose="-v" in sys.argv))
+    print(build_host_mirror())

@@ -207,3 +207,43 @@ MI355_API void mi355_rope_backward_inplace(float *dx, int seq, int dim, int hd) 
     if (mi355_rope_dev(x_d, nullptr, x_d, nullptr, dim / hd, 0, hd, seq, 1, c_d, s_d, -1)) return;
     d2h(dx, x_d, nb);
 }
+
+// SiLU-gate backward as one call: the 13 vDSP/vForce calls of training/training_dynamic/train.m:537-554.
+MI355_API void mi355_swiglu_bwd(float *dh1, float *dh3, const float *dsilu, const float *h1, const float *h3, size_t n) {
+    if (!mi355_ready("swiglu_bwd")) return;
+    if (!dh1 || !dh3 || !dsilu || !h1 || !h3 || n == 0) { mi355_fail("swiglu_bwd: bad arguments"); return; }
+    const size_t nb = n * sizeof(float);
+    float *d = (float *)slot(0, nb), *a = (float *)slot(1, nb), *b = (float *)slot(2, nb);
+    float *o1 = (float *)slot(3, nb), *o3 = (float *)slot(4, nb);
+    if (!d || !a || !b || !o1 || !o3) return;
+    if (!h2d(d, dsilu, nb) || !h2d(a, h1, nb) || !h2d(b, h3, nb)) return;
+    if (mi355_swiglu_bwd_dev(o1, o3, d, a, b, n)) return;
+    if (!d2h(dh1, o1, nb)) return;
+    d2h(dh3, o3, nb);
+}
+
+// SiLU-gate forward: out = (h1*sigmoid(h1))*h3 (training/forward.h:101,149-151).
+MI355_API void mi355_swiglu_fwd(float *out, const float *h1, const float *h3, size_t n) {
+    if (!mi355_ready("swiglu_fwd")) return;
+    if (!out || !h1 || !h3 || n == 0) { mi355_fail("swiglu_fwd: bad arguments"); return; }
+    const size_t nb = n * sizeof(float);
+    float *a = (float *)slot(0, nb), *b = (float *)slot(1, nb), *o = (float *)slot(2, nb);
+    if (!a || !b || !o) return;
+    if (!h2d(a, h1, nb) || !h2d(b, h3, nb)) return;
+    if (mi355_swiglu_fwd_dev(o, a, b, n)) return;
+    d2h(out, o, nb);
+}
+
+// Residual family on host pointers: vDSP_vsma / vDSP_vsmul / vDSP_vadd
+// (training/training_dynamic/train.m:460,523,595; training/train_large.m:427,442).
+MI355_API void mi355_axpby(float *y, const float *a, const float *b, float alpha, size_t n, int mode) {
+    if (!mi355_ready("axpby")) return;
+    if (!y || !a || (mode != 1 && !b) || n == 0 || mode < 0 || mode > 2) { mi355_fail("axpby: bad arguments"); return; }
+    const size_t nb = n * sizeof(float);
+    float *ad = (float *)slot(0, nb), *bd = (float *)slot(1, nb), *yd = (float *)slot(2, nb);
+    if (!ad || !bd || !yd) return;
+    if (!h2d(ad, a, nb)) return;
+    if (mode != 1 && !h2d(bd, b, nb)) return;
+    if (mi355_axpby_dev(yd, ad, mode != 1 ? bd : nullptr, alpha, n, mode)) return;
+    d2h(y, yd, nb);
+}

@@ -207,6 +207,13 @@ void mi355_embed_backward(float *d_embed, const float *dx, const uint16_t *token
                           int dim, int seq);
 /* rope_backward_inplace — training/training_dynamic/cpu_ops.h:168 (theta = 10000) */
 void mi355_rope_backward_inplace(float *dx, int seq, int dim, int hd);
+/* The inline vDSP blocks of the dynamic loop as calls: SiLU-gate backward
+ * (training/training_dynamic/train.m:537-554), its forward (training/forward.h:101,149-151), and the
+ * residual family vDSP_vsma / vDSP_vsmul / vDSP_vadd (train.m:460,523,595; modes as mi355_axpby_dev). */
+void mi355_swiglu_bwd(float *dh1, float *dh3, const float *dsilu, const float *h1, const float *h3,
+                      size_t n);
+void mi355_swiglu_fwd(float *out, const float *h1, const float *h3, size_t n);
+void mi355_axpby(float *y, const float *a, const float *b, float alpha, size_t n, int mode);
 
 #ifdef __cplusplus
 }
