@@ -13,6 +13,16 @@
  * order of a reduction unpublished (vDSP_sve, vDSP_maxv) an 8-lane strided accumulation is used,
  * which is what a vectorised loop does; the parity tests arbitrate with float64 closed forms.
  *
+ * Pinning (tests/test_oracle.py): every function here is checked against the committed golden
+ * vectors (inputs from the reference's own test recipes), float64 closed forms, finite differences,
+ * invariants and hand-computed cases.  Parity unpinned by anything the reference holds:
+ *   - orc_int8_quant with rounding 0 (ties to even): the reference's only C quantizer rounds half
+ *     away from zero (rounding 1); ties-to-even is pinned by a hand-computed tie table only;
+ *   - orc_qknorm_rope_*: the op does not exist in the reference; it is pinned as the composition
+ *     of orc_rmsnorm(_bwd) and orc_rope_*;
+ *   - bit-level behaviour of vvrsqrtf / vvexpf / vDSP_sve (closed source): parity is held at the
+ *     1e-5 tolerance of the path, not bit for bit.
+ *
  * All citations are relative to the reference tree.
  *
  * Layout: channel-first x[c*S + s] (training/stories_cpu_ops.h:110-118).
