@@ -52,6 +52,8 @@ SIGNATURES = {
     "mi355_fill_randint_dev": (_i, [_p, _z, C.c_uint64, C.c_int32, C.c_int32]),
     "mi355_rmsnorm_fwd_dev": (_i, [_p, _p, _p, _i, _i, _i, _f]),
     "mi355_rmsnorm_bwd_dev": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _f, _i]),
+    "mi355_dw_defer": (_i, [_i]),
+    "mi355_dw_flush": (_i, []),
     "mi355_residual_rmsnorm_fwd_dev": (_i, [_p, _p, _p, _p, _f, _p, _i, _i, _i, _f]),
     "mi355_swiglu_fwd_dev": (_i, [_p, _p, _p, _z]),
     "mi355_swiglu_bwd_dev": (_i, [_p, _p, _p, _p, _p, _z]),

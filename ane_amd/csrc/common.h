@@ -35,6 +35,8 @@ int mi355_fail(const char *fmt, ...);
 bool mi355_ready(const char *who);
 // Workspace of at least `bytes` (256-byte aligned), NULL on failure.
 void *mi355_ws(size_t bytes);
+// Runs every queued weight-gradient reduction (dw_reduce.hip).
+extern "C" int mi355_dw_flush(void);
 
 #define HIP_OK(expr)                                                                          \
     do {                                                                                      \

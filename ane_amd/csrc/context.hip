@@ -69,11 +69,13 @@ MI355_API int mi355_init(void) {
 }
 
 void mi355_free_caches(void);   // rope tables, host drop-in staging (other translation units)
+void mi355_dw_free(void);       // queued weight-gradient reductions and their arena
 
 MI355_API void mi355_shutdown(void) {
     if (!g_ctx.ready) return;
     (void)hipDeviceSynchronize();
     mi355_free_caches();
+    mi355_dw_free();
     if (g_ctx.ws) (void)hipFree(g_ctx.ws);
     g_ctx = Mi355Ctx{};
 }
@@ -97,12 +99,14 @@ MI355_API int mi355_device_info(char *name, size_t name_len, double *peak_hbm_gb
 
 MI355_API int mi355_set_stream(void *hip_stream) {
     if (!mi355_ready("set_stream")) return -1;
+    if (mi355_dw_flush()) return -1;        // queued reductions belong to the old stream
     g_ctx.stream = (hipStream_t)hip_stream;
     return 0;
 }
 
 MI355_API int mi355_sync(void) {
     if (!mi355_ready("sync")) return -1;
+    if (mi355_dw_flush()) return -1;
     HIP_OK(hipStreamSynchronize(g_ctx.stream));
     return 0;
 }
@@ -169,6 +173,7 @@ MI355_API void mi355_buf_write(mi355_buf *b, size_t offset, const void *src, siz
 
 MI355_API void mi355_buf_read(mi355_buf *b, size_t offset, void *dst, size_t bytes) {
     if (!b || !dst || !g_ctx.ready || offset > b->bytes || bytes > b->bytes - offset || bytes == 0) return;
+    (void)mi355_dw_flush();                 // a read may be of a gradient that is still queued
     hipError_t e = hipMemcpyAsync(dst, (const char *)b->dev + offset, bytes, hipMemcpyDeviceToHost, g_ctx.stream);
     if (e == hipSuccess) e = hipStreamSynchronize(g_ctx.stream);
     if (e != hipSuccess) mi355_fail("buf_read: %s", hipGetErrorString(e));

@@ -428,7 +428,7 @@ struct RopeCache {
     float theta;
     float *cos_d, *sin_d;
 };
-static RopeCache g_rope[8];
+static RopeCache g_rope[64];
 static int g_rope_n = 0;
 
 void mi355_free_rope_cache(void) {
@@ -445,7 +445,7 @@ MI355_API int mi355_rope_tables_dev(const float **cos_dev, const float **sin_dev
             *sin_dev = g_rope[i].sin_d;
             return 0;
         }
-    if (g_rope_n == 8) return mi355_fail("rope_tables_dev: table cache full (8 distinct (S,hd,theta))");
+    if (g_rope_n == 64) return mi355_fail("rope_tables_dev: table cache full (64 distinct (S,hd,theta))");
     if (S <= 0 || hd <= 0 || (hd & 1) || !(theta > 0.f)) return mi355_fail("rope_tables_dev: bad S/hd/theta");
     const size_t n = (size_t)(hd / 2) * S;
     float *host = (float *)malloc(2 * n * sizeof(float));

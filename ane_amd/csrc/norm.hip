@@ -74,6 +74,7 @@ __global__ __launch_bounds__(THREADS) void rms_fwd_kernel(float *__restrict__ y,
         }
     } else {
         if (col_ok)
+#pragma unroll 4
             for (int c = row0; c < C; c += RPS) {
                 float t[VEC];
                 ldv<VEC>(t, xs + (size_t)c * S);
@@ -85,6 +86,7 @@ __global__ __launch_bounds__(THREADS) void rms_fwd_kernel(float *__restrict__ y,
 #pragma unroll
         for (int j = 0; j < VEC; j++) rr[j] = 1.0f / sqrtf(acc[0][j] * invC + eps);
         if (col_ok)
+#pragma unroll 4
             for (int c = row0; c < C; c += RPS) {
                 float t[VEC], o[VEC];
                 ldv_nt<VEC>(t, xs + (size_t)c * S);
@@ -173,6 +175,7 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
         }
     } else {
         if (col_ok)
+#pragma unroll 4
             for (int c = row0; c < C; c += RPS) {
                 float a[VEC], b[VEC];
                 ldv<VEC>(a, xs + (size_t)c * S);
@@ -187,6 +190,7 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
         strip_reduce<VEC, LPR, THREADS, 2>(acc, lds);
         float rr[VEC], dotn[VEC];
         finish(rr, dotn);
+#pragma unroll 4
         for (int c = row0; c < C; c += RPS) {
             float a[VEC], b[VEC];
             if (col_ok) {
@@ -265,6 +269,7 @@ __global__ __launch_bounds__(THREADS) void res_rms_fwd_kernel(float *y, float *_
     } else {
         // y is stored in the first sweep and read back by the same lane in the second
         if (col_ok)
+#pragma unroll 4
             for (int c = row0; c < C; c += RPS) {
                 float av[VEC], bv[VEC], t[VEC];
                 ldv_nt<VEC>(av, a + base + (size_t)c * S);
@@ -281,6 +286,7 @@ __global__ __launch_bounds__(THREADS) void res_rms_fwd_kernel(float *y, float *_
 #pragma unroll
         for (int j = 0; j < VEC; j++) rr[j] = 1.0f / sqrtf(acc[0][j] * invC + eps);
         if (col_ok)
+#pragma unroll 4
             for (int c = row0; c < C; c += RPS) {
                 float t[VEC], o[VEC];
                 ldv<VEC>(t, y + base + (size_t)c * S);
@@ -289,44 +295,6 @@ __global__ __launch_bounds__(THREADS) void res_rms_fwd_kernel(float *y, float *_
                 for (int j = 0; j < VEC; j++) o[j] = (t[j] * rr[j]) * wc;
                 stv_nt<VEC>(yn + base + (size_t)c * S, o);
             }
-    }
-}
-
-// out[c] += sum_r part[r][c], rows taken in a fixed order: 32 interleaved row groups, each
-// summed with four independent accumulators (so four loads are in flight), then combined in a
-// fixed order.  One workgroup handles 32 channels; blockIdx.y selects one of two jobs so that
-// two reductions (dwq and dwk) share a launch.
-struct ReduceJob {
-    float *out;
-    const float *part;
-    int nrows;
-};
-
-__global__ __launch_bounds__(1024) void reduce_rows_kernel(ReduceJob j0, ReduceJob j1, int C) {
-    __shared__ float lds[32][33];
-    const ReduceJob job = blockIdx.y == 0 ? j0 : j1;
-    const int cl = threadIdx.x & 31, g = threadIdx.x >> 5;
-    const int c = blockIdx.x * 32 + cl;
-    const float *__restrict__ part = job.part;
-    const int nrows = job.nrows;
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-    if (c < C) {
-        int r = g;
-        for (; r + 96 < nrows; r += 128) {
-            s0 += part[(size_t)r * C + c];
-            s1 += part[(size_t)(r + 32) * C + c];
-            s2 += part[(size_t)(r + 64) * C + c];
-            s3 += part[(size_t)(r + 96) * C + c];
-        }
-        for (; r < nrows; r += 32) s0 += part[(size_t)r * C + c];
-    }
-    lds[g][cl] = (s0 + s1) + (s2 + s3);
-    __syncthreads();
-    if (g == 0 && c < C) {
-        float t = 0.f;
-#pragma unroll
-        for (int k = 0; k < 32; k++) t += lds[k][cl];
-        job.out[c] = job.out[c] + t;
     }
 }
 
@@ -418,19 +386,6 @@ void launch_bwd(float *dx, float *part, const float *dy, const float *x, const f
 
 }   // namespace
 
-int mi355_reduce_rows2(float *out0, const float *part0, int nrows0, float *out1, const float *part1, int nrows1,
-                       int C) {
-    const int jobs = (out1 && nrows1 > 0) ? 2 : 1;
-    hipLaunchKernelGGL(reduce_rows_kernel, dim3((unsigned)ceil_div((size_t)C, 32), jobs), dim3(1024), 0, g_ctx.stream,
-                       ReduceJob{out0, part0, nrows0}, ReduceJob{out1, part1, nrows1}, C);
-    LAUNCH_OK("reduce_rows");
-    return 0;
-}
-
-int mi355_reduce_rows(float *out, const float *part, int nrows, int C) {
-    return mi355_reduce_rows2(out, part, nrows, nullptr, nullptr, 0, C);
-}
-
 MI355_API int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, int C, int S, int batch, float eps) {
     if (!mi355_ready("rmsnorm_fwd")) return -1;
     if (!y || !x || !w) return mi355_fail("rmsnorm_fwd: NULL pointer");
@@ -452,11 +407,12 @@ MI355_API int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const
     NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 16, 0, g_ctx.rms_lpr, g_ctx.rms_threads, true);
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
-    float *part = (float *)mi355_ws((size_t)nblk * C * sizeof(float));
+    float *part = mi355_dw_partials((size_t)nblk * C, dw, nullptr);
     if (!part) return -1;
     NORM_DISPATCH(launch_bwd, cfg, dx, part, dy, x, w, C, S, batch, eps, variant);
     LAUNCH_OK("rmsnorm_bwd");
-    return mi355_reduce_rows(dw, part, nblk, C);
+    if (mi355_dw_submit(dw, part, nblk, C)) return -1;
+    return mi355_dw_op_end();
 }
 
 MI355_API int mi355_residual_rmsnorm_fwd_dev(float *y, float *yn, const float *a, const float *b, float alpha,

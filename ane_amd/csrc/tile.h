@@ -73,8 +73,12 @@ __device__ __forceinline__ void strip_reduce(float (&acc)[NV][VEC], float *lds) 
 }
 
 
-// out[c] += sum over rows of part[rows][C] in a fixed order (norm.hip)
-int mi355_reduce_rows(float *out, const float *part, int nrows, int C);
-// two such reductions in one launch (the second is skipped when out1 is NULL or nrows1 == 0)
-int mi355_reduce_rows2(float *out0, const float *part0, int nrows0, float *out1, const float *part1, int nrows1,
-                       int C);
+// ---- weight-gradient reductions (dw_reduce.hip) -------------------------------------------------
+// A backward op writes per-workgroup partial rows part[nrows][C] and submits "out[c] += sum_r part[r][c]".
+// Immediately (default) the jobs of one op go out as one launch when the op ends; in deferred mode they
+// are queued and reduced together by mi355_dw_flush().
+//
+// Buffer for `floats` partials of the op that will accumulate into out0 / out1 (either may be NULL).
+float *mi355_dw_partials(size_t floats, const float *out0, const float *out1);
+int mi355_dw_submit(float *out, const float *part, int nrows, int C);
+int mi355_dw_op_end(void);

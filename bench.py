@@ -178,6 +178,9 @@ class Workload:
         for d in reversed(self.lay):
             for name in self.BWD:
                 self.op(name, d)
+        # the weight-gradient reductions queued by the backward ops (mi355_dw_defer) run here, where the
+        # optimizer would read them (training/training_dynamic/train.m:748)
+        self.br.check(self.br.lib.mi355_dw_flush())
         self.int8()
 
 
@@ -202,6 +205,7 @@ def per_op_table(br, wl, reps):
         def run():
             for d in wl.lay:
                 wl.op(opname, d)
+            br.check(br.lib.mi355_dw_flush())
         run()
         ms = time_region(br, run, reps) / len(wl.lay)
         table.append(dict(op=key, ms=ms, alg_mb=ab[key] / 1e6, gbs=ab[key] / ms / 1e6, frac=ab[key] / ms / 1e6 / PEAK_HBM_GBS))
@@ -285,6 +289,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=Q3["layers"], help="layers in the sweep (28 = the named workload)")
     ap.add_argument("--cpu-layers", type=int, default=28, help="layers in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--immediate-dw", action="store_true",
+                    help="reduce weight-gradient partials behind every backward op instead of once per step")
     ap.add_argument("--fuse", action="store_true",
                     help="run each residual and the RMSNorm after it as one launch (mi355_residual_rmsnorm_fwd_dev)")
     ap.add_argument("--op-reps", type=int, default=3)
@@ -297,6 +303,7 @@ def main():
     dev_name, drv_peak, cus = br.device_info()
     cfg = dict(Q3)
     wl = Workload(br, cfg, args.layers, fuse=args.fuse)
+    br.check(br.lib.mi355_dw_defer(0 if args.immediate_dw else 1))
 
     for _ in range(args.warmup):
         wl.step()
@@ -331,7 +338,8 @@ def main():
                                "(batch 16 x S 256, C 1024, H 3072, 16/8 heads x 128) + softmax-CE [151936,256] + "
                                "INT8 [1024,4096]" % args.layers,
                    "layers": args.layers, "tokens_per_step": tokens, "alg_gb_per_step": total_bytes / 1e9,
-                   "residual_fused_into_next_rmsnorm": wl.fuse},
+                   "residual_fused_into_next_rmsnorm": wl.fuse,
+                   "weight_gradients": "reduced per op" if args.immediate_dw else "queued, reduced once per step"},
         "aggregate_gbs": total_bytes / ms / 1e6, "aggregate_frac_of_peak": total_bytes / ms / 1e6 / PEAK_HBM_GBS,
         "host_wall_ms_per_step": wall_ms,
         "device": dev_name, "compute_units": cus, "driver_reported_peak_gbs": drv_peak,

@@ -100,6 +100,16 @@ int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, int C, int S
 int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const float *x, const float *w,
                           int C, int S, int batch, float eps, int variant);
 
+/* Weight-gradient accumulation mode.  By default dw / dwq / dwk are up to date (in stream order) when
+ * the backward call that adds into them returns.  The loops read these gradients only at the optimizer
+ * step, after the whole backward pass (training/training_dynamic/train.m:748-869); with
+ * mi355_dw_defer(1) the library uses that: each backward op queues its reduction and
+ * mi355_dw_flush() runs everything queued in a few launches.  mi355_sync(), mi355_buf_read(),
+ * mi355_set_stream() and mi355_dw_defer(0) flush too.  Results are bit-identical in both modes.
+ * Gradient pointers passed while deferred must be distinct or identical, not partially overlapping. */
+int mi355_dw_defer(int on);
+int mi355_dw_flush(void);
+
 /* Residual add fused with the RMSNorm that follows it in the loops: vDSP_vsma + rmsnorm at
  * training/training_dynamic/train.m:460-461 (and a layer's x_next feeding the next rmsnorm at :417).
  * y = a + alpha*b (as mode 0 of mi355_axpby_dev); yn = rmsnorm(y, w).  One launch instead of two; the

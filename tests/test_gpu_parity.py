@@ -286,6 +286,38 @@ def test_qknorm_rope_golden(br):
     assert H.rel_err(dxd.numpy(), GOLD["qk_dx_v0"]) <= TOL and H.rel_err(dwd.numpy(), GOLD["qk_dw"]) <= TOL
 
 
+def test_deferred_weight_gradients_equal_immediate(br):
+    """mi355_dw_defer(1): reductions queue up and run at mi355_dw_flush(); same bits as the immediate mode,
+    including two ops that add into the same dw (they must keep their order) and more jobs than one launch holds."""
+    B, Cc, S, hd, heads, kvh = 2, 256, 64, 32, 4, 2
+    cd, sd = br.rope_tables_dev(S, hd, 1e6)
+    w = dev(br, H.normal(1, Cc, 1.0, 0.02)); wq = dev(br, H.normal(2, hd, 1.0, 0.02)); wk = dev(br, H.normal(3, hd, 1.0, 0.02))
+    xs = [dev(br, H.normal(10 + i, (B, Cc, S))) for i in range(20)]
+    dys = [dev(br, H.normal(40 + i, (B, Cc, S))) for i in range(20)]
+    q = dev(br, H.normal(70, (B, heads * hd, S))); k = dev(br, H.normal(71, (B, kvh * hd, S)))
+    gq = dev(br, H.normal(72, (B, heads * hd, S))); gk = dev(br, H.normal(73, (B, kvh * hd, S)))
+
+    def run(defer):
+        br.check(br.lib.mi355_dw_defer(1 if defer else 0))
+        dws = [dev(br, H.normal(90 + i, Cc)) for i in range(19)]
+        dwq = dev(br, H.normal(120, hd)); dwk = dev(br, H.normal(121, hd))
+        dx = br.DevArray((B, Cc, S)); dq = br.DevArray((B, heads * hd, S)); dk = br.DevArray((B, kvh * hd, S))
+        for i in range(20):
+            tgt = dws[min(i, 18)]                       # ops 18 and 19 accumulate into the same dw
+            br.check(br.lib.mi355_rmsnorm_bwd_dev(dx.ptr, tgt.ptr, dys[i].ptr, xs[i].ptr, w.ptr, Cc, S, B, 1e-5, 0))
+            br.check(br.lib.mi355_qknorm_rope_bwd_dev(dq.ptr, dk.ptr, dwq.ptr, dwk.ptr, gq.ptr, gk.ptr, q.ptr, k.ptr,
+                                                      wq.ptr, wk.ptr, heads, kvh, hd, S, B, cd, sd, 1e-5, 0))
+        br.check(br.lib.mi355_dw_flush())
+        out = [d.numpy().tobytes() for d in dws] + [dwq.numpy().tobytes(), dwk.numpy().tobytes()]
+        br.check(br.lib.mi355_dw_defer(0))
+        return out
+
+    try:
+        assert run(False) == run(True)
+    finally:
+        br.lib.mi355_dw_defer(0)
+
+
 # ---------------------------------------------------------------------------------------------
 # embedding
 # ---------------------------------------------------------------------------------------------
