@@ -309,10 +309,10 @@ NormCfg pick_cfg(int C, int S, int batch, bool vec_ok, int max_cap, int max_cap_
     NormCfg best{};
     if (!vec_ok) return NormCfg{1, 64, 256, 0};
     if (!lpr_knob && !thr_knob && C >= 512) {
-        // Tall tensors, measured on MI355X at C=1024 and 16x256 columns: 16 waves per workgroup win.
-        // forward: 64-byte strips held in registers, 9.6 us; backward: 128-byte strips read twice
-        // (second read from L2), 17.7 us against 20.9 us for the single-pass register tile.
+        // Tall tensors, measured on MI355X at C=1024 and 16x256 columns with operands cold in HBM: forward, 64-byte strips in registers of a 16-wave workgroup
+        // 9.6 us; backward, the single-pass register tile 16.3 us against 19.9 us for a two-sweep variant.
         if (!backward) return NormCfg{4, 4, 1024, C <= 2048 ? 8 : 0};
+        if (C <= 1024) return NormCfg{4, 4, 256, 16};
         const long strips8 = (long)ceil_div((size_t)S, 32);
         return NormCfg{4, strips8 * batch >= 128 ? 8 : 4, 1024, 0};
     }
