@@ -14,9 +14,12 @@
 //      segment (all positions of one token) is a run of consecutive rows;
 //   3. each (segment, 64-float chunk) is summed sequentially starting from the value already
 //      in dE — short segments by one wave straight from memory, long segments by a whole
-//      workgroup that stages 256 rows at a time in LDS to keep enough loads in flight while one
-//      wave performs the ordered adds.
+//      workgroup that stages 240 rows at a time in LDS to keep enough loads in flight while one
+//      wave performs the ordered adds; both kinds share one launch so the long chains overlap
+//      the many short ones.
 #include "common.h"
+
+#include <algorithm>
 
 #include <rocprim/rocprim.hpp>
 
@@ -25,7 +28,8 @@ namespace {
 constexpr int TT = 64;   // tokens per tile
 constexpr int TD = 64;   // dims per tile
 constexpr int LONG_SEG = 64;    // segments longer than this take the workgroup path
-constexpr int STAGE_ROWS = 256;
+constexpr int STAGE_PER_WAVE = 15;
+constexpr int STAGE_ROWS = 16 * STAGE_PER_WAVE;   // 240 rows x 256 B = 60 KiB of LDS, plus a 4 KiB work list
 
 // ---------------------------------------------------------------------------------------------
 // Gather
@@ -102,8 +106,9 @@ __global__ __launch_bounds__(256) void gather_kernel(float *__restrict__ x, cons
 // ---------------------------------------------------------------------------------------------
 // Scatter-add
 // ---------------------------------------------------------------------------------------------
-__global__ void prep_keys_kernel(int *keys, int *vals, const int32_t *ids, int N, int V) {
+__global__ void prep_keys_kernel(int *keys, int *vals, int *meta, const int32_t *ids, int N, int V) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n == 0) { meta[0] = 0; meta[1] = 0; meta[2] = N; }
     if (n < N) {
         const int id = ids[n];
         keys[n] = (id < 0 || id >= V) ? V : id;   // out-of-range ids sort last and are skipped
@@ -111,46 +116,87 @@ __global__ void prep_keys_kernel(int *keys, int *vals, const int32_t *ids, int N
     }
 }
 
-// meta[0] = number of segments, meta[1] = number of long segments, meta[2] = number of valid entries
-__global__ __launch_bounds__(1024) void plan_kernel(int *rank, int *seg_start, int *long_list, int *meta,
-                                                    const int *keys, const int *vals, int N, int V) {
-    __shared__ int cnt[1024];
-    __shared__ int s_nvalid, s_nlong;
-    const int tid = threadIdx.x;
-    const int per = (N + 1023) / 1024;
-    const int lo = tid * per, hi = min(N, lo + per);
-    if (tid == 0) { s_nvalid = N; s_nlong = 0; }
+// meta[0] = number of segments, meta[2] = number of valid (in-range) entries.
+//
+// Segment starts are found in three small launches: (1) every workgroup flags the heads among its
+// 1024 sorted entries (key differs from its predecessor), counts them and writes the inverse
+// permutation; (2) one workgroup scans the per-workgroup counts; (3) every workgroup writes the
+// positions of its heads at its offset.
+constexpr int PLAN_T = 1024;
+
+__device__ __forceinline__ int block_excl_scan_1024(int v, int *lds, int &total) {
+    // exclusive scan of one int per thread over 1024 threads: wave scan by shuffles, then the 16 wave totals
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int x = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int y = __shfl_up(x, off, 64);
+        if (lane >= off) x += y;
+    }
+    if (lane == 63) lds[wave] = x;
     __syncthreads();
-    int c = 0;
-    for (int i = lo; i < hi; i++) {
+    int base = 0, tot = 0;
+#pragma unroll
+    for (int k = 0; k < PLAN_T / 64; k++) {
+        const int t = lds[k];
+        if (k < wave) base += t;
+        tot += t;
+    }
+    total = tot;
+    __syncthreads();
+    return base + x - v;
+}
+
+__global__ __launch_bounds__(PLAN_T) void plan_flags_kernel(int *__restrict__ rank, int *__restrict__ blk_count,
+                                                            int *__restrict__ meta, const int *__restrict__ keys,
+                                                            const int *__restrict__ vals, int N, int V) {
+    __shared__ int lds[PLAN_T / 64];
+    const int i = blockIdx.x * PLAN_T + threadIdx.x;
+    int head = 0;
+    if (i < N) {
         const int k = keys[i];
+        const int kp = i > 0 ? keys[i - 1] : -1;
         rank[vals[i]] = i;
-        const int kp = i > 0 ? keys[i - 1] : -1;
-        if (k < V && k != kp) c++;
-        if (k >= V && kp < V) s_nvalid = i;   // at most one thread writes
+        head = (k < V && k != kp) ? 1 : 0;
+        if (k >= V && kp < V) meta[2] = i;          // first out-of-range key: at most one thread writes
     }
-    cnt[tid] = c;
-    __syncthreads();
-    // exclusive scan of 1024 counts (Hillis-Steele, in place with double sync)
-    for (int off = 1; off < 1024; off <<= 1) {
-        int v = tid >= off ? cnt[tid - off] : 0;
-        __syncthreads();
-        cnt[tid] += v;
-        __syncthreads();
+    int total;
+    (void)block_excl_scan_1024(head, lds, total);
+    if (threadIdx.x == 0) blk_count[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(PLAN_T) void plan_scan_kernel(int *__restrict__ blk_off, int *__restrict__ seg_start,
+                                                           int *__restrict__ meta, const int *__restrict__ blk_count,
+                                                           int nb) {
+    __shared__ int lds[PLAN_T / 64];
+    int carry = 0;
+    for (int b0 = 0; b0 < nb; b0 += PLAN_T) {
+        const int b = b0 + threadIdx.x;
+        const int v = b < nb ? blk_count[b] : 0;
+        int total;
+        const int ex = block_excl_scan_1024(v, lds, total);
+        if (b < nb) blk_off[b] = carry + ex;
+        carry += total;
     }
-    int pos = cnt[tid] - c;
-    const int nseg = cnt[1023];
-    for (int i = lo; i < hi; i++) {
+    if (threadIdx.x == 0) {
+        meta[0] = carry;
+        seg_start[carry] = meta[2];                 // end of the last segment = number of valid entries
+    }
+}
+
+__global__ __launch_bounds__(PLAN_T) void plan_write_kernel(int *__restrict__ seg_start, const int *__restrict__ blk_off,
+                                                            const int *__restrict__ keys, int N, int V) {
+    __shared__ int lds[PLAN_T / 64];
+    const int i = blockIdx.x * PLAN_T + threadIdx.x;
+    int head = 0;
+    if (i < N) {
         const int k = keys[i];
         const int kp = i > 0 ? keys[i - 1] : -1;
-        if (k < V && k != kp) seg_start[pos++] = i;
+        head = (k < V && k != kp) ? 1 : 0;
     }
-    if (tid == 0) seg_start[nseg] = s_nvalid;
-    __syncthreads();
-    for (int j = tid; j < nseg; j += 1024)
-        if (seg_start[j + 1] - seg_start[j] > LONG_SEG) long_list[atomicAdd(&s_nlong, 1)] = j;
-    __syncthreads();
-    if (tid == 0) { meta[0] = nseg; meta[1] = s_nlong; meta[2] = s_nvalid; }
+    int total;
+    const int ex = block_excl_scan_1024(head, lds, total);
+    if (head) seg_start[blk_off[blockIdx.x] + ex] = i;
 }
 
 // dx [batch][D][S] -> rows[rank[n]][D] (token-major, in sorted order), through a 64x64 LDS tile
@@ -174,7 +220,7 @@ __global__ __launch_bounds__(256) void transpose_sorted_kernel(float *__restrict
             if (d >= D) continue;
             const float *src = dx + ((size_t)b * D + d) * S + t;
             if (s_vec && t + 3 < S) {
-                v4f v = ld4(src);
+                v4f v = ld4_nt(src);
                 tile[dl][4 * tq + 0] = v.x; tile[dl][4 * tq + 1] = v.y;
                 tile[dl][4 * tq + 2] = v.z; tile[dl][4 * tq + 3] = v.w;
             } else {
@@ -207,16 +253,81 @@ __global__ __launch_bounds__(256) void transpose_sorted_kernel(float *__restrict
     }
 }
 
-// Short segments: one wave per (segment, 64-float chunk); rows are consecutive in `rows`.
-__global__ __launch_bounds__(256) void seg_sum_short_kernel(float *__restrict__ dE, const float *__restrict__ rows,
-                                                            const int *__restrict__ seg_start,
-                                                            const int *__restrict__ keys, const int *__restrict__ meta,
-                                                            int D, int nchunk) {
-    const int lane = threadIdx.x & 63;
-    const int wave = (blockIdx.x * 4) + (threadIdx.x >> 6);
-    const int nwaves = gridDim.x * 4;
-    const long units = (long)meta[0] * nchunk;
-    for (long u = wave; u < units; u += nwaves) {
+// Segment sums.  One launch, two kinds of workgroup (1024 threads each):
+//  * the first `long_blocks` workgroups take the LONG segments (more than LONG_SEG rows): workgroup
+//    (x, chunk) walks segments x, x + gridDim.x/..., and for each long one sums its 64-float chunk: 16 waves
+//    stage 240 rows in LDS (15 loads in flight per lane), wave 0 adds them in order, 16 rows per batch of
+//    LDS reads so the adds are not exposed to the LDS latency;
+//  * the others take the short segments: one wave per (segment, 64-float chunk), rows read straight
+//    from memory, eight loads in flight.
+// Either way every (row of dE, d) is written by exactly one lane, sequentially in position order,
+// starting from the value already in dE.
+__global__ __launch_bounds__(1024) void seg_sum_kernel(float *__restrict__ dE, const float *__restrict__ rows,
+                                                       const int *__restrict__ seg_start, const int *__restrict__ keys,
+                                                       const int *__restrict__ meta, int D, int nchunk,
+                                                       int long_x, int short_blocks) {
+    __shared__ float stage[STAGE_ROWS][64];
+    __shared__ int work[1023];      // with nwork: 4 KiB, for 64 KiB of LDS in all
+    __shared__ int nwork;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nseg = meta[0];
+    const int long_blocks = long_x * nchunk;
+    if ((int)blockIdx.x < long_blocks) {
+        const int ch = blockIdx.x % nchunk, x0 = blockIdx.x / nchunk;
+        const int d = ch * 64 + lane;
+        const bool d_ok = d < D;
+        // candidates of this workgroup column: segments x0, x0+long_x, ...; 1023 are screened at a time
+        for (int j0 = 0; x0 + (long)j0 * long_x < nseg; j0 += 1023) {
+            if (threadIdx.x == 0) nwork = 0;
+            __syncthreads();
+            {
+                const long seg = x0 + (long)(j0 + (int)threadIdx.x) * long_x;
+                if (threadIdx.x < 1023 && seg < nseg && seg_start[seg + 1] - seg_start[seg] > LONG_SEG)
+                    work[atomicAdd(&nwork, 1)] = (int)seg;
+            }
+            __syncthreads();
+            const int nw = nwork;
+            for (int k = 0; k < nw; k++) {
+                const int seg = work[k];
+                const int lo = seg_start[seg], hi = seg_start[seg + 1];
+                const int tok = keys[lo];
+                float acc = 0.f;
+                if (wave == 0 && d_ok) acc = dE[(size_t)tok * D + d];
+                for (int base = lo; base < hi; base += STAGE_ROWS) {
+                    const int nrow = min(STAGE_ROWS, hi - base);
+                    float v[STAGE_PER_WAVE];
+#pragma unroll
+                    for (int j = 0; j < STAGE_PER_WAVE; j++) {
+                        const int rl = wave * STAGE_PER_WAVE + j;
+                        v[j] = (rl < nrow && d_ok) ? __builtin_nontemporal_load(rows + (size_t)(base + rl) * D + d) : 0.f;
+                    }
+#pragma unroll
+                    for (int j = 0; j < STAGE_PER_WAVE; j++) stage[wave * STAGE_PER_WAVE + j][lane] = v[j];
+                    __syncthreads();
+                    if (wave == 0) {
+                        int rl = 0;
+                        for (; rl + 16 <= nrow; rl += 16) {
+                            float t[16];
+#pragma unroll
+                            for (int j = 0; j < 16; j++) t[j] = stage[rl + j][lane];
+#pragma unroll
+                            for (int j = 0; j < 16; j++) acc += t[j];
+                        }
+                        for (; rl < nrow; rl++) acc += stage[rl][lane];
+                    }
+                    __syncthreads();
+                }
+                if (wave == 0 && d_ok) dE[(size_t)tok * D + d] = acc;
+            }
+            __syncthreads();
+        }
+        return;
+    }
+    // short segments
+    const int gw = ((int)blockIdx.x - long_blocks) * 16 + wave;
+    const int nwaves = short_blocks * 16;
+    const long units = (long)nseg * nchunk;
+    for (long u = gw; u < units; u += nwaves) {
         const int seg = (int)(u / nchunk), ch = (int)(u - (long)seg * nchunk);
         const int lo = seg_start[seg], hi = seg_start[seg + 1];
         if (hi - lo > LONG_SEG) continue;
@@ -230,50 +341,13 @@ __global__ __launch_bounds__(256) void seg_sum_short_kernel(float *__restrict__ 
         for (; r + 8 <= hi; r += 8) {
             float v[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) v[j] = src[(size_t)j * D];
+            for (int j = 0; j < 8; j++) v[j] = __builtin_nontemporal_load(src + (size_t)j * D);
 #pragma unroll
             for (int j = 0; j < 8; j++) acc += v[j];
             src += (size_t)8 * D;
         }
-        for (; r < hi; r++) { acc += *src; src += D; }
+        for (; r < hi; r++) { acc += __builtin_nontemporal_load(src); src += D; }
         *dst = acc;
-    }
-}
-
-// Long segments: one workgroup per (segment, 64-float chunk); 16 waves stage 256 rows in LDS,
-// wave 0 adds them in order.
-__global__ __launch_bounds__(1024) void seg_sum_long_kernel(float *__restrict__ dE, const float *__restrict__ rows,
-                                                            const int *__restrict__ seg_start,
-                                                            const int *__restrict__ long_list,
-                                                            const int *__restrict__ keys, const int *__restrict__ meta,
-                                                            int D, int nchunk) {
-    __shared__ float stage[STAGE_ROWS][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const long units = (long)meta[1] * nchunk;
-    for (long u = blockIdx.x; u < units; u += gridDim.x) {
-        const int seg = long_list[u / nchunk], ch = (int)(u % nchunk);
-        const int lo = seg_start[seg], hi = seg_start[seg + 1];
-        const int d = ch * 64 + lane;
-        const bool d_ok = d < D;
-        const int tok = keys[lo];
-        float acc = 0.f;
-        if (wave == 0 && d_ok) acc = dE[(size_t)tok * D + d];
-        for (int base = lo; base < hi; base += STAGE_ROWS) {
-            const int nrow = min(STAGE_ROWS, hi - base);
-            float v[16];
-#pragma unroll
-            for (int j = 0; j < 16; j++) {
-                const int rl = wave * 16 + j;
-                v[j] = (rl < nrow && d_ok) ? rows[(size_t)(base + rl) * D + d] : 0.f;
-            }
-#pragma unroll
-            for (int j = 0; j < 16; j++) stage[wave * 16 + j][lane] = v[j];
-            __syncthreads();
-            if (wave == 0)
-                for (int rl = 0; rl < nrow; rl++) acc += stage[rl][lane];
-            __syncthreads();
-        }
-        if (wave == 0 && d_ok) dE[(size_t)tok * D + d] = acc;
     }
 }
 
@@ -317,26 +391,32 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
 
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
     const size_t nb = al((size_t)N * sizeof(int));
+    const int nplan = (int)ceil_div((size_t)N, PLAN_T);
     const size_t off_keys_in = 0, off_vals_in = nb, off_keys = 2 * nb, off_vals = 3 * nb, off_rank = 4 * nb;
-    const size_t off_seg = 5 * nb, off_long = off_seg + al((size_t)(N + 1) * sizeof(int));
-    const size_t off_meta = off_long + nb, off_temp = off_meta + 256;
+    const size_t off_seg = 5 * nb, off_cnt = off_seg + al((size_t)(N + 1) * sizeof(int));
+    const size_t off_boff = off_cnt + al((size_t)nplan * sizeof(int));
+    const size_t off_meta = off_boff + al((size_t)nplan * sizeof(int)), off_temp = off_meta + 256;
     const size_t off_rows = off_temp + al(temp_bytes);
     const size_t total = off_rows + al((size_t)N * D * sizeof(float));
     char *ws = (char *)mi355_ws(total);
     if (!ws) return -1;
     int *keys_in = (int *)(ws + off_keys_in), *vals_in = (int *)(ws + off_vals_in);
     int *keys = (int *)(ws + off_keys), *vals = (int *)(ws + off_vals), *rank = (int *)(ws + off_rank);
-    int *seg_start = (int *)(ws + off_seg), *long_list = (int *)(ws + off_long), *meta = (int *)(ws + off_meta);
+    int *seg_start = (int *)(ws + off_seg), *blk_count = (int *)(ws + off_cnt), *blk_off = (int *)(ws + off_boff);
+    int *meta = (int *)(ws + off_meta);
     float *rows = (float *)(ws + off_rows);
 
     hipLaunchKernelGGL(prep_keys_kernel, dim3((unsigned)ceil_div((size_t)N, 256)), dim3(256), 0, g_ctx.stream, keys_in,
-                       vals_in, ids, N, V);
+                       vals_in, meta, ids, N, V);
     LAUNCH_OK("embed_scatter_add prep");
     e = rocprim::radix_sort_pairs(ws + off_temp, temp_bytes, keys_in, keys, vals_in, vals, (size_t)N, 0, bits,
                                   g_ctx.stream);
     if (e != hipSuccess) return mi355_fail("embed_scatter_add: sort: %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(1024), 0, g_ctx.stream, rank, seg_start, long_list, meta, keys, vals,
+    hipLaunchKernelGGL(plan_flags_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, rank, blk_count, meta, keys, vals,
                        N, V);
+    hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(PLAN_T), 0, g_ctx.stream, blk_off, seg_start, meta, blk_count,
+                       nplan);
+    hipLaunchKernelGGL(plan_write_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, seg_start, blk_off, keys, N, V);
     LAUNCH_OK("embed_scatter_add plan");
     const int t_tiles = (int)ceil_div((size_t)S, TT);
     const dim3 tgrid((unsigned)(batch * t_tiles), (unsigned)ceil_div((size_t)D, TD));
@@ -345,13 +425,12 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     LAUNCH_OK("embed_scatter_add transpose");
     const int nchunk = (int)ceil_div((size_t)D, 64);
     const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
-    hipLaunchKernelGGL(seg_sum_long_kernel, dim3((unsigned)(cu)), dim3(1024), 0, g_ctx.stream, dE, rows, seg_start,
-                       long_list, keys, meta, D, nchunk);
-    LAUNCH_OK("embed_scatter_add long");
-    size_t sblocks = ceil_div((size_t)N * nchunk, 4);
-    if (sblocks > (size_t)cu * 16) sblocks = (size_t)cu * 16;
-    hipLaunchKernelGGL(seg_sum_short_kernel, dim3((unsigned)sblocks), dim3(256), 0, g_ctx.stream, dE, rows, seg_start,
-                       keys, meta, D, nchunk);
-    LAUNCH_OK("embed_scatter_add short");
+    // at most N/LONG_SEG segments can be long; a few dozen workgroup columns cover them
+    int long_x = (int)std::min<size_t>((size_t)N / LONG_SEG + 1, (size_t)std::max(1, cu / nchunk));
+    size_t short_blocks = ceil_div((size_t)N * nchunk, 16);
+    if (short_blocks > (size_t)cu * 4) short_blocks = (size_t)cu * 4;
+    hipLaunchKernelGGL(seg_sum_kernel, dim3((unsigned)(long_x * nchunk + short_blocks)), dim3(1024), 0, g_ctx.stream, dE,
+                       rows, seg_start, keys, meta, D, nchunk, long_x, (int)short_blocks);
+    LAUNCH_OK("embed_scatter_add segment sums");
     return 0;
 }
