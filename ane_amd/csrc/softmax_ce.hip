@@ -8,8 +8,8 @@
 // four waves of a workgroup are combined through LDS.
 //   pass 1  each workgroup reduces a block of rows to per-column (max, sum exp) partials
 //           (online rescaling between 64-row register tiles);
-//   combine per column, partials are merged in a fixed order, the target logit is read, the
-//           per-column loss term is formed and the mean is taken by a fixed tree;
+//   combine per column, partials are merged in a fixed order, the target logit is read and the
+//           per-column loss term is formed (the mean is taken, by a fixed tree, by one workgroup of pass 2);
 //   pass 2  dlogits = (exp(l - M) * (1/L) - onehot) * (1/S) * grad_scale.  Row blocks are visited
 //           in the reverse order of pass 1 so the most recently read rows are re-read first
 //           (they are the most likely to still sit in the last-level cache).
@@ -161,28 +161,28 @@ __global__ __launch_bounds__(1024) void ce_combine_kernel(float *__restrict__ co
     }
 }
 
-// loss = (sum_t colLoss[t]) / S with a fixed summation tree
-__global__ __launch_bounds__(256) void ce_loss_kernel(float *__restrict__ loss_out, const float *__restrict__ colLoss,
-                                                      int S) {
-    __shared__ float red[256];
-    float s = 0.f;
-    for (int t = threadIdx.x; t < S; t += 256) s += colLoss[t];
-    red[threadIdx.x] = s;
-    __syncthreads();
-    for (int off = 128; off > 0; off >>= 1) {
-        if (threadIdx.x < off) red[threadIdx.x] += red[threadIdx.x + off];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) *loss_out = red[0] / (float)S;
-}
-
 template <int VEC>
 __global__ __launch_bounds__(CE_THREADS) void ce_grad_kernel(float *dlogits, const float *logits,
                                                              const float *__restrict__ colM,
                                                              const float *__restrict__ colInv,
                                                              const int32_t *__restrict__ targets, int V, int S,
-                                                             int rows_per_block, float invS, float grad_scale) {
+                                                             int rows_per_block, float invS, float grad_scale,
+                                                             float *__restrict__ loss_out,
+                                                             const float *__restrict__ colLoss) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (blockIdx.x == 0 && blockIdx.y == 0) {
+        // loss = (sum_t colLoss[t]) / S with a fixed summation tree; one workgroup does it on the side
+        __shared__ float red[CE_THREADS];
+        float sl = 0.f;
+        for (int t = threadIdx.x; t < S; t += CE_THREADS) sl += colLoss[t];
+        red[threadIdx.x] = sl;
+        __syncthreads();
+        for (int off = CE_THREADS / 2; off > 0; off >>= 1) {
+            if ((int)threadIdx.x < off) red[threadIdx.x] += red[threadIdx.x + off];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) *loss_out = red[0] / (float)S;
+    }
     const int col = (blockIdx.y * 64 + lane) * VEC;
     if (col >= S) return;
     const int rb = gridDim.x - 1 - blockIdx.x;           // reverse order of pass 1
@@ -261,14 +261,12 @@ MI355_API int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float 
     hipLaunchKernelGGL(ce_combine_kernel, dim3((unsigned)ceil_div((size_t)S, 64)), dim3(1024), 0, g_ctx.stream, colM,
                        colInv, colLoss, pm, pl, logits, targets, V, S, nblk);
     LAUNCH_OK("softmax_ce combine");
-    hipLaunchKernelGGL(ce_loss_kernel, dim3(1), dim3(256), 0, g_ctx.stream, loss_dev, colLoss, S);
-    LAUNCH_OK("softmax_ce loss");
     if (vec_ok)
         hipLaunchKernelGGL((ce_grad_kernel<4>), grid, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
-                           targets, V, S, rpb, 1.0f / (float)S, grad_scale);
+                           targets, V, S, rpb, 1.0f / (float)S, grad_scale, loss_dev, colLoss);
     else
         hipLaunchKernelGGL((ce_grad_kernel<1>), grid, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
-                           targets, V, S, rpb, 1.0f / (float)S, grad_scale);
+                           targets, V, S, rpb, 1.0f / (float)S, grad_scale, loss_dev, colLoss);
     LAUNCH_OK("softmax_ce grad");
     return 0;
 }

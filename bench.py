@@ -98,6 +98,7 @@ class Workload:
         self.q8 = A(n8, np.int8)
         self.y8 = A(n8)
         self.scale8 = A(1)
+        self.scratch_h = A((B, H, S))          # output of the copy-shaped calibration op only
         self.cos, self.sin = br.rope_tables_dev(S, cfg["hd"], cfg["theta"])
         self.alpha = float(np.float32(1.0 / np.sqrt(2.0 * cfg["layers"])))   # training/training_dynamic/train.m:188
         br.sync()
@@ -123,7 +124,7 @@ class Workload:
             ck(lib.mi355_residual_rmsnorm_fwd_dev(d["x_next"].ptr, d["xn_next"].ptr, d["x2"].ptr, d["f"].ptr,
                                                   self.alpha, d["w_att"].ptr, C, S, B, 1e-5))
         elif name == "scale_copy":     # dffn = alpha*dy shaped stream over the SwiGLU-sized buffers
-            ck(lib.mi355_axpby_dev(d["dh1"].ptr, d["dsilu"].ptr, None, self.alpha, n_h, 1))
+            ck(lib.mi355_axpby_dev(self.scratch_h.ptr, d["dsilu"].ptr, None, self.alpha, n_h, 1))
         elif name == "swiglu_fwd":
             ck(lib.mi355_swiglu_fwd_dev(d["gate"].ptr, d["h1"].ptr, d["h3"].ptr, n_h))
         elif name == "residual2":
