@@ -69,6 +69,12 @@ SIGNATURES = {
     "mi355_int8_scale_dev": (_i, [_p, _p, _z]),
     "mi355_int8_quant_dev": (_i, [_p, _p, _p, _z, _i]),
     "mi355_int8_dequant_dev": (_i, [_p, _p, _p, _z]),
+    "mi355_sumsq_accum_dev": (_i, [_p, _p, _z, _f]),
+    "mi355_clip_scale_dev": (_i, [_p, _p, _f]),
+    "mi355_adam_update_dev": (_i, [_p, _p, _p, _p, _z, _i, _f, _f, _f, _f, _f, _f, _p, _i]),
+    "mi355_gqa_tile_dev": (_i, [_p, _p, _i, _i, _i, _i, _i]),
+    "mi355_gqa_reduce_dev": (_i, [_p, _p, _i, _i, _i, _i, _i]),
+    "mi355_adam_update": (None, [_p, _p, _p, _p, _z, _i, _f, _f, _f, _f, _f]),
     "mi355_rmsnorm": (None, [_p, _p, _p, _i, _i]),
     "mi355_rmsnorm_bwd": (None, [_p, _p, _p, _p, _p, _i, _i]),
     "mi355_cross_entropy_loss": (_f, [_p, _p, _p, _i, _i]),

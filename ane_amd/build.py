@@ -9,7 +9,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmi355_ops.so")
 
-SOURCES = ["context.hip", "dw_reduce.hip", "norm.hip", "eltwise.hip", "qknorm_rope.hip", "embed.hip", "softmax_ce.hip",
+SOURCES = ["context.hip", "dw_reduce.hip", "norm.hip", "eltwise.hip", "qknorm_rope.hip", "embed.hip", "softmax_ce.hip", "optim.hip",
            "host_dropins.hip"]
 
 # -ffp-contract=off: products and sums round separately, as the reference's sequences of vDSP calls do;

@@ -303,6 +303,44 @@ __global__ void dequant_scalar(float *x, const int8_t *q, const float *scale_p, 
 
 // One 128-bit access per lane and as many workgroups as that takes measured fastest on MI355X
 // (75-77 % of peak for the SwiGLU streams against 68-70 % with four accesses per lane).
+// ---- GQA tile / reduce (training/training_dynamic/io.h:330-351) ----
+// slab = hd*S floats of one head; one lane = one 128-bit column group of one KV-head slab
+template <int VEC>
+__global__ __launch_bounds__(EW_THREADS) void gqa_tile_kernel(float *__restrict__ out, const float *__restrict__ in,
+                                                              int kv_heads, int ratio, size_t slabv, size_t total) {
+    const size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;      // over batch*kv_heads*slabv
+    if (i >= total) return;
+    const size_t head = i / slabv, off = i - head * slabv;             // head = b*kv_heads + kv
+    const size_t b = head / kv_heads, kv = head - b * kv_heads;
+    const size_t dst0 = ((b * kv_heads + kv) * ratio) * slabv + off;
+    if constexpr (VEC == 4) {
+        const v4f v = ld4_nt(in + 4 * i);
+        for (int r = 0; r < ratio; r++) st4_nt(out + 4 * (dst0 + (size_t)r * slabv), v);
+    } else {
+        const float v = in[i];
+        for (int r = 0; r < ratio; r++) out[dst0 + (size_t)r * slabv] = v;
+    }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(EW_THREADS) void gqa_reduce_kernel(float *__restrict__ out, const float *__restrict__ in,
+                                                                int kv_heads, int ratio, size_t slabv, size_t total) {
+    const size_t i = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;      // over batch*kv_heads*slabv (outputs)
+    if (i >= total) return;
+    const size_t head = i / slabv, off = i - head * slabv;
+    const size_t b = head / kv_heads, kv = head - b * kv_heads;
+    const size_t src0 = ((b * kv_heads + kv) * ratio) * slabv + off;
+    if constexpr (VEC == 4) {
+        v4f acc = {0.f, 0.f, 0.f, 0.f};                                 // memset, then += in head order (io.h:342-350)
+        for (int r = 0; r < ratio; r++) acc += ld4_nt(in + 4 * (src0 + (size_t)r * slabv));
+        st4_nt(out + 4 * i, acc);
+    } else {
+        float acc = 0.f;
+        for (int r = 0; r < ratio; r++) acc += in[src0 + (size_t)r * slabv];
+        out[i] = acc;
+    }
+}
+
 inline int pick_unroll(size_t n4, int deflt) {
     int u = g_ctx.ew_unroll ? g_ctx.ew_unroll : deflt;
     if (u != 1 && u != 2 && u != 4 && u != 8) u = deflt;
@@ -546,4 +584,35 @@ MI355_API int mi355_int8_dequant_dev(float *x, const int8_t *q, const float *sca
         LAUNCH_OK("int8_dequant tail");
     }
     return 0;
+}
+
+// ---- GQA tile / reduce ----
+static int gqa_run(bool reduce, float *out, const float *in, int kv_heads, int ratio, int hd, int S, int batch) {
+    const char *who = reduce ? "gqa_reduce" : "gqa_tile";
+    if (!mi355_ready(who)) return -1;
+    if (!out || !in) return mi355_fail("%s: NULL pointer", who);
+    if (kv_heads <= 0 || ratio <= 0 || hd <= 0 || S <= 0 || batch <= 0)
+        return mi355_fail("%s: bad shape kv_heads=%d ratio=%d hd=%d S=%d batch=%d", who, kv_heads, ratio, hd, S, batch);
+    const size_t slab = (size_t)hd * S;
+    const bool vec = (slab % 4 == 0) && aligned16(out) && aligned16(in);
+    const size_t slabv = vec ? slab / 4 : slab;
+    const size_t total = (size_t)batch * kv_heads * slabv;
+    const unsigned blocks = (unsigned)ceil_div(total, EW_THREADS);
+    if (reduce) {
+        if (vec) hipLaunchKernelGGL((gqa_reduce_kernel<4>), dim3(blocks), dim3(EW_THREADS), 0, g_ctx.stream, out, in, kv_heads, ratio, slabv, total);
+        else hipLaunchKernelGGL((gqa_reduce_kernel<1>), dim3(blocks), dim3(EW_THREADS), 0, g_ctx.stream, out, in, kv_heads, ratio, slabv, total);
+    } else {
+        if (vec) hipLaunchKernelGGL((gqa_tile_kernel<4>), dim3(blocks), dim3(EW_THREADS), 0, g_ctx.stream, out, in, kv_heads, ratio, slabv, total);
+        else hipLaunchKernelGGL((gqa_tile_kernel<1>), dim3(blocks), dim3(EW_THREADS), 0, g_ctx.stream, out, in, kv_heads, ratio, slabv, total);
+    }
+    LAUNCH_OK(who);
+    return 0;
+}
+
+MI355_API int mi355_gqa_tile_dev(float *out, const float *in, int kv_heads, int ratio, int hd, int S, int batch) {
+    return gqa_run(false, out, in, kv_heads, ratio, hd, S, batch);
+}
+
+MI355_API int mi355_gqa_reduce_dev(float *out, const float *in, int kv_heads, int ratio, int hd, int S, int batch) {
+    return gqa_run(true, out, in, kv_heads, ratio, hd, S, batch);
 }

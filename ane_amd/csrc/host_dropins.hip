@@ -247,3 +247,20 @@ MI355_API void mi355_axpby(float *y, const float *a, const float *b, float alpha
     if (mi355_axpby_dev(yd, ad, mode != 1 ? bd : nullptr, alpha, n, mode)) return;
     d2h(y, yd, nb);
 }
+
+// adam_update (training/training_dynamic/cpu_ops.h:56-64) on host arrays.
+MI355_API void mi355_adam_update(float *w, const float *g, float *m, float *v, size_t n, int t, float lr, float b1,
+                                 float b2, float eps, float wd) {
+    if (!mi355_ready("adam_update")) return;
+    if (!w || !g || !m || !v || n == 0 || t < 1) { mi355_fail("adam_update: bad arguments"); return; }
+    const size_t nb = n * sizeof(float);
+    float *wd_ = (float *)slot(0, nb), *gd = (float *)slot(1, nb), *md = (float *)slot(2, nb), *vd = (float *)slot(3, nb);
+    if (!wd_ || !gd || !md || !vd) return;
+    if (!h2d(wd_, w, nb) || !h2d(gd, g, nb) || !h2d(md, m, nb) || !h2d(vd, v, nb)) return;
+    if (mi355_adam_update_dev(wd_, gd, md, vd, n, t, lr, b1, b2, eps, wd, 1.0f, nullptr, 0)) return;
+    std::vector<float> w2(n), m2(n);
+    if (!d2h(w2.data(), wd_, nb) || !d2h(m2.data(), md, nb)) return;
+    if (!d2h(v, vd, nb)) return;
+    memcpy(w, w2.data(), nb);
+    memcpy(m, m2.data(), nb);
+}

@@ -9,8 +9,8 @@
  * Everything else is the reference's call order, operand order and accumulate-vs-assign rules.
  *
  * Model shape comes from compile-time macros, as the reference's models/*.h headers do.
- * Output: a binary dump (floats) of loss, final dy, the RMSNorm weight gradients and the
- * embedding gradient, written to argv[1].
+ * Output: a binary dump (floats) of loss, final dy, the (scaled) RMSNorm weight gradients and
+ * embedding gradient, and the RMSNorm weights and embedding table after one Adam step, written to argv[1].
  *
  *   gcc -O2 -ffp-contract=off -Iinclude ane_amd/host/train_step_mirror.c -Lane_amd -lmi355_ops -lm
  */
@@ -145,6 +145,26 @@ int main(int argc, char **argv) {
     }
     embed_backward(gembed, dy, input_tokens, DIM, SEQ);                                 /* :728 */
 
+    /* ===== optimizer tail (train.m:748-877), the tensors this mirror owns ===== */
+    {
+        const float gsc = 1.0f / loss_scale;                  /* accum_steps = 1 (:750) */
+        const float lr = 3e-4f, b1 = 0.9f, b2 = 0.95f, eps = 1e-8f, wd = 0.1f;
+        const int adam_t = 1;
+        for (int L = 0; L < NLAYERS; L++)
+            for (int i = 0; i < DIM; i++) { g_rms_att[L][i] *= gsc; g_rms_ffn[L][i] *= gsc; }      /* :766 */
+        for (int i = 0; i < DIM; i++) grms_final[i] *= gsc;                                        /* :768 */
+        for (size_t i = 0; i < (size_t)VOCAB * DIM; i++) gembed[i] *= gsc;                         /* :770 */
+        AdamState a_final = {fmalloc(DIM), fmalloc(DIM), DIM};
+        AdamState a_embed = {fmalloc((size_t)VOCAB * DIM), fmalloc((size_t)VOCAB * DIM), (size_t)VOCAB * DIM};
+        for (int L = 0; L < NLAYERS; L++) {
+            AdamState a1 = {fmalloc(DIM), fmalloc(DIM), DIM}, a2 = {fmalloc(DIM), fmalloc(DIM), DIM};
+            adam_update(rms_att[L], g_rms_att[L], &a1, adam_t, lr, b1, b2, eps, 0.0f);              /* :851 */
+            adam_update(rms_ffn[L], g_rms_ffn[L], &a2, adam_t, lr, b1, b2, eps, 0.0f);              /* :852 */
+        }
+        adam_update(rms_final, grms_final, &a_final, adam_t, lr, b1, b2, eps, 0.0f);                /* :866 */
+        adam_update(embed, gembed, &a_embed, adam_t, lr, b1, b2, eps, wd);                          /* :867 */
+    }
+
     FILE *f = fopen(argv[1], "wb");
     if (!f) { perror(argv[1]); return 4; }
     fwrite(&loss, 4, 1, f);
@@ -152,6 +172,10 @@ int main(int argc, char **argv) {
     fwrite(grms_final, 4, DIM, f);
     for (int L = 0; L < NLAYERS; L++) { fwrite(g_rms_att[L], 4, DIM, f); fwrite(g_rms_ffn[L], 4, DIM, f); }
     fwrite(gembed, 4, (size_t)VOCAB * DIM, f);
+    /* weights after the Adam step */
+    fwrite(rms_final, 4, DIM, f);
+    for (int L = 0; L < NLAYERS; L++) { fwrite(rms_att[L], 4, DIM, f); fwrite(rms_ffn[L], 4, DIM, f); }
+    fwrite(embed, 4, (size_t)VOCAB * DIM, f);
     fclose(f);
     printf("loss=%.6f\n", loss);
     mi355_shutdown();

@@ -192,6 +192,28 @@ int mi355_int8_scale_dev(float *scale_dev, const float *x, size_t n);
 int mi355_int8_quant_dev(int8_t *q, const float *x, const float *scale_dev, size_t n, int rounding);
 int mi355_int8_dequant_dev(float *x, const int8_t *q, const float *scale_dev, size_t n);
 
+/* Optimizer tail — training/training_dynamic/train.m:748-877 in two sweeps instead of five.
+ * mi355_sumsq_accum_dev: *acc_dev += sum_i (pre_scale*g_i)^2 — the gradient-scale loop (:754-769) and the
+ * vDSP_dotpr per tensor (:771-787) in one read; deterministic for a given n.
+ * mi355_clip_scale_dev: *scale_dev = grad_clip/sqrt(*sumsq_dev) if grad_clip > 0 and the norm exceeds it,
+ * else 1 (:806-808); stays on the device, so no host round trip sits between norm and update.
+ * mi355_adam_update_dev: adam_update — training/training_dynamic/cpu_ops.h:56-64 (AdamW; wd = 0 is
+ * training/stories_cpu_ops.h:55-63) — on g' = (g*scale1)*scale2 (scale2_dev may be NULL = 1), i.e. with
+ * the scale pass (:754-769) and the clip pass (:806-821) folded in; zero_grad != 0 also clears g
+ * (layer_grads_zero / memset, :873-877).  t >= 1 is the Adam step count. */
+int mi355_sumsq_accum_dev(float *acc_dev, const float *g, size_t n, float pre_scale);
+int mi355_clip_scale_dev(float *scale_dev, const float *sumsq_dev, float grad_clip);
+int mi355_adam_update_dev(float *w, float *g, float *m, float *v, size_t n, int t, float lr, float b1,
+                          float b2, float eps, float wd, float scale1, const float *scale2_dev,
+                          int zero_grad);
+
+/* GQA helpers of the dynamic loop — training/training_dynamic/io.h:330-351 (calls at
+ * training/training_dynamic/train.m:620-621,653-654).  tile: out[batch][kv_heads*ratio*hd][S] gets each KV
+ * head `ratio` times; reduce: out[batch][kv_heads*hd][S] = sum over the `ratio` query heads of each group,
+ * added in head order (the reference's memset + += loop). */
+int mi355_gqa_tile_dev(float *out, const float *in, int kv_heads, int ratio, int hd, int S, int batch);
+int mi355_gqa_reduce_dev(float *out, const float *in, int kv_heads, int ratio, int hd, int S, int batch);
+
 /* ------------------------------------------------------------------------------------------
  * Host-pointer drop-ins: the reference signatures verbatim (host float* in, host float* out),
  * so a caller swaps the symbol only.  Each call stages through cached device buffers
@@ -224,6 +246,9 @@ void mi355_swiglu_bwd(float *dh1, float *dh3, const float *dsilu, const float *h
                       size_t n);
 void mi355_swiglu_fwd(float *out, const float *h1, const float *h3, size_t n);
 void mi355_axpby(float *y, const float *a, const float *b, float alpha, size_t n, int mode);
+/* adam_update — training/training_dynamic/cpu_ops.h:56 with the AdamState fields spelled out */
+void mi355_adam_update(float *w, const float *g, float *m, float *v, size_t n, int t, float lr, float b1,
+                       float b2, float eps, float wd);
 
 #ifdef __cplusplus
 }

@@ -47,6 +47,17 @@ static inline void rope_backward_inplace(float *dx, int seq, int dim, int hd) {
     mi355_rope_backward_inplace(dx, seq, dim, hd);
 }
 
+/* adam_update — training/training_dynamic/cpu_ops.h:56-64 (the static loop's version,
+ * training/stories_cpu_ops.h:55-63, is the same with wd = 0).  AdamState as in
+ * training/training_dynamic/config.h:46; define MI355_HAVE_ADAMSTATE if the including file already has it. */
+#ifndef MI355_HAVE_ADAMSTATE
+typedef struct { float *m, *v; size_t n; } AdamState;
+#endif
+static inline void adam_update(float *w, const float *g, AdamState *s, int t, float lr, float b1, float b2, float eps,
+                               float wd) {
+    mi355_adam_update(w, g, s->m, s->v, s->n, t, lr, b1, b2, eps, wd);
+}
+
 /* The loops' inline Accelerate blocks, as calls with the same operand order:
  *   vDSP_vsma(b, 1, &alpha, a, 1, y, 1, n)   -> mi355_vsma(b, alpha, a, y, n)     train.m:460
  *   vDSP_vsmul(a, 1, &alpha, y, 1, n)        -> mi355_vsmul(a, alpha, y, n)       train.m:497,523,595

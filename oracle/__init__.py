@@ -63,6 +63,8 @@ def _load():
         "orc_axpby_mt": (None, [_f32p, _f32p, C.c_void_p, C.c_float, C.c_size_t, C.c_int, C.c_int]),
         "orc_embed_lookup_batched": (C.c_int, [_f32p, _f32p, _i32p, C.c_int, C.c_int, C.c_int, C.c_int]),
         "orc_embed_backward_batched": (None, [_f32p, _f32p, _i32p, C.c_int, C.c_int, C.c_int, C.c_int]),
+        "orc_sumsq_scaled": (C.c_float, [_f32p, C.c_size_t, C.c_float]),
+        "orc_clip_scale": (C.c_float, [C.c_float, C.c_float]),
         "orc_recipe_drand48": (None, [C.c_int, C.c_long, _f32p, _f32p, _f32p, C.c_size_t, C.c_int]),
         "orc_now_s": (C.c_double, []),
         "orc_max_threads": (C.c_int, []),
@@ -234,3 +236,12 @@ def recipe_drand48(recipe, seed, n, d):
     x = np.zeros(n, np.float32); dy = np.zeros(n, np.float32); w = np.zeros(max(d, 1), np.float32)
     lib.orc_recipe_drand48(recipe, seed, x, dy, w, n, d)
     return x, dy, w
+
+
+def sumsq_scaled(g, pre_scale=1.0):
+    g = _f32(g)
+    return float(lib.orc_sumsq_scaled(g.reshape(-1), g.size, pre_scale))
+
+
+def clip_scale(sumsq, grad_clip):
+    return float(lib.orc_clip_scale(sumsq, grad_clip))

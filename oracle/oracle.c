@@ -412,6 +412,22 @@ ORC_API void orc_adam_update(float *w, const float *g, float *m, float *v, size_
     }
 }
 
+/* Global gradient norm pieces — training/training_dynamic/train.m:754-787,806-808: the scale pass
+ * g *= gsc followed by vDSP_dotpr(g,g) (order unpublished: 8 strided lanes, as sve), and the clip scale. */
+ORC_API float orc_sumsq_scaled(const float *g, size_t n, float pre_scale) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (size_t i = 0; i < n; i++) {
+        float t = g[i] * pre_scale;
+        acc[i & 7] += t * t;
+    }
+    return ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+}
+
+ORC_API float orc_clip_scale(float sumsq, float grad_clip) {
+    float norm = sqrtf(sumsq);
+    return (grad_clip > 0 && norm > grad_clip) ? grad_clip / norm : 1.0f;
+}
+
 /* ---------------------------------------------------------------------------------------------
  * Batched wrappers: the reference processes one [C,S] sequence per call; "batch B" is B calls
  * on consecutive slabs (dw accumulates across the calls in slab order).  With threads > 1 the

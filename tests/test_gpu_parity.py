@@ -485,6 +485,59 @@ def test_int8_golden_and_zero_tensor(br):
 
 
 # ---------------------------------------------------------------------------------------------
+# next rows: optimizer tail and GQA helpers
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [1024 * 3072, 1024, 100003, 5])
+def test_optimizer_tail(br, n):
+    """Scale + global norm + clip + AdamW as two sweeps (training/training_dynamic/train.m:748-877)."""
+    say("optimizer tail n=%d" % n)
+    w = H.normal(50, n, 0, 0.05); g = H.normal(51, n) * 40; m = H.normal(52, n, 0, 0.01)
+    v = np.abs(H.normal(53, n, 0, 0.01))
+    gsc = np.float32(1.0 / 256.0); clip = np.float32(1e-3)
+    t, lr, b1, b2, eps, wd = 7, 3e-4, 0.9, 0.95, 1e-8, 0.1
+    wd_, gd, md, vd = dev(br, w), dev(br, g), dev(br, m), dev(br, v)
+    ss = dev(br, np.zeros(1, np.float32)); cs = br.DevArray(1)
+    br.check(br.lib.mi355_sumsq_accum_dev(ss.ptr, gd.ptr, n, gsc))
+    br.check(br.lib.mi355_sumsq_accum_dev(ss.ptr, gd.ptr, n, gsc))           # accumulates over tensors
+    t64 = 2 * float(np.sum((g * gsc).astype(np.float64) ** 2))
+    assert abs(ss.numpy()[0] - t64) <= TOL * t64
+    # the oracle sums millions of float32 terms in eight running lanes (vDSP_dotpr's order is unpublished); its own
+    # distance from the float64 sum is ~1e-4 at this length, so it can only be held to that
+    r_ss = O.sumsq_scaled(g, gsc)
+    assert abs(ss.numpy()[0] - 2 * r_ss) <= 5e-4 * 2 * r_ss
+    br.check(br.lib.mi355_clip_scale_dev(cs.ptr, ss.ptr, clip))
+    r_cs = O.clip_scale(float(ss.numpy()[0]), clip)
+    assert cs.numpy()[0] == np.float32(r_cs) and r_cs < 1.0
+    br.check(br.lib.mi355_adam_update_dev(wd_.ptr, gd.ptr, md.ptr, vd.ptr, n, t, lr, b1, b2, eps, wd, gsc, cs.ptr, 1))
+    g2 = (g * gsc) * np.float32(r_cs)                                         # the two scale passes of the reference
+    rw, rm, rv = O.adam_update(w, g2, m, v, t, lr, b1, b2, eps, wd)
+    assert H.rel_err(md.numpy(), rm) <= TOL and H.rel_err(vd.numpy(), rv) <= TOL
+    assert H.rel_err(wd_.numpy(), rw) <= TOL
+    assert H.rel_err(wd_.numpy() - w, rw - w) <= 1e-4                         # the update itself, not just w
+    assert not gd.numpy().any()                                               # zero_grad
+    # no clip, no zeroing, NULL scale pointer
+    wd_, gd, md, vd = dev(br, w), dev(br, g), dev(br, m), dev(br, v)
+    br.check(br.lib.mi355_adam_update_dev(wd_.ptr, gd.ptr, md.ptr, vd.ptr, n, 1, lr, b1, b2, eps, 0.0, 1.0, None, 0))
+    rw, rm, rv = O.adam_update(w, g, m, v, 1, lr, b1, b2, eps, 0.0)
+    assert H.rel_err(wd_.numpy(), rw) <= TOL and H.rel_err(md.numpy(), rm) <= TOL and H.rel_err(vd.numpy(), rv) <= TOL
+    assert np.array_equal(gd.numpy(), g)
+    br.check(br.lib.mi355_clip_scale_dev(cs.ptr, ss.ptr, np.float32(1e9)))
+    assert cs.numpy()[0] == 1.0
+
+
+@pytest.mark.parametrize("B,kvh,ratio,hd,S", [(16, 8, 2, 128, 256), (2, 3, 4, 6, 5), (1, 1, 1, 4, 4)])
+def test_gqa_tile_reduce(br, B, kvh, ratio, hd, S):
+    k = H.normal(54, (B, kvh * hd, S)); g = H.normal(55, (B, kvh * ratio * hd, S))
+    kd, gd = dev(br, k), dev(br, g)
+    td = br.DevArray(g.shape); rd = br.DevArray(k.shape)
+    br.check(br.lib.mi355_gqa_tile_dev(td.ptr, kd.ptr, kvh, ratio, hd, S, B))
+    br.check(br.lib.mi355_gqa_reduce_dev(rd.ptr, gd.ptr, kvh, ratio, hd, S, B))
+    for b in range(B):
+        assert np.array_equal(td.numpy()[b], O.gqa_tile(k[b], kvh, ratio, hd))
+        assert np.array_equal(rd.numpy()[b], O.gqa_reduce(g[b], kvh, ratio, hd))   # same add order: bit-exact
+
+
+# ---------------------------------------------------------------------------------------------
 # host-pointer drop-ins (reference signatures) and error behaviour
 # ---------------------------------------------------------------------------------------------
 def _p(a):

@@ -91,7 +91,17 @@ def replay():
         dx_rms, g_att[L] = O.rmsnorm_bwd(dx_attn, ac["layer_in"], rms_att[L])
         dy = O.axpby(dx_rms, dx2, 0.0, 2)
     gembed = O.embed_backward(np.zeros((VOCAB, DIM), f32), dy[None], tok[None])
-    return loss, dy, grms_final, g_att, g_ffn, gembed
+    # optimizer tail: scale by 1/loss_scale, then one Adam step (AdamW with wd on the embedding only)
+    gsc = f32(1.0) / f32(256.0)
+    g_att = [g * gsc for g in g_att]; g_ffn = [g * gsc for g in g_ffn]
+    grms_final = grms_final * gsc; gembed = gembed * gsc
+    hp = dict(t=1, lr=3e-4, b1=0.9, b2=0.95, eps=1e-8)
+    z = lambda a: np.zeros_like(a)
+    w_att = [O.adam_update(rms_att[L], g_att[L], z(rms_att[L]), z(rms_att[L]), wd=0.0, **hp)[0] for L in range(NLAYERS)]
+    w_ffn = [O.adam_update(rms_ffn[L], g_ffn[L], z(rms_ffn[L]), z(rms_ffn[L]), wd=0.0, **hp)[0] for L in range(NLAYERS)]
+    w_final = O.adam_update(rms_final, grms_final, z(rms_final), z(rms_final), wd=0.0, **hp)[0]
+    w_embed = O.adam_update(embed, gembed, z(embed), z(embed), wd=0.1, **hp)[0]
+    return loss, dy, grms_final, g_att, g_ffn, gembed, w_final, w_att, w_ffn, w_embed
 
 
 def test_training_step_mirror_matches_oracle_replay(tmp_path):
@@ -101,10 +111,10 @@ def test_training_step_mirror_matches_oracle_replay(tmp_path):
     assert r.returncode == 0, r.stdout + r.stderr
     raw = np.fromfile(out, f32)
     DS = DIM * SEQ
-    sizes = [1, DS, DIM] + [DIM] * (2 * NLAYERS) + [VOCAB * DIM]
+    sizes = [1, DS, DIM] + [DIM] * (2 * NLAYERS) + [VOCAB * DIM] + [DIM] + [DIM] * (2 * NLAYERS) + [VOCAB * DIM]
     assert raw.size == sum(sizes)
     parts = np.split(raw, np.cumsum(sizes)[:-1])
-    loss, dy, grms_final, g_att, g_ffn, gembed = replay()
+    loss, dy, grms_final, g_att, g_ffn, gembed, w_final, w_att, w_ffn, w_embed = replay()
     # a chain of ~40 ops: each is held to 1e-5 on its own (test_gpu_parity.py); the chain to 1e-4
     tol = 1e-4
     assert abs(parts[0][0] - loss) <= 1e-5 * abs(loss)
@@ -113,7 +123,14 @@ def test_training_step_mirror_matches_oracle_replay(tmp_path):
     for L in range(NLAYERS):
         assert H.rel_err(parts[3 + 2 * L], g_att[L]) <= tol
         assert H.rel_err(parts[4 + 2 * L], g_ffn[L]) <= tol
-    assert H.rel_err(parts[-1], gembed) <= tol
+    ge = 3 + 2 * NLAYERS
+    assert H.rel_err(parts[ge], gembed) <= tol
     touched = np.unique([(7 * t + 13) % 256 + 1 for t in range(SEQ)])
     untouched = np.setdiff1d(np.arange(VOCAB), touched)
-    assert not parts[-1].reshape(VOCAB, DIM)[untouched].any()
+    assert not parts[ge].reshape(VOCAB, DIM)[untouched].any()
+    # weights after the Adam step (first step: the update is ~lr*sign(g), so compare the CHANGE as well)
+    assert H.rel_err(parts[ge + 1], w_final) <= 1e-6
+    for L in range(NLAYERS):
+        assert H.rel_err(parts[ge + 2 + 2 * L], w_att[L]) <= 1e-6
+        assert H.rel_err(parts[ge + 3 + 2 * L], w_ffn[L]) <= 1e-6
+    assert H.rel_err(parts[-1], w_embed) <= 1e-5

@@ -231,6 +231,16 @@ def test_adam_matches_formula():
     assert H.rel_err(m2, m64) < 2e-6 and H.rel_err(v2, v64) < 2e-6 and H.rel_err(w2, w64) < 2e-6
 
 
+def test_sumsq_and_clip_scale():
+    g = H.normal(40, 100003) * 3
+    gsc = np.float32(1.0 / 256.0)
+    ref = float(np.sum((g * gsc).astype(np.float64) ** 2))          # the scale pass rounds to float32 first
+    assert abs(O.sumsq_scaled(g, gsc) - ref) <= 2e-6 * ref
+    assert O.sumsq_scaled(np.array([3.0, 4.0], np.float32), 1.0) == 25.0
+    assert O.clip_scale(25.0, 1.0) == np.float32(1.0) / np.float32(5.0)   # norm 5 > clip 1 -> 1/5
+    assert O.clip_scale(25.0, 10.0) == 1.0 and O.clip_scale(25.0, 0.0) == 1.0
+
+
 # ---------------------------------------------------------------------------------------------
 # embedding
 # ---------------------------------------------------------------------------------------------
