@@ -72,6 +72,8 @@ SIGNATURES = {
     "mi355_sumsq_accum_dev": (_i, [_p, _p, _z, _f]),
     "mi355_clip_scale_dev": (_i, [_p, _p, _f]),
     "mi355_adam_update_dev": (_i, [_p, _p, _p, _p, _z, _i, _f, _f, _f, _f, _f, _f, _p, _i]),
+    "mi355_sumsq_accum_multi_dev": (_i, [_p, _p, _p, _i, _f]),
+    "mi355_adam_update_multi_dev": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _f, _f, _f, _f, _f, _p, _i]),
     "mi355_gqa_tile_dev": (_i, [_p, _p, _i, _i, _i, _i, _i]),
     "mi355_gqa_reduce_dev": (_i, [_p, _p, _i, _i, _i, _i, _i]),
     "mi355_adam_update": (None, [_p, _p, _p, _p, _z, _i, _f, _f, _f, _f, _f]),

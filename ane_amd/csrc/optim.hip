@@ -106,7 +106,129 @@ __global__ __launch_bounds__(OPT_THREADS) void adam_kernel(float *__restrict__ w
     }
 }
 
+// ---- several tensors per launch: blockIdx.y selects the tensor ----
+constexpr int MT_MAX = 16;
+struct MtSumsq {
+    const float *g[MT_MAX];
+    size_t n[MT_MAX];
+};
+struct MtAdam {
+    float *w[MT_MAX], *g[MT_MAX], *m[MT_MAX], *v[MT_MAX];
+    size_t n[MT_MAX];
+    float wd[MT_MAX];
+};
+
+// partials laid out [tensor][gridDim.x]; every tensor uses the same fixed grid, so the sum is deterministic
+__global__ __launch_bounds__(OPT_THREADS) void sumsq_partial_mt_kernel(float *__restrict__ part, MtSumsq a, float pre) {
+    __shared__ float red[OPT_THREADS / 64];
+    const float *__restrict__ g = a.g[blockIdx.y];
+    const size_t n = a.n[blockIdx.y], n4 = n / 4;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    const size_t tid = (size_t)blockIdx.x * OPT_THREADS + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * OPT_THREADS;
+    for (size_t i = tid; i < n4; i += stride) {
+        v4f v = ld4_nt(g + 4 * i) * pre;
+        s0 += v.x * v.x; s1 += v.y * v.y; s2 += v.z * v.z; s3 += v.w * v.w;
+    }
+    if (blockIdx.x == 0)
+        for (size_t i = n4 * 4 + threadIdx.x; i < n; i += OPT_THREADS) { float t = g[i] * pre; s0 += t * t; }
+    float s = (s0 + s1) + (s2 + s3);
+#pragma unroll
+    for (int k = 32; k >= 1; k >>= 1) s += __shfl_xor(s, k, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) part[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+template <bool ZERO>
+__global__ __launch_bounds__(OPT_THREADS) void adam_mt_kernel(MtAdam a, float lr, float b1, float b2, float eps,
+                                                              float bc1, float bc2, float scale1,
+                                                              const float *__restrict__ scale2_p) {
+    const size_t n = a.n[blockIdx.y], n4 = n / 4;
+    const size_t i = (size_t)blockIdx.x * OPT_THREADS + threadIdx.x;
+    if (i >= n4 && !(blockIdx.x == 0 && threadIdx.x < n - n4 * 4)) return;
+    float *__restrict__ w = a.w[blockIdx.y], *__restrict__ g = a.g[blockIdx.y];
+    float *__restrict__ m = a.m[blockIdx.y], *__restrict__ v = a.v[blockIdx.y];
+    const float wd = a.wd[blockIdx.y];
+    const float scale2 = scale2_p ? *scale2_p : 1.0f;
+    const float omb1 = 1.0f - b1, omb2 = 1.0f - b2;
+    if (i < n4) {
+        v4f wv = ld4_nt(w + 4 * i), gv = ld4_nt(g + 4 * i), mv = ld4_nt(m + 4 * i), vv = ld4_nt(v + 4 * i);
+        gv = (gv * scale1) * scale2;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float x = wv[j], y = mv[j], z = vv[j];
+            adam1(x, y, z, gv[j], lr, b1, b2, omb1, omb2, eps, wd, bc1, bc2);
+            wv[j] = x; mv[j] = y; vv[j] = z;
+        }
+        st4_nt(w + 4 * i, wv);
+        st4_nt(m + 4 * i, mv);
+        st4_nt(v + 4 * i, vv);
+        if (ZERO) { const v4f z4 = {0.f, 0.f, 0.f, 0.f}; st4_nt(g + 4 * i, z4); }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < n - n4 * 4) {
+        const size_t k = n4 * 4 + threadIdx.x;
+        float gg = (g[k] * scale1) * scale2;
+        adam1(w[k], m[k], v[k], gg, lr, b1, b2, omb1, omb2, eps, wd, bc1, bc2);
+        if (ZERO) g[k] = 0.f;
+    }
+}
+
 }   // namespace
+
+MI355_API int mi355_sumsq_accum_multi_dev(float *acc_dev, const float *const *g, const size_t *n, int count,
+                                          float pre_scale) {
+    if (!mi355_ready("sumsq_accum_multi")) return -1;
+    if (!acc_dev || !g || !n || count <= 0) return mi355_fail("sumsq_accum_multi: bad arguments");
+    for (int i = 0; i < count; i++)
+        if (!g[i] || n[i] == 0 || !aligned16(g[i])) return mi355_fail("sumsq_accum_multi: tensor %d is NULL, empty or not 16-byte aligned", i);
+    for (int i0 = 0; i0 < count; i0 += MT_MAX) {
+        const int k = count - i0 < MT_MAX ? count - i0 : MT_MAX;
+        MtSumsq a = {};
+        size_t nmax = 0;
+        for (int i = 0; i < k; i++) { a.g[i] = g[i0 + i]; a.n[i] = n[i0 + i]; if (n[i0 + i] > nmax) nmax = n[i0 + i]; }
+        size_t blocks = ceil_div(nmax / 4 + 1, (size_t)OPT_THREADS * 4);
+        if (blocks > 1024) blocks = 1024;
+        float *part = (float *)mi355_ws((size_t)k * blocks * sizeof(float));
+        if (!part) return -1;
+        hipLaunchKernelGGL(sumsq_partial_mt_kernel, dim3((unsigned)blocks, (unsigned)k), dim3(OPT_THREADS), 0, g_ctx.stream,
+                           part, a, pre_scale);
+        hipLaunchKernelGGL(sumsq_final_kernel, dim3(1), dim3(1024), 0, g_ctx.stream, acc_dev, part, (int)(k * blocks));
+        LAUNCH_OK("sumsq_accum_multi");
+    }
+    return 0;
+}
+
+MI355_API int mi355_adam_update_multi_dev(float *const *w, float *const *g, float *const *m, float *const *v,
+                                          const size_t *n, const float *wd, int count, int t, float lr, float b1,
+                                          float b2, float eps, float scale1, const float *scale2_dev, int zero_grad) {
+    if (!mi355_ready("adam_update_multi")) return -1;
+    if (!w || !g || !m || !v || !n || !wd || count <= 0 || t < 1) return mi355_fail("adam_update_multi: bad arguments");
+    for (int i = 0; i < count; i++)
+        if (!w[i] || !g[i] || !m[i] || !v[i] || n[i] == 0 || !aligned16(w[i]) || !aligned16(g[i]) || !aligned16(m[i]) ||
+            !aligned16(v[i]))
+            return mi355_fail("adam_update_multi: tensor %d is NULL, empty or not 16-byte aligned", i);
+    const float bc1 = 1.0f - powf(b1, (float)t), bc2 = 1.0f - powf(b2, (float)t);
+    for (int i0 = 0; i0 < count; i0 += MT_MAX) {
+        const int k = count - i0 < MT_MAX ? count - i0 : MT_MAX;
+        MtAdam a = {};
+        size_t nmax = 0;
+        for (int i = 0; i < k; i++) {
+            a.w[i] = w[i0 + i]; a.g[i] = g[i0 + i]; a.m[i] = m[i0 + i]; a.v[i] = v[i0 + i];
+            a.n[i] = n[i0 + i]; a.wd[i] = wd[i0 + i];
+            if (n[i0 + i] > nmax) nmax = n[i0 + i];
+        }
+        const dim3 grid((unsigned)ceil_div(nmax / 4 + 1, (size_t)OPT_THREADS), (unsigned)k);
+        if (zero_grad)
+            hipLaunchKernelGGL((adam_mt_kernel<true>), grid, dim3(OPT_THREADS), 0, g_ctx.stream, a, lr, b1, b2, eps, bc1,
+                               bc2, scale1, scale2_dev);
+        else
+            hipLaunchKernelGGL((adam_mt_kernel<false>), grid, dim3(OPT_THREADS), 0, g_ctx.stream, a, lr, b1, b2, eps, bc1,
+                               bc2, scale1, scale2_dev);
+        LAUNCH_OK("adam_update_multi");
+    }
+    return 0;
+}
 
 MI355_API int mi355_sumsq_accum_dev(float *acc_dev, const float *g, size_t n, float pre_scale) {
     if (!mi355_ready("sumsq_accum")) return -1;

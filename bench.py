@@ -343,6 +343,60 @@ def bench_embed(br, args):
     print(json.dumps(out))
 
 
+def bench_optimizer(br, args):
+    """Optimizer tail of training/training_dynamic/train.m:748-877 on one Qwen3-0.6B layer's matrices
+    (Wq,Wk,Wv,Wo,W1,W2,W3 = 15.7 M parameters) x 8 rotating sets: norm sweep + fused AdamW sweep."""
+    sizes = [2048 * 1024, 1024 * 1024, 1024 * 1024, 1024 * 2048, 3072 * 1024, 1024 * 3072, 3072 * 1024]
+    nset = 8
+    A = br.DevArray
+    sets = []
+    seed = 1
+    for _ in range(nset):
+        ts = []
+        for n in sizes:
+            w, g, m, v = A(n), A(n), A(n), A(n)
+            for buf, std in ((w, 0.02), (g, 1.0), (m, 0.01)):
+                br.check(br.lib.mi355_fill_normal_dev(buf.ptr, n, seed, 0.0, std)); seed += 1
+            br.check(br.lib.mi355_fill_normal_dev(v.ptr, n, seed, 1.0, 0.1)); seed += 1      # positive second moments
+            ts.append((w, g, m, v, n))
+        sets.append(ts)
+    ss, cs = A(1), A(1)
+    gsc = 1.0 / 256.0
+    br.sync()
+
+    import ctypes as C
+    k = len(sizes)
+    arr = lambda ts, j: (C.c_void_p * k)(*[t[j].ptr for t in ts])
+    packs = [(arr(ts, 0), arr(ts, 1), arr(ts, 2), arr(ts, 3)) for ts in sets]
+    narr = (C.c_size_t * k)(*sizes)
+    wdarr = (C.c_float * k)(*([0.1] * k))
+
+    def norm_pass():          # one layer's tensors per launch (mi355_sumsq_accum_multi_dev)
+        for (pw, pg, pm, pv) in packs:
+            br.check(br.lib.mi355_sumsq_accum_multi_dev(ss.ptr, pg, narr, k, gsc))
+
+    def adam_pass():
+        br.check(br.lib.mi355_clip_scale_dev(cs.ptr, ss.ptr, 1.0))
+        for (pw, pg, pm, pv) in packs:
+            br.check(br.lib.mi355_adam_update_multi_dev(pw, pg, pm, pv, narr, wdarr, k, 3, 3e-4, 0.9, 0.95, 1e-8, gsc,
+                                                        cs.ptr, 1))
+
+    for _ in range(args.warmup):
+        norm_pass(); adam_pass()
+    t_n = time_region(br, norm_pass, args.steps) / nset
+    t_a = time_region(br, adam_pass, args.steps) / nset
+    P = sum(sizes)
+    b_n, b_a = 4 * P, 32 * P           # read g | read w,g,m,v + write w,m,v,g(=0)
+    out = {"metric": "optimizer tail (scaled global norm + clip + AdamW + gradient clear), parameters/s",
+           "value": P / ((t_n + t_a) / 1e3), "unit": "parameters/s", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": t_n + t_a, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "one Qwen3-0.6B layer's 7 weight matrices (%d parameters), fp32 w/g/m/v" % P},
+           "ops": [dict(op="sumsq_accum (7 tensors)", ms=t_n, alg_mb=b_n / 1e6, gbs=b_n / t_n / 1e6, frac=b_n / t_n / 1e6 / PEAK_HBM_GBS),
+                   dict(op="adam_update (7 tensors)", ms=t_a, alg_mb=b_a / 1e6, gbs=b_a / t_a / 1e6, frac=b_a / t_a / 1e6 / PEAK_HBM_GBS)]}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -355,8 +409,9 @@ def main():
     ap.add_argument("--fuse", action="store_true",
                     help="run each residual and the RMSNorm after it as one launch (mi355_residual_rmsnorm_fwd_dev)")
     ap.add_argument("--op-reps", type=int, default=3)
-    ap.add_argument("--workload", default="qwen3", choices=["qwen3", "embed"],
-                    help="qwen3 = the headline sweep (default); embed = BASELINE config 2 (its own JSON line)")
+    ap.add_argument("--workload", default="qwen3", choices=["qwen3", "embed", "optimizer"],
+                    help="qwen3 = the headline sweep (default); embed = BASELINE config 2; optimizer = the Adam tail "
+                         "(each prints its own JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path needs no collectives); run with --gpus 1")
@@ -366,6 +421,8 @@ def main():
     dev_name, drv_peak, cus = br.device_info()
     if args.workload == "embed":
         return bench_embed(br, args)
+    if args.workload == "optimizer":
+        return bench_optimizer(br, args)
     cfg = dict(Q3)
     wl = Workload(br, cfg, args.layers, fuse=args.fuse)
     br.check(br.lib.mi355_dw_defer(0 if args.immediate_dw else 1))

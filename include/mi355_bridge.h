@@ -207,6 +207,15 @@ int mi355_adam_update_dev(float *w, float *g, float *m, float *v, size_t n, int 
                           float b2, float eps, float wd, float scale1, const float *scale2_dev,
                           int zero_grad);
 
+/* The same two sweeps over several tensors per launch (the loop updates 9 tensors per layer, train.m:843-852):
+ * host arrays of `count` device pointers / sizes / per-tensor weight decay; tensors must be 16-byte aligned.
+ * Results equal the per-tensor calls (the norm up to summation order). */
+int mi355_sumsq_accum_multi_dev(float *acc_dev, const float *const *g, const size_t *n, int count,
+                                float pre_scale);
+int mi355_adam_update_multi_dev(float *const *w, float *const *g, float *const *m, float *const *v,
+                                const size_t *n, const float *wd, int count, int t, float lr, float b1,
+                                float b2, float eps, float scale1, const float *scale2_dev, int zero_grad);
+
 /* GQA helpers of the dynamic loop — training/training_dynamic/io.h:330-351 (calls at
  * training/training_dynamic/train.m:620-621,653-654).  tile: out[batch][kv_heads*ratio*hd][S] gets each KV
  * head `ratio` times; reduce: out[batch][kv_heads*hd][S] = sum over the `ratio` query heads of each group,

@@ -525,6 +525,37 @@ def test_optimizer_tail(br, n):
     assert cs.numpy()[0] == 1.0
 
 
+def test_optimizer_tail_multi_tensor_equals_per_tensor(br):
+    import ctypes as C
+    sizes = [4096, 1024 * 1024 + 4, 12, 300000] + [2048] * 17                  # more tensors than one launch holds
+    ws = [H.normal(60 + i, n, 0, 0.05) for i, n in enumerate(sizes)]
+    gs = [H.normal(90 + i, n) for i, n in enumerate(sizes)]
+    ms = [H.normal(120 + i, n, 0, 0.01) for i, n in enumerate(sizes)]
+    vs = [np.abs(H.normal(150 + i, n, 0, 0.01)) for i, n in enumerate(sizes)]
+    wds = [0.1 if i % 2 else 0.0 for i in range(len(sizes))]
+    hp = dict(t=4, lr=1e-3, b1=0.9, b2=0.95, eps=1e-8)
+    D = lambda arrs: [dev(br, a) for a in arrs]
+    w1, g1, m1, v1 = D(ws), D(gs), D(ms), D(vs)
+    w2, g2, m2, v2 = D(ws), D(gs), D(ms), D(vs)
+    ss1 = dev(br, np.zeros(1, np.float32)); ss2 = dev(br, np.zeros(1, np.float32))
+    k = len(sizes)
+    parr = lambda ds: (C.c_void_p * k)(*[d.ptr for d in ds])
+    narr = (C.c_size_t * k)(*sizes); wdarr = (C.c_float * k)(*wds)
+    for i in range(k):
+        br.check(br.lib.mi355_sumsq_accum_dev(ss1.ptr, g1[i].ptr, sizes[i], 0.5))
+        br.check(br.lib.mi355_adam_update_dev(w1[i].ptr, g1[i].ptr, m1[i].ptr, v1[i].ptr, sizes[i], hp["t"], hp["lr"],
+                                              hp["b1"], hp["b2"], hp["eps"], wds[i], 0.5, None, 1))
+    br.check(br.lib.mi355_sumsq_accum_multi_dev(ss2.ptr, parr(g2), narr, k, 0.5))
+    br.check(br.lib.mi355_adam_update_multi_dev(parr(w2), parr(g2), parr(m2), parr(v2), narr, wdarr, k, hp["t"], hp["lr"],
+                                                hp["b1"], hp["b2"], hp["eps"], 0.5, None, 1))
+    assert abs(ss1.numpy()[0] - ss2.numpy()[0]) <= 2e-6 * ss1.numpy()[0]
+    for i in range(k):
+        assert np.array_equal(w1[i].numpy(), w2[i].numpy()) and np.array_equal(m1[i].numpy(), m2[i].numpy())
+        assert np.array_equal(v1[i].numpy(), v2[i].numpy()) and not g2[i].numpy().any()
+        rw, rm, rv = O.adam_update(ws[i], gs[i] * np.float32(0.5), ms[i], vs[i], wd=wds[i], **hp)
+        assert H.rel_err(w2[i].numpy(), rw) <= TOL
+
+
 @pytest.mark.parametrize("B,kvh,ratio,hd,S", [(16, 8, 2, 128, 256), (2, 3, 4, 6, 5), (1, 1, 1, 4, 4)])
 def test_gqa_tile_reduce(br, B, kvh, ratio, hd, S):
     k = H.normal(54, (B, kvh * hd, S)); g = H.normal(55, (B, kvh * ratio * hd, S))
