@@ -310,14 +310,15 @@ NormCfg pick_cfg(int C, int S, int batch, bool vec_ok, int max_cap, int max_cap_
     if (!vec_ok) return NormCfg{1, 64, 256, 0};
     if (!lpr_knob && !thr_knob && C >= 512) {
         // Tall tensors, measured on MI355X at C=1024 and 16x256 columns with operands cold in HBM: forward, 64-byte strips in registers of a 16-wave workgroup
-        // 9.6 us; backward, the single-pass register tile 16.3 us against 19.9 us for a two-sweep variant.
+        // 9.6 us; backward, the single-pass register tile with 8 waves 13.9 us, with 4 waves 16.3 us, a two-sweep
+        // 16-wave variant 19.9 us.
         if (!backward) return NormCfg{4, 4, 1024, C <= 2048 ? 8 : 0};
-        if (C <= 1024) return NormCfg{4, 4, 256, 16};
+        if (C <= 1024) return NormCfg{4, 4, 512, 8};
         const long strips8 = (long)ceil_div((size_t)S, 32);
         return NormCfg{4, strips8 * batch >= 128 ? 8 : 4, 1024, 0};
     }
     const int lprs[3] = {16, 8, 4};
-    const int thrs[2] = {256, 1024};
+    const int thrs[3] = {256, 512, 1024};
     const int caps[2] = {8, 16};
     long best_score = -1;
     for (int lpr : lprs) {
@@ -370,6 +371,12 @@ void launch_bwd(float *dx, float *part, const float *dy, const float *x, const f
             case 4160116: FN<4, 16, 256, 16>(__VA_ARGS__); break;                                     \
             case 4160400: FN<4, 16, 1024, 0>(__VA_ARGS__); break;                                     \
             case 4160408: FN<4, 16, 1024, 8>(__VA_ARGS__); break;                                     \
+            case 4040208: FN<4, 4, 512, 8>(__VA_ARGS__); break;                                       \
+            case 4040216: FN<4, 4, 512, 16>(__VA_ARGS__); break;                                      \
+            case 4080208: FN<4, 8, 512, 8>(__VA_ARGS__); break;                                       \
+            case 4080216: FN<4, 8, 512, 16>(__VA_ARGS__); break;                                      \
+            case 4040200: FN<4, 4, 512, 0>(__VA_ARGS__); break;                                       \
+            case 4080200: FN<4, 8, 512, 0>(__VA_ARGS__); break;                                       \
             case 4080100: FN<4, 8, 256, 0>(__VA_ARGS__); break;                                       \
             case 4080108: FN<4, 8, 256, 8>(__VA_ARGS__); break;                                       \
             case 4080116: FN<4, 8, 256, 16>(__VA_ARGS__); break;                                      \
