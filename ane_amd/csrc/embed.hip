@@ -351,6 +351,50 @@ __global__ __launch_bounds__(1024) void seg_sum_kernel(float *__restrict__ dE, c
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Vocabulary compaction (training/training_dynamic/cpu_ops.h:127-148): whole-row copies by index.
+// One workgroup row of 64 lanes x 128 bit covers 1 KiB of a table row.
+// MODE 0: dst[i] = src[idx[i]] (vocab_compact_embed)   MODE 1: dst[idx[i]] = src[i] (vocab_update_full)
+// MODE 2: dst[idx[i]] += src[i] (vocab_scatter_grads; idx holds distinct rows, so no two lanes meet)
+// ---------------------------------------------------------------------------------------------
+template <int MODE, int VEC>
+__global__ __launch_bounds__(256) void rows_by_index_kernel(float *__restrict__ dst, const float *__restrict__ src,
+                                                            const int32_t *__restrict__ idx, int n, int D, int rows_dst,
+                                                            int rows_src) {
+    const int dv = (D + VEC - 1) / VEC;                          // column groups per row
+    const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= (size_t)n * dv) return;
+    const int i = (int)(t / dv), cg = (int)(t - (size_t)i * dv);
+    const int r = idx[i];
+    if (r < 0 || r >= (MODE == 0 ? rows_src : rows_dst)) return;  // an index outside the table is skipped
+    const size_t a = (MODE == 0 ? (size_t)r : (size_t)i) * D + (size_t)cg * VEC;      // source offset
+    const size_t b = (MODE == 0 ? (size_t)i : (size_t)r) * D + (size_t)cg * VEC;      // destination offset
+    if constexpr (VEC == 4) {
+        v4f v = ld4(src + a);
+        if (MODE == 2) v = ld4(dst + b) + v;
+        st4(dst + b, v);
+    } else {
+        float v = src[a];
+        if (MODE == 2) v = dst[b] + v;
+        dst[b] = v;
+    }
+}
+
+template <int MODE>
+int rows_by_index(const char *who, float *dst, const float *src, const int32_t *idx, int n, int D, int rows_dst,
+                  int rows_src) {
+    if (!mi355_ready(who)) return -1;
+    if (!dst || !src || !idx) return mi355_fail("%s: NULL pointer", who);
+    if (n <= 0 || D <= 0 || rows_dst <= 0 || rows_src <= 0) return mi355_fail("%s: bad shape n=%d D=%d", who, n, D);
+    const bool vec = (D % 4 == 0) && aligned16(dst) && aligned16(src);
+    const size_t work = (size_t)n * (vec ? D / 4 : D);
+    const unsigned blocks = (unsigned)ceil_div(work, 256);
+    if (vec) hipLaunchKernelGGL((rows_by_index_kernel<MODE, 4>), dim3(blocks), dim3(256), 0, g_ctx.stream, dst, src, idx, n, D, rows_dst, rows_src);
+    else hipLaunchKernelGGL((rows_by_index_kernel<MODE, 1>), dim3(blocks), dim3(256), 0, g_ctx.stream, dst, src, idx, n, D, rows_dst, rows_src);
+    LAUNCH_OK(who);
+    return 0;
+}
+
 int key_bits(int V) {
     int bits = 1;
     while (bits < 31 && (1L << bits) <= (long)V) bits++;   // keys range over [0, V]
@@ -433,4 +477,19 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
                        rows, seg_start, keys, meta, D, nchunk, long_x, (int)short_blocks);
     LAUNCH_OK("embed_scatter_add segment sums");
     return 0;
+}
+
+MI355_API int mi355_vocab_compact_embed_dev(float *compact, const float *full, const int32_t *compact_to_full, int CV,
+                                            int V, int D) {
+    return rows_by_index<0>("vocab_compact_embed", compact, full, compact_to_full, CV, D, CV, V);
+}
+
+MI355_API int mi355_vocab_update_full_dev(float *full, const float *compact, const int32_t *compact_to_full, int CV,
+                                          int V, int D) {
+    return rows_by_index<1>("vocab_update_full", full, compact, compact_to_full, CV, D, V, CV);
+}
+
+MI355_API int mi355_vocab_scatter_grads_dev(float *full_grad, const float *compact_grad, const int32_t *compact_to_full,
+                                            int CV, int V, int D) {
+    return rows_by_index<2>("vocab_scatter_grads", full_grad, compact_grad, compact_to_full, CV, D, V, CV);
 }

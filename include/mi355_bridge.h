@@ -223,6 +223,19 @@ int mi355_adam_update_multi_dev(float *const *w, float *const *g, float *const *
 int mi355_gqa_tile_dev(float *out, const float *in, int kv_heads, int ratio, int hd, int S, int batch);
 int mi355_gqa_reduce_dev(float *out, const float *in, int kv_heads, int ratio, int hd, int S, int batch);
 
+/* Vocabulary compaction — training/training_dynamic/cpu_ops.h:127-148.  compact_to_full[CV] is the map that
+ * vocab_map_build (cpu_ops.h:103-125, host code, unchanged) produces: distinct row numbers of the full table.
+ *   compact_embed: compact[c] = full[map[c]]           (vocab_compact_embed, cpu_ops.h:127-132)
+ *   update_full:   full[map[c]] = compact[c]           (vocab_update_full,   cpu_ops.h:145-148)
+ *   scatter_grads: full_grad[map[c]] += compact_grad[c] (vocab_scatter_grads, cpu_ops.h:135-142)
+ * Rows are [D] floats; a map entry outside [0,V) is skipped.  Pure copies: bit-exact. */
+int mi355_vocab_compact_embed_dev(float *compact, const float *full, const int32_t *compact_to_full, int CV,
+                                  int V, int D);
+int mi355_vocab_update_full_dev(float *full, const float *compact, const int32_t *compact_to_full, int CV,
+                                int V, int D);
+int mi355_vocab_scatter_grads_dev(float *full_grad, const float *compact_grad, const int32_t *compact_to_full,
+                                  int CV, int V, int D);
+
 /* ------------------------------------------------------------------------------------------
  * Host-pointer drop-ins: the reference signatures verbatim (host float* in, host float* out),
  * so a caller swaps the symbol only.  Each call stages through cached device buffers

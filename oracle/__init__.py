@@ -65,6 +65,11 @@ def _load():
         "orc_embed_backward_batched": (None, [_f32p, _f32p, _i32p, C.c_int, C.c_int, C.c_int, C.c_int]),
         "orc_sumsq_scaled": (C.c_float, [_f32p, C.c_size_t, C.c_float]),
         "orc_clip_scale": (C.c_float, [C.c_float, C.c_float]),
+        "orc_vocab_map_build": (C.c_int, [_i32p, _i32p, np.ctypeslib.ndpointer(dtype=np.uint16, flags="C_CONTIGUOUS"),
+                                          C.c_size_t, C.c_int]),
+        "orc_vocab_compact_embed": (None, [_f32p, _f32p, _i32p, C.c_int, C.c_int]),
+        "orc_vocab_scatter_grads": (None, [_f32p, _f32p, _i32p, C.c_int, C.c_int]),
+        "orc_vocab_update_full": (None, [_f32p, _f32p, _i32p, C.c_int, C.c_int]),
         "orc_recipe_drand48": (None, [C.c_int, C.c_long, _f32p, _f32p, _f32p, C.c_size_t, C.c_int]),
         "orc_now_s": (C.c_double, []),
         "orc_max_threads": (C.c_int, []),
@@ -245,3 +250,30 @@ def sumsq_scaled(g, pre_scale=1.0):
 
 def clip_scale(sumsq, grad_clip):
     return float(lib.orc_clip_scale(sumsq, grad_clip))
+
+
+def vocab_map_build(data, full_vocab):
+    """Returns (full_to_compact [V], compact_to_full [CV])."""
+    data = np.ascontiguousarray(data, np.uint16)
+    f2c = np.empty(full_vocab, np.int32); c2f = np.empty(full_vocab, np.int32)
+    cv = lib.orc_vocab_map_build(f2c, c2f, data, data.size, full_vocab)
+    return f2c, c2f[:cv].copy()
+
+
+def vocab_compact_embed(full, c2f):
+    full = _f32(full); c2f = _i32(c2f)
+    ce = np.empty((c2f.size, full.shape[1]), np.float32)
+    lib.orc_vocab_compact_embed(ce, full, c2f, c2f.size, full.shape[1])
+    return ce
+
+
+def vocab_scatter_grads(full_g, compact_g, c2f):
+    out = _f32(full_g).copy(); c2f = _i32(c2f)
+    lib.orc_vocab_scatter_grads(out, _f32(compact_g), c2f, c2f.size, out.shape[1])
+    return out
+
+
+def vocab_update_full(full, compact, c2f):
+    out = _f32(full).copy(); c2f = _i32(c2f)
+    lib.orc_vocab_update_full(out, _f32(compact), c2f, c2f.size, out.shape[1])
+    return out

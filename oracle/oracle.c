@@ -412,6 +412,40 @@ ORC_API void orc_adam_update(float *w, const float *g, float *m, float *v, size_
     }
 }
 
+/* ---------------------------------------------------------------------------------------------
+ * Vocabulary compaction — training/training_dynamic/cpu_ops.h:96-148.
+ * orc_vocab_map_build returns the compact vocabulary size and fills full_to_compact[V] (-1 = unused)
+ * and compact_to_full[<=V]: used ids get compact ids in ascending id order.
+ * ------------------------------------------------------------------------------------------- */
+ORC_API int orc_vocab_map_build(int *full_to_compact, int *compact_to_full, const uint16_t *data, size_t n_tokens,
+                                int full_vocab) {
+    for (int v = 0; v < full_vocab; v++) full_to_compact[v] = -1;
+    for (size_t i = 0; i < n_tokens; i++) full_to_compact[data[i]] = 0;
+    int cid = 0;
+    for (int v = 0; v < full_vocab; v++) {
+        if (full_to_compact[v] == 0) full_to_compact[v] = cid++;
+        else full_to_compact[v] = -1;
+    }
+    for (int v = 0; v < full_vocab; v++)
+        if (full_to_compact[v] >= 0) compact_to_full[full_to_compact[v]] = v;
+    return cid;
+}
+
+ORC_API void orc_vocab_compact_embed(float *ce, const float *full, const int *compact_to_full, int cv, int dim) {
+    for (int c = 0; c < cv; c++) memcpy(ce + (size_t)c * dim, full + (size_t)compact_to_full[c] * dim, (size_t)dim * 4);
+}
+
+ORC_API void orc_vocab_scatter_grads(float *full_g, const float *compact_g, const int *compact_to_full, int cv, int dim) {
+    for (int c = 0; c < cv; c++) {
+        int fv = compact_to_full[c];
+        for (int d = 0; d < dim; d++) full_g[(size_t)fv * dim + d] += compact_g[(size_t)c * dim + d];
+    }
+}
+
+ORC_API void orc_vocab_update_full(float *full, const float *compact, const int *compact_to_full, int cv, int dim) {
+    for (int c = 0; c < cv; c++) memcpy(full + (size_t)compact_to_full[c] * dim, compact + (size_t)c * dim, (size_t)dim * 4);
+}
+
 /* Global gradient norm pieces — training/training_dynamic/train.m:754-787,806-808: the scale pass
  * g *= gsc followed by vDSP_dotpr(g,g) (order unpublished: 8 strided lanes, as sve), and the clip scale. */
 ORC_API float orc_sumsq_scaled(const float *g, size_t n, float pre_scale) {

@@ -556,6 +556,24 @@ def test_optimizer_tail_multi_tensor_equals_per_tensor(br):
         assert H.rel_err(w2[i].numpy(), rw) <= TOL
 
 
+@pytest.mark.parametrize("V,D,ntok", [(32000, 768, 20000), (300, 6, 500), (1000, 1024, 64)])
+def test_vocab_compaction_bit_exact(br, V, D, ntok):
+    data = H.zipf_ids(45, ntok, V).astype(np.uint16)
+    _, c2f = O.vocab_map_build(data, V)
+    CV = c2f.size
+    E = H.normal(46, (V, D), 0, 0.02); g = H.normal(47, (CV, D)); G0 = H.normal(48, (V, D))
+    Ed, md, gd, Gd = dev(br, E), dev(br, c2f), dev(br, g), dev(br, G0)
+    ce = br.DevArray((CV, D))
+    br.check(br.lib.mi355_vocab_compact_embed_dev(ce.ptr, Ed.ptr, md.ptr, CV, V, D))
+    assert ce.numpy().tobytes() == O.vocab_compact_embed(E, c2f).tobytes()
+    br.check(br.lib.mi355_vocab_scatter_grads_dev(Gd.ptr, gd.ptr, md.ptr, CV, V, D))
+    assert Gd.numpy().tobytes() == O.vocab_scatter_grads(G0, g, c2f).tobytes()
+    new = (ce.numpy() * np.float32(0.5)).astype(np.float32)
+    nd = dev(br, new)
+    br.check(br.lib.mi355_vocab_update_full_dev(Ed.ptr, nd.ptr, md.ptr, CV, V, D))
+    assert Ed.numpy().tobytes() == O.vocab_update_full(E, new, c2f).tobytes()
+
+
 @pytest.mark.parametrize("B,kvh,ratio,hd,S", [(16, 8, 2, 128, 256), (2, 3, 4, 6, 5), (1, 1, 1, 4, 4)])
 def test_gqa_tile_reduce(br, B, kvh, ratio, hd, S):
     k = H.normal(54, (B, kvh * hd, S)); g = H.normal(55, (B, kvh * ratio * hd, S))

@@ -231,6 +231,24 @@ def test_adam_matches_formula():
     assert H.rel_err(m2, m64) < 2e-6 and H.rel_err(v2, v64) < 2e-6 and H.rel_err(w2, w64) < 2e-6
 
 
+def test_vocab_compaction():
+    V, D = 300, 6
+    data = H.zipf_ids(41, 500, V).astype(np.uint16)
+    f2c, c2f = O.vocab_map_build(data, V)
+    used = np.unique(data)
+    assert np.array_equal(c2f, used)                                   # compact ids in ascending id order
+    assert np.array_equal(f2c[used], np.arange(used.size)) and (np.delete(f2c, used) == -1).all()
+    E = H.normal(42, (V, D)); ce = O.vocab_compact_embed(E, c2f)
+    assert np.array_equal(ce, E[used])
+    g = H.normal(43, (used.size, D)); G0 = H.normal(44, (V, D))
+    G1 = O.vocab_scatter_grads(G0, g, c2f)
+    ref = G0.copy(); ref[used] += g
+    assert np.array_equal(G1, ref)
+    E2 = O.vocab_update_full(E, ce * 2, c2f)
+    ref = E.copy(); ref[used] = ce * 2
+    assert np.array_equal(E2, ref)
+
+
 def test_sumsq_and_clip_scale():
     g = H.normal(40, 100003) * 3
     gsc = np.float32(1.0 / 256.0)
