@@ -238,8 +238,11 @@ MI355_API int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float 
     if (!mi355_ready("softmax_ce")) return -1;
     if (!dlogits || !loss_dev || !logits || !targets) return mi355_fail("softmax_ce: NULL pointer");
     if (V <= 0 || S <= 0) return mi355_fail("softmax_ce: bad shape V=%d S=%d", V, S);
-    int rpb = g_ctx.ce_rows > 0 ? g_ctx.ce_rows : 256;
+    // rows per workgroup: about 600 workgroups per column strip (2+ per compute unit), between one and
+    // four 64-row register tiles; 256 rows measured best at V = 151936
+    int rpb = g_ctx.ce_rows > 0 ? g_ctx.ce_rows : (int)ceil_div((size_t)V, 600);
     rpb = (int)ceil_div((size_t)rpb, CE_TILE_ROWS) * CE_TILE_ROWS;
+    if (g_ctx.ce_rows <= 0 && rpb > 4 * CE_TILE_ROWS) rpb = 4 * CE_TILE_ROWS;
     const int nblk = (int)ceil_div((size_t)V, (size_t)rpb);
     const bool vec_ok = (S % 4 == 0) && aligned16(logits) && aligned16(dlogits);
     const int vec = vec_ok ? 4 : 1;

@@ -34,7 +34,11 @@ MEASURED_TRAFFIC_BYTES = {"swiglu_bwd": 251.54e6}
 
 # Qwen3-0.6B (training/training_dynamic/models/qwen3_06b.h:6-16), batch 16
 Q3 = dict(C=1024, H=3072, heads=16, kv_heads=8, hd=128, S=256, batch=16, layers=28, V=151936, theta=1e6,
-          int8_shape=(1024, 4096))
+          int8_shape=(1024, 4096), qk_norm=True, name="qwen3-0.6b")
+# Stories110M (training/training_dynamic/models/stories110m.h:6-16): one sequence per step as the reference
+# runs it, RoPE theta 10000, no QK-norm (BASELINE configs 0 and 1)
+S110 = dict(C=768, H=2048, heads=12, kv_heads=12, hd=64, S=256, batch=1, layers=12, V=32000, theta=1e4,
+            int8_shape=(1024, 4096), qk_norm=False, name="stories110m")
 
 
 def alg_bytes(cfg):
@@ -48,7 +52,7 @@ def alg_bytes(cfg):
         "rmsnorm_fwd": 8 * C * St + 4 * C,
         "rmsnorm_bwd": 12 * C * St + 12 * C,
         "qknorm_rope_fwd": 8 * qkd * St,
-        "qknorm_rope_bwd": 12 * qkd * St,
+        "qknorm_rope_bwd": (12 if cfg["qk_norm"] else 8) * qkd * St,
         "swiglu_fwd": 12 * H * St,
         "swiglu_bwd": 20 * H * St,
         "residual": 12 * C * St,
@@ -105,7 +109,8 @@ class Workload:
         self.scale8 = A(1)
         self.scratch_h = A((B, H, S))          # output of the copy-shaped calibration op only
         self.cos, self.sin = br.rope_tables_dev(S, cfg["hd"], cfg["theta"])
-        self.alpha = float(np.float32(1.0 / np.sqrt(2.0 * cfg["layers"])))   # training/training_dynamic/train.m:188
+        # training/training_dynamic/train.m:188; BASELINE config 1 asks for (2*12)^0.25 at the Stories110M shape
+        self.alpha = float(np.float32((2.0 * 12) ** 0.25 if not cfg["qk_norm"] else 1.0 / np.sqrt(2.0 * cfg["layers"])))
         br.sync()
 
     # ---- single ops on layer buffers d -------------------------------------------------------
@@ -117,6 +122,12 @@ class Workload:
             ck(lib.mi355_rmsnorm_fwd_dev(d["xn"].ptr, d["x"].ptr, d["w_att"].ptr, C, S, B, 1e-5))
         elif name == "rmsnorm_fwd2":
             ck(lib.mi355_rmsnorm_fwd_dev(d["x2n"].ptr, d["x2"].ptr, d["w_ffn"].ptr, C, S, B, 1e-5))
+        elif name == "qknorm_rope_fwd" and not c["qk_norm"]:      # plain RoPE on Q and K
+            ck(lib.mi355_rope_dev(d["q_rot"].ptr, d["k_rot"].ptr, d["q"].ptr, d["k"].ptr, c["heads"], c["kv_heads"], hd,
+                                  S, B, self.cos, self.sin, +1))
+        elif name == "qknorm_rope_bwd" and not c["qk_norm"]:      # rope_backward_inplace on dQ, dK (train.m:659-660)
+            ck(lib.mi355_rope_dev(d["dq"].ptr, d["dk"].ptr, d["gq"].ptr, d["gk"].ptr, c["heads"], c["kv_heads"], hd,
+                                  S, B, self.cos, self.sin, -1))
         elif name == "qknorm_rope_fwd":
             ck(lib.mi355_qknorm_rope_fwd_dev(d["q_rot"].ptr, d["k_rot"].ptr, d["q"].ptr, d["k"].ptr, d["wq"].ptr,
                                              d["wk"].ptr, c["heads"], c["kv_heads"], hd, S, B, self.cos, self.sin, 1e-5))
@@ -238,8 +249,12 @@ def cpu_baseline(br, wl, sample_layers, threads_mt):
         out = {}
         t0 = now()
         out["xn"] = O.rmsnorm(h["x"], h["w_att"], threads=threads)
-        out["q_rot"] = O.qknorm_rope_fwd(h["q"], h["wq"], hd, c["theta"], threads=threads)
-        out["k_rot"] = O.qknorm_rope_fwd(h["k"], h["wk"], hd, c["theta"], threads=threads)
+        if c["qk_norm"]:
+            out["q_rot"] = O.qknorm_rope_fwd(h["q"], h["wq"], hd, c["theta"], threads=threads)
+            out["k_rot"] = O.qknorm_rope_fwd(h["k"], h["wk"], hd, c["theta"], threads=threads)
+        else:
+            out["q_rot"] = O.rope(h["q"], hd, c["theta"], +1, threads=threads)
+            out["k_rot"] = O.rope(h["k"], hd, c["theta"], +1, threads=threads)
         out["x2"] = O.axpby(h["x"], h["o"], wl.alpha, 0, threads=threads)
         out["x2n"] = O.rmsnorm(out["x2"], h["w_ffn"], threads=threads)
         out["gate"] = O.swiglu_fwd(h["h1"], h["h3"], threads=threads)
@@ -248,8 +263,12 @@ def cpu_baseline(br, wl, sample_layers, threads_mt):
             out["xn_next"] = O.rmsnorm(out["x_next"], h["w_att"], threads=threads)
         out["dh1"], out["dh3"] = O.swiglu_bwd(h["dsilu"], h["h1"], h["h3"], threads=threads)
         out["dx2"], out["dw_ffn"] = O.rmsnorm_bwd(h["dx_ffn"], out["x2"], h["w_ffn"], threads=threads)
-        out["dq"], out["dwq"] = O.qknorm_rope_bwd(h["gq"], h["q"], h["wq"], hd, c["theta"], threads=threads)
-        out["dk"], out["dwk"] = O.qknorm_rope_bwd(h["gk"], h["k"], h["wk"], hd, c["theta"], threads=threads)
+        if c["qk_norm"]:
+            out["dq"], out["dwq"] = O.qknorm_rope_bwd(h["gq"], h["q"], h["wq"], hd, c["theta"], threads=threads)
+            out["dk"], out["dwk"] = O.qknorm_rope_bwd(h["gk"], h["k"], h["wk"], hd, c["theta"], threads=threads)
+        else:
+            out["dq"] = O.rope(h["gq"], hd, c["theta"], -1, threads=threads)
+            out["dk"] = O.rope(h["gk"], hd, c["theta"], -1, threads=threads)
         out["dx1"], out["dw_att"] = O.rmsnorm_bwd(h["dx_attn"], h["x"], h["w_att"], threads=threads)
         return now() - t0, out
 
@@ -407,16 +426,18 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--layers", type=int, default=Q3["layers"], help="layers in the sweep (28 = the named workload)")
+    ap.add_argument("--layers", type=int, default=0, help="layers in the sweep (default: the model's, 28 / 12)")
     ap.add_argument("--cpu-layers", type=int, default=28, help="layers in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--immediate-dw", action="store_true",
                     help="reduce weight-gradient partials behind every backward op instead of once per step")
     ap.add_argument("--fuse", action="store_true",
                     help="run each residual and the RMSNorm after it as one launch (mi355_residual_rmsnorm_fwd_dev)")
     ap.add_argument("--op-reps", type=int, default=3)
-    ap.add_argument("--workload", default="qwen3", choices=["qwen3", "embed", "optimizer"],
-                    help="qwen3 = the headline sweep (default); embed = BASELINE config 2; optimizer = the Adam tail "
-                         "(each prints its own JSON line)")
+    ap.add_argument("--workload", default="qwen3", choices=["qwen3", "stories110m", "embed", "optimizer"],
+                    help="qwen3 = the headline sweep (default); stories110m = the same sweep at the Stories110M shape "
+                         "(BASELINE configs 0/1: one [C,256] sequence per op, 12 layers, RoPE without QK-norm); "
+                         "embed = BASELINE config 2; optimizer = the Adam tail (each prints its own JSON line)")
+    ap.add_argument("--batch", type=int, default=0, help="sequences per op (default: 16 for qwen3, 1 for stories110m)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path needs no collectives); run with --gpus 1")
@@ -428,7 +449,11 @@ def main():
         return bench_embed(br, args)
     if args.workload == "optimizer":
         return bench_optimizer(br, args)
-    cfg = dict(Q3)
+    cfg = dict(S110 if args.workload == "stories110m" else Q3)
+    if args.batch > 0:
+        cfg["batch"] = args.batch
+    if args.layers <= 0:
+        args.layers = cfg["layers"]
     wl = Workload(br, cfg, args.layers, fuse=args.fuse)
     br.check(br.lib.mi355_dw_defer(0 if args.immediate_dw else 1))
 
@@ -454,18 +479,22 @@ def main():
                                                                ("softmax_ce", "int8_scale", "int8_quant", "int8_dequant") else 1))
     roofline = dict(bound="hbm", kernel=dom["op"], achieved=dom["gbs"], peak=PEAK_HBM_GBS, unit="GB/s",
                     frac=dom["gbs"] / PEAK_HBM_GBS,
-                    traffic=MEASURED_TRAFFIC_BYTES.get(dom["op"]) if args.layers == Q3["layers"] else None,
+                    traffic=MEASURED_TRAFFIC_BYTES.get(dom["op"]) if (cfg["name"], cfg["batch"]) == ("qwen3-0.6b", 16) else None,
                     traffic_source="profiles/qwen3_sweep_pmc_fetch_write.md", alg_bytes_per_launch=ab[dom["op"]],
                     avg_launch_ms=dom["ms"])
 
     out = {
-        "metric": "layer-op tokens/s at Qwen3-0.6B shape (fused-op HBM GB/s and % of peak in `ops`)",
+        "metric": "layer-op tokens/s at %s shape (fused-op HBM GB/s and %% of peak in `ops`)" % (
+            "Qwen3-0.6B" if cfg["name"] == "qwen3-0.6b" else "Stories110M"),
         "value": tokens / (ms / 1e3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "qwen3-0.6b full-step fused-op sweep (BASELINE config 4): %d layers x 10 ops "
-                               "(batch 16 x S 256, C 1024, H 3072, 16/8 heads x 128) + softmax-CE [151936,256] + "
-                               "INT8 [1024,4096]" % args.layers,
+        "config": {"workload": "%s full-step fused-op sweep%s: %d layers x 10 ops (batch %d x S %d, C %d, H %d, %d/%d "
+                               "heads x %d, %s) + softmax-CE [%d,%d] + INT8 [1024,4096]" % (
+                                   cfg["name"], " (BASELINE config 4)" if cfg["name"] == "qwen3-0.6b" else
+                                   " (BASELINE configs 0/1 shapes)", args.layers, cfg["batch"], cfg["S"], cfg["C"],
+                                   cfg["H"], cfg["heads"], cfg["kv_heads"], cfg["hd"],
+                                   "QK-norm + RoPE" if cfg["qk_norm"] else "RoPE", cfg["V"], cfg["S"]),
                    "layers": args.layers, "tokens_per_step": tokens, "alg_gb_per_step": total_bytes / 1e9,
                    "residual_fused_into_next_rmsnorm": wl.fuse,
                    "weight_gradients": "reduced per op" if args.immediate_dw else "queued, reduced once per step"},
