@@ -421,6 +421,55 @@ def bench_optimizer(br, args):
     print(json.dumps(out))
 
 
+def bench_aux(br, args):
+    """The helpers either side of the hot path at the Qwen3-0.6B shape: GQA tile / reduce
+    (training/training_dynamic/io.h:330-351) on 16 x 256 tokens, and the vocabulary-compaction row copies
+    (training/training_dynamic/cpu_ops.h:127-148) for a 32000-row compact vocabulary of a [151936,1024] table."""
+    c = Q3
+    B, S, hd, kvh, ratio = c["batch"], c["S"], c["hd"], c["kv_heads"], c["heads"] // c["kv_heads"]
+    A = br.DevArray
+    nset = 8
+    ks = [A((B, kvh * hd, S)) for _ in range(nset)]
+    qs = [A((B, kvh * ratio * hd, S)) for _ in range(nset)]
+    for i in range(nset):
+        br.check(br.lib.mi355_fill_normal_dev(ks[i].ptr, ks[i].size, 1 + i, 0.0, 1.0))
+        br.check(br.lib.mi355_fill_normal_dev(qs[i].ptr, qs[i].size, 20 + i, 0.0, 1.0))
+    V, D, CV = c["V"], c["C"], 32000
+    full = A((V, D)); gfull = A((V, D))
+    br.check(br.lib.mi355_fill_normal_dev(full.ptr, full.size, 50, 0.0, 0.02))
+    cmap = np.sort(np.random.default_rng(0).choice(V, CV, replace=False)).astype(np.int32)
+    cmapd = br.DevArray.from_numpy(cmap)
+    comp = [A((CV, D)) for _ in range(4)]
+    br.sync()
+    rows = []
+
+    def add(name, fn, nbytes, n):
+        for _ in range(args.warmup):
+            fn()
+        ms = time_region(br, fn, args.steps) / n
+        rows.append(dict(op=name, ms=ms, alg_mb=nbytes / 1e6, gbs=nbytes / ms / 1e6, frac=nbytes / ms / 1e6 / PEAK_HBM_GBS))
+
+    kb, qb = ks[0].nbytes, qs[0].nbytes
+    add("gqa_tile", lambda: [br.check(br.lib.mi355_gqa_tile_dev(q.ptr, k.ptr, kvh, ratio, hd, S, B)) for q, k in zip(qs, ks)],
+        kb + qb, nset)
+    add("gqa_reduce", lambda: [br.check(br.lib.mi355_gqa_reduce_dev(k.ptr, q.ptr, kvh, ratio, hd, S, B)) for q, k in zip(qs, ks)],
+        kb + qb, nset)
+    rb = CV * D * 4
+    add("vocab_compact_embed", lambda: [br.check(br.lib.mi355_vocab_compact_embed_dev(x.ptr, full.ptr, cmapd.ptr, CV, V, D)) for x in comp],
+        2 * rb, len(comp))
+    add("vocab_scatter_grads", lambda: [br.check(br.lib.mi355_vocab_scatter_grads_dev(gfull.ptr, x.ptr, cmapd.ptr, CV, V, D)) for x in comp],
+        3 * rb, len(comp))
+    add("vocab_update_full", lambda: [br.check(br.lib.mi355_vocab_update_full_dev(full.ptr, x.ptr, cmapd.ptr, CV, V, D)) for x in comp],
+        2 * rb, len(comp))
+    total_ms = sum(r["ms"] for r in rows)
+    print(json.dumps({"metric": "GQA tile/reduce and vocabulary-compaction row copies at the Qwen3-0.6B shape",
+                      "value": sum(r["alg_mb"] for r in rows) / total_ms, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+                      "warmup": args.warmup, "ms_per_step": total_ms, "higher_is_better": True, "scaling": "weak",
+                      "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": "gqa 8->16 heads x 128 on 16x256 tokens; compact vocab 32000 of 151936 x 1024"},
+                      "ops": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -433,7 +482,7 @@ def main():
     ap.add_argument("--fuse", action="store_true",
                     help="run each residual and the RMSNorm after it as one launch (mi355_residual_rmsnorm_fwd_dev)")
     ap.add_argument("--op-reps", type=int, default=3)
-    ap.add_argument("--workload", default="qwen3", choices=["qwen3", "stories110m", "embed", "optimizer"],
+    ap.add_argument("--workload", default="qwen3", choices=["qwen3", "stories110m", "embed", "optimizer", "aux"],
                     help="qwen3 = the headline sweep (default); stories110m = the same sweep at the Stories110M shape "
                          "(BASELINE configs 0/1: one [C,256] sequence per op, 12 layers, RoPE without QK-norm); "
                          "embed = BASELINE config 2; optimizer = the Adam tail (each prints its own JSON line)")
@@ -449,6 +498,8 @@ def main():
         return bench_embed(br, args)
     if args.workload == "optimizer":
         return bench_optimizer(br, args)
+    if args.workload == "aux":
+        return bench_aux(br, args)
     cfg = dict(S110 if args.workload == "stories110m" else Q3)
     if args.batch > 0:
         cfg["batch"] = args.batch
