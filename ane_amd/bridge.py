@@ -79,6 +79,9 @@ SIGNATURES = {
     "mi355_vocab_scatter_grads_dev": (_i, [_p, _p, _p, _i, _i, _i]),
     "mi355_gqa_tile_dev": (_i, [_p, _p, _i, _i, _i, _i, _i]),
     "mi355_gqa_reduce_dev": (_i, [_p, _p, _i, _i, _i, _i, _i]),
+    "mi355_cvt_f32_f16_dev": (_i, [_p, _z, _p, _z, _z, _z]),
+    "mi355_cvt_f16_f32_dev": (_i, [_p, _z, _p, _z, _z, _z]),
+    "mi355_attn_grads_finish_dev": (_i, [_p, _p, _p, _p, _p, _p, _i, _z, _z, _z, _i, _i, _i, _i, _i, _p, _p]),
     "mi355_adam_update": (None, [_p, _p, _p, _p, _z, _i, _f, _f, _f, _f, _f]),
     "mi355_rmsnorm": (None, [_p, _p, _p, _i, _i]),
     "mi355_rmsnorm_bwd": (None, [_p, _p, _p, _p, _p, _i, _i]),

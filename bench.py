@@ -461,8 +461,24 @@ def bench_aux(br, args):
         3 * rb, len(comp))
     add("vocab_update_full", lambda: [br.check(br.lib.mi355_vocab_update_full_dev(full.ptr, x.ptr, cmapd.ptr, CV, V, D)) for x in comp],
         2 * rb, len(comp))
+    # fp16 staging (training/training_dynamic/io.h:33-96) and the chain of train.m:646-660 in one pass
+    heads = kvh * ratio
+    nq = B * heads * hd * S
+    h16 = [A((B, heads * hd, S), np.uint16) for _ in range(nset)]
+    add("cvt_f32_f16", lambda: [br.check(br.lib.mi355_cvt_f32_f16_dev(h.ptr, nq, q.ptr, nq, 1, nq)) for h, q in zip(h16, qs)],
+        6 * nq, nset)
+    add("cvt_f16_f32", lambda: [br.check(br.lib.mi355_cvt_f16_f32_dev(q.ptr, nq, h.ptr, nq, 1, nq)) for h, q in zip(h16, qs)],
+        6 * nq, nset)
+    cosd, sind = br.rope_tables_dev(S, hd, c["theta"])
+    dvs = [A((B, kvh * hd, S)) for _ in range(2)]
+    trip = [(h16[i], h16[i + 1], h16[i + 2]) for i in (0, 3)]
+    add("attn_grads_finish(fp16 in)",
+        lambda: [br.check(br.lib.mi355_attn_grads_finish_dev(qs[j].ptr, ks[j].ptr, dvs[j].ptr, t[0].ptr, t[1].ptr, t[2].ptr, 1,
+                                                             0, 0, 0, heads, kvh, hd, S, B, cosd, sind))
+                 for j, t in enumerate(trip)],
+        3 * 2 * nq + 4 * nq + 2 * kb, len(trip))
     total_ms = sum(r["ms"] for r in rows)
-    print(json.dumps({"metric": "GQA tile/reduce and vocabulary-compaction row copies at the Qwen3-0.6B shape",
+    print(json.dumps({"metric": "GQA tile/reduce, fp16 staging and vocabulary-compaction row copies at the Qwen3-0.6B shape",
                       "value": sum(r["alg_mb"] for r in rows) / total_ms, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
                       "warmup": args.warmup, "ms_per_step": total_ms, "higher_is_better": True, "scaling": "weak",
                       "vs_baseline": None, "dtype": "f32", "data": "synthetic",

@@ -223,6 +223,28 @@ int mi355_adam_update_multi_dev(float *const *w, float *const *g, float *const *
 int mi355_gqa_tile_dev(float *out, const float *in, int kv_heads, int ratio, int hd, int S, int batch);
 int mi355_gqa_reduce_dev(float *out, const float *in, int kv_heads, int ratio, int hd, int S, int batch);
 
+/* fp32 <-> fp16 staging converts — cvt_f32_f16 / cvt_f16_f32, training/training_dynamic/io.h:33-50, as used by
+ * io_write_fp16 / io_read_fp16 / io_write_fp16_at / io_write_dyn / io_read_dyn (io.h:53-96) and the per-kernel
+ * packers (io.h:160-310).  A rectangle of `rows` runs of `cols` contiguous elements; dst_ld / src_ld are the
+ * row pitches in elements (>= cols; equal to cols for one contiguous run).  fp16 values travel as uint16_t bit
+ * patterns (IEEE binary16).  fp32 -> fp16 rounds to nearest even, overflows to infinity and keeps subnormals,
+ * as the reference's vcvt_f16_f32 does. */
+int mi355_cvt_f32_f16_dev(uint16_t *dst, size_t dst_ld, const float *src, size_t src_ld, size_t rows, size_t cols);
+int mi355_cvt_f16_f32_dev(float *dst, size_t dst_ld, const uint16_t *src, size_t src_ld, size_t rows, size_t cols);
+
+/* What the dynamic loop does between the attention backward kernels and the QKV backward —
+ * training/training_dynamic/train.m:646-660: io_read_fp16 of dQ, dK, dV (all at `heads` query heads),
+ * gqa_reduce_kv of dK and dV to `kv_heads`, the copy of dQ, rope_backward_inplace of dQ and dK — in one pass.
+ * Inputs [batch][heads*hd][S], fp16 bit patterns (in_f16 = 1) or fp32 (in_f16 = 0); q/k/v_stride = elements
+ * between consecutive sequences of each input (0 = heads*hd*S, i.e. packed), so that the three may be channel
+ * ranges of larger surfaces.  Outputs fp32: dq [batch][heads*hd][S], dk and dv [batch][kv_heads*hd][S].
+ * cos/sin: tables of mi355_rope_tables(_dev), or both NULL for no rotation.  dq may alias dq_full when fp32.
+ * Results equal the separate calls bit for bit. */
+int mi355_attn_grads_finish_dev(float *dq, float *dk, float *dv, const void *dq_full, const void *dk_full,
+                                const void *dv_full, int in_f16, size_t q_stride, size_t k_stride, size_t v_stride,
+                                int heads, int kv_heads, int hd, int S, int batch, const float *cos_dev,
+                                const float *sin_dev);
+
 /* Vocabulary compaction — training/training_dynamic/cpu_ops.h:127-148.  compact_to_full[CV] is the map that
  * vocab_map_build (cpu_ops.h:103-125, host code, unchanged) produces: distinct row numbers of the full table.
  *   compact_embed: compact[c] = full[map[c]]           (vocab_compact_embed, cpu_ops.h:127-132)

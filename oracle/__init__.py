@@ -13,6 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "liboracle.so")
 
 _f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
+_u16p = np.ctypeslib.ndpointer(dtype=np.uint16, flags="C_CONTIGUOUS")
 _i32p = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
 _i8p = np.ctypeslib.ndpointer(dtype=np.int8, flags="C_CONTIGUOUS")
 
@@ -24,9 +25,16 @@ def build(force=False):
     subprocess.check_call(["make", "-C", _HERE, "liboracle.so"], stdout=subprocess.DEVNULL)
 
 
-def _load():
+def _stale():
     if not os.path.exists(_SO):
-        build()
+        return True
+    built = os.path.getmtime(_SO)
+    return any(os.path.getmtime(os.path.join(_HERE, f)) > built for f in ("oracle.c", "Makefile"))
+
+
+def _load():
+    if _stale():
+        build(force=True)
     lib = C.CDLL(_SO)
     sig = {
         "orc_rmsnorm": (None, [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_float]),
@@ -48,6 +56,8 @@ def _load():
         "orc_int8_dequant": (None, [_f32p, _i8p, C.c_size_t, C.c_float]),
         "orc_gqa_tile": (None, [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int]),
         "orc_gqa_reduce": (None, [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int]),
+        "orc_cvt_f32_f16": (None, [_u16p, C.c_size_t, _f32p, C.c_size_t, C.c_size_t, C.c_size_t]),
+        "orc_cvt_f16_f32": (None, [_f32p, C.c_size_t, _u16p, C.c_size_t, C.c_size_t, C.c_size_t]),
         "orc_adam_update": (None, [_f32p, _f32p, _f32p, _f32p, C.c_size_t, C.c_int, C.c_float,
                                    C.c_float, C.c_float, C.c_float, C.c_float]),
         "orc_rmsnorm_batched": (None, [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int]),
@@ -213,6 +223,22 @@ def int8_dequant(q, scale):
     x = np.empty(q.shape, np.float32)
     lib.orc_int8_dequant(x.reshape(-1), q.reshape(-1), q.size, scale)
     return x
+
+
+def cvt_f32_f16(x):
+    """fp32 -> fp16 bit patterns (uint16), same shape."""
+    x = _f32(x)
+    out = np.empty(x.shape, np.uint16)
+    lib.orc_cvt_f32_f16(out.reshape(-1), x.size, x.reshape(-1), x.size, 1, x.size)
+    return out
+
+
+def cvt_f16_f32(h):
+    """fp16 bit patterns (uint16) -> fp32, same shape."""
+    h = np.ascontiguousarray(h, np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib.orc_cvt_f16_f32(out.reshape(-1), h.size, h.reshape(-1), h.size, 1, h.size)
+    return out
 
 
 def gqa_tile(x, kv_heads, ratio, hd):

@@ -399,6 +399,56 @@ ORC_API void orc_gqa_reduce(float *out, const float *in, int kv_heads, int ratio
 }
 
 /* ---------------------------------------------------------------------------------------------
+ * fp32 <-> fp16 staging converts — training/training_dynamic/io.h:33-50.  The reference converts with the
+ * ARM instructions behind vcvt_f16_f32 / vcvt_f32_f16 (and the scalar _Float16 casts for the tail), which are
+ * IEEE 754 binary32 <-> binary16 conversions in the default rounding mode: nearest even, overflow to
+ * infinity, subnormals produced and accepted.  Restated on the bit patterns; fp16 values are uint16_t.
+ * NaNs come out as quiet NaNs with the top payload bits kept.
+ * ------------------------------------------------------------------------------------------- */
+static uint16_t f32_to_f16_bits(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint32_t sign = (x >> 16) & 0x8000u, mag = x & 0x7fffffffu;
+    if (mag >= 0x7f800000u) return (uint16_t)(sign | 0x7c00u | (mag > 0x7f800000u ? (0x0200u | ((mag >> 13) & 0x3ffu)) : 0));
+    if (mag >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);          /* >= 65520 rounds to infinity */
+    if (mag < 0x33000001u) return (uint16_t)sign;                       /* <= 2^-25 rounds to zero (tie to even) */
+    int e = (int)(mag >> 23) - 127;                                     /* unbiased exponent */
+    uint32_t man = (mag & 0x7fffffu) | 0x800000u;                       /* 24-bit significand */
+    int shift = e >= -14 ? 13 : 13 + (-14 - e);                         /* bits dropped (subnormal: more) */
+    uint32_t kept = man >> shift, rem = man & ((1u << shift) - 1), halfway = 1u << (shift - 1);
+    if (rem > halfway || (rem == halfway && (kept & 1u))) kept++;
+    /* normal: kept has the implicit bit at 2^10; adding the biased exponent minus one lets a carry out of the
+     * significand bump the exponent.  subnormal: exponent field 0 and the same carry trick gives 2^-14. */
+    uint32_t h = e >= -14 ? ((uint32_t)(e + 15 - 1) << 10) + kept : kept;
+    return (uint16_t)(sign | h);
+}
+
+static float f16_bits_to_f32(uint16_t h) {
+    uint32_t sign = ((uint32_t)h & 0x8000u) << 16, ex = (h >> 10) & 0x1fu, man = h & 0x3ffu, x;
+    if (ex == 0x1fu) x = sign | 0x7f800000u | (man ? (0x400000u | (man << 13)) : 0);
+    else if (ex) x = sign | ((ex + 112u) << 23) | (man << 13);
+    else if (!man) x = sign;
+    else {
+        int e = -1;
+        do { man <<= 1; e++; } while (!(man & 0x400u));
+        x = sign | ((uint32_t)(112 - e) << 23) | ((man & 0x3ffu) << 13);
+    }
+    float f;
+    memcpy(&f, &x, 4);
+    return f;
+}
+
+ORC_API void orc_cvt_f32_f16(uint16_t *dst, size_t dst_ld, const float *src, size_t src_ld, size_t rows, size_t cols) {
+    for (size_t r = 0; r < rows; r++)
+        for (size_t c = 0; c < cols; c++) dst[r * dst_ld + c] = f32_to_f16_bits(src[r * src_ld + c]);
+}
+
+ORC_API void orc_cvt_f16_f32(float *dst, size_t dst_ld, const uint16_t *src, size_t src_ld, size_t rows, size_t cols) {
+    for (size_t r = 0; r < rows; r++)
+        for (size_t c = 0; c < cols; c++) dst[r * dst_ld + c] = f16_bits_to_f32(src[r * src_ld + c]);
+}
+
+/* ---------------------------------------------------------------------------------------------
  * Adam / AdamW — training/stories_cpu_ops.h:55-63 (wd = 0) and training_dynamic/cpu_ops.h:56-64.
  * ------------------------------------------------------------------------------------------- */
 ORC_API void orc_adam_update(float *w, const float *g, float *m, float *v, size_t n, int t,

@@ -159,3 +159,17 @@ def np_embed_backward_f32(dE, dx, tokens):
             if 0 <= k < V:
                 dE[k] = dE[k] + dx[b, :, t]
     return dE
+
+
+def f16_boundary_values():
+    """float32 inputs on and around every rounding boundary of binary16."""
+    h = np.arange(0x0000, 0x7c01, dtype=np.uint16).view(np.float16).astype(np.float64)     # all finite halves >= 0, inf
+    mids = (h[:-1] + h[1:]) / 2                                                            # the exact ties
+    mids = mids[np.isfinite(mids)]
+    near = np.concatenate([mids, np.nextafter(mids.astype(np.float32), np.float32(np.inf)),
+                           np.nextafter(mids.astype(np.float32), np.float32(-np.inf))]).astype(np.float32)
+    extra = np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 65536.0, 1e9, np.inf, -np.inf, 2.0 ** -24, 2.0 ** -25,
+                      2.0 ** -25 * 1.0000001, 2.0 ** -26, 1e-40, 5.9604645e-08, 6.1035156e-05, 6.0975552e-05],
+                     np.float32)
+    v = np.concatenate([h[np.isfinite(h)].astype(np.float32), near, extra])
+    return np.concatenate([v, -v])

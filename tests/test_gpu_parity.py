@@ -587,6 +587,126 @@ def test_gqa_tile_reduce(br, B, kvh, ratio, hd, S):
 
 
 # ---------------------------------------------------------------------------------------------
+# fp16 staging converts and the attention-gradient finish
+# ---------------------------------------------------------------------------------------------
+def test_cvt_f16_all_bit_patterns(br):
+    allh = np.arange(65536, dtype=np.uint16)
+    hd_ = dev(br, allh)
+    fd = br.DevArray(allh.shape)
+    br.check(br.lib.mi355_cvt_f16_f32_dev(fd.ptr, allh.size, hd_.ptr, allh.size, 1, allh.size))
+    got, ref = fd.numpy(), O.cvt_f16_f32(allh)
+    nan = np.isnan(ref)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), ref[~nan].view(np.uint32))
+    # and back: every non-NaN half is reproduced
+    bd = br.DevArray(allh.shape, np.uint16)
+    br.check(br.lib.mi355_cvt_f32_f16_dev(bd.ptr, allh.size, fd.ptr, allh.size, 1, allh.size))
+    assert np.array_equal(bd.numpy()[~nan], allh[~nan])
+    assert np.isnan(bd.numpy()[nan].view(np.float16)).all()
+
+
+def test_cvt_f32_f16_rounding_boundaries(br):
+    v = H.f16_boundary_values()
+    rnd = np.random.default_rng(6).integers(0, 2 ** 32, 1 << 20, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    v = np.concatenate([v, rnd[~np.isnan(rnd)]])
+    v = v[:v.size // 8 * 8]
+    vd = dev(br, v)
+    od = br.DevArray(v.shape, np.uint16)
+    br.check(br.lib.mi355_cvt_f32_f16_dev(od.ptr, v.size, vd.ptr, v.size, 1, v.size))
+    assert np.array_equal(od.numpy(), O.cvt_f32_f16(v))
+
+
+@pytest.mark.parametrize("rows,cols,dst_ld,src_ld", [(1024, 256, 256 + 3072, 256), (7, 13, 19, 13), (5, 16, 16, 24),
+                                                     (3, 8, 12, 8)])
+def test_cvt_rectangles(br, rows, cols, dst_ld, src_ld):
+    """The packers write runs of `cols` elements at a row pitch (io_write_dyn: [ic, seq+oc] surfaces)."""
+    src = H.normal(120, (rows, src_ld), 0, 30.0)
+    dst0 = np.random.default_rng(121).integers(0, 65536, (rows, dst_ld)).astype(np.uint16)
+    sd, dd = dev(br, src), dev(br, dst0)
+    br.check(br.lib.mi355_cvt_f32_f16_dev(dd.ptr, dst_ld, sd.ptr, src_ld, rows, cols))
+    want = dst0.copy()
+    want[:, :cols] = O.cvt_f32_f16(src[:, :cols])
+    assert np.array_equal(dd.numpy(), want)                       # converted rectangle, everything else untouched
+    back0 = H.normal(122, (rows, src_ld))
+    bd = dev(br, back0)
+    br.check(br.lib.mi355_cvt_f16_f32_dev(bd.ptr, src_ld, dd.ptr, dst_ld, rows, cols))
+    wantb = back0.copy()
+    wantb[:, :cols] = O.cvt_f16_f32(want[:, :cols])
+    assert np.array_equal(bd.numpy().view(np.uint32), wantb.view(np.uint32))
+
+
+def _finish_reference(dq16, dk16, dv16, heads, kvh, hd, theta, in_f16, rotate=True):
+    """train.m:646-660 with the oracle's pieces: read (convert), reduce dK and dV, copy dQ, un-rotate dQ and dK."""
+    cv = O.cvt_f16_f32 if in_f16 else (lambda a: a)
+    ratio = heads // kvh
+    B = dq16.shape[0]
+    dq = np.stack([cv(dq16[b]) for b in range(B)])
+    dk = np.stack([O.gqa_reduce(cv(dk16[b]), kvh, ratio, hd) for b in range(B)])
+    dv = np.stack([O.gqa_reduce(cv(dv16[b]), kvh, ratio, hd) for b in range(B)])
+    if rotate:
+        dq, dk = O.rope(dq, hd, theta, -1), O.rope(dk, hd, theta, -1)
+    return dq, dk, dv
+
+
+@pytest.mark.parametrize("B,heads,kvh,hd,S,in_f16", [(16, 16, 8, 128, 256, 1), (2, 12, 12, 64, 256, 1),
+                                                      (2, 6, 2, 8, 24, 1), (1, 4, 2, 6, 5, 1), (1, 2, 1, 4, 7, 0),
+                                                      (3, 8, 2, 16, 32, 0)])
+def test_attn_grads_finish_equals_separate_steps(br, B, heads, kvh, hd, S, in_f16):
+    theta = 1e6
+    full = (B, heads * hd, S)
+    src = [H.normal(130 + i, full) for i in range(3)]
+    ins = [O.cvt_f32_f16(a) for a in src] if in_f16 else src
+    ind = [dev(br, a) for a in ins]
+    dq, dk, dv = br.DevArray(full), br.DevArray((B, kvh * hd, S)), br.DevArray((B, kvh * hd, S))
+    cosd, sind = br.rope_tables_dev(S, hd, theta)
+    br.check(br.lib.mi355_attn_grads_finish_dev(dq.ptr, dk.ptr, dv.ptr, ind[0].ptr, ind[1].ptr, ind[2].ptr, in_f16,
+                                                0, 0, 0, heads, kvh, hd, S, B, cosd, sind))
+    rq, rk, rv = _finish_reference(*ins, heads, kvh, hd, theta, in_f16)
+    for got, ref in ((dq, rq), (dk, rk), (dv, rv)):
+        assert np.array_equal(got.numpy().view(np.uint32), ref.view(np.uint32))
+    # equals the library's own separate calls too
+    if not in_f16:
+        k2, q2 = br.DevArray((B, kvh * hd, S)), br.DevArray(full)
+        br.check(br.lib.mi355_gqa_reduce_dev(k2.ptr, ind[1].ptr, kvh, heads // kvh, hd, S, B))
+        br.check(br.lib.mi355_rope_dev(q2.ptr, k2.ptr, ind[0].ptr, k2.ptr, heads, kvh, hd, S, B, cosd, sind, -1))
+        assert np.array_equal(q2.numpy(), dq.numpy()) and np.array_equal(k2.numpy(), dk.numpy())
+
+
+def test_attn_grads_finish_surface_offsets_in_place_and_no_rotation(br):
+    """dQ and dK as channel ranges of one [2*Q_DIM, S] fp16 surface per sequence (the layout the reference reads at
+    train.m:647-648); fp32 in place; NULL tables leave the rotation out."""
+    B, heads, kvh, hd, S, theta = 3, 4, 2, 8, 16, 1e4
+    qd = heads * hd
+    surf = O.cvt_f32_f16(H.normal(140, (B, 2 * qd, S)))
+    dv16 = O.cvt_f32_f16(H.normal(141, (B, qd, S)))
+    sd, vd = dev(br, surf), dev(br, dv16)
+    dq, dk, dv = br.DevArray((B, qd, S)), br.DevArray((B, kvh * hd, S)), br.DevArray((B, kvh * hd, S))
+    cosd, sind = br.rope_tables_dev(S, hd, theta)
+    br.check(br.lib.mi355_attn_grads_finish_dev(dq.ptr, dk.ptr, dv.ptr, sd.ptr, sd.ptr + qd * S * 2, vd.ptr, 1,
+                                                2 * qd * S, 2 * qd * S, 0, heads, kvh, hd, S, B, cosd, sind))
+    rq, rk, rv = _finish_reference(surf[:, :qd], surf[:, qd:], dv16, heads, kvh, hd, theta, 1)
+    assert np.array_equal(dq.numpy(), rq) and np.array_equal(dk.numpy(), rk) and np.array_equal(dv.numpy(), rv)
+
+    src = [H.normal(142 + i, (B, qd, S)) for i in range(3)]
+    qd_, kd_, vd_ = (dev(br, a) for a in src)
+    br.check(br.lib.mi355_attn_grads_finish_dev(qd_.ptr, dk.ptr, dv.ptr, qd_.ptr, kd_.ptr, vd_.ptr, 0, 0, 0, 0, heads,
+                                                kvh, hd, S, B, None, None))
+    rq, rk, rv = _finish_reference(*src, heads, kvh, hd, theta, 0, rotate=False)
+    assert np.array_equal(qd_.numpy(), rq) and np.array_equal(dk.numpy(), rk) and np.array_equal(dv.numpy(), rv)
+
+
+def test_staging_bad_arguments(br):
+    a = br.DevArray(64); h = br.DevArray(64, np.uint16)
+    assert br.lib.mi355_cvt_f32_f16_dev(h.ptr, 4, a.ptr, 8, 2, 8) == -1            # pitch below the run length
+    assert br.lib.mi355_cvt_f16_f32_dev(None, 8, h.ptr, 8, 1, 8) == -1
+    assert br.lib.mi355_attn_grads_finish_dev(a.ptr, a.ptr, a.ptr, a.ptr, a.ptr, a.ptr, 0, 0, 0, 0, 3, 2, 4, 4, 1,
+                                              None, None) == -1                    # heads not a multiple of kv_heads
+    assert br.lib.mi355_attn_grads_finish_dev(a.ptr, a.ptr, a.ptr, a.ptr, a.ptr, a.ptr, 0, 0, 0, 0, 2, 2, 4, 4, 1,
+                                              a.ptr, None) == -1                   # one table only
+    assert "attn_grads_finish" in br.last_error()
+
+
+# ---------------------------------------------------------------------------------------------
 # host-pointer drop-ins (reference signatures) and error behaviour
 # ---------------------------------------------------------------------------------------------
 def _p(a):

@@ -219,6 +219,28 @@ def test_gqa_tile_reduce():
     assert abs(np.vdot(t.astype(np.float64), g) - np.vdot(k.astype(np.float64), r)) < 1e-4
 
 
+def test_fp16_converts_match_ieee_binary16():
+    """cvt_f32_f16 / cvt_f16_f32 (training/training_dynamic/io.h:33-50) are the IEEE conversions; numpy's float16
+    is an independent implementation of the same standard."""
+    allh = np.arange(65536, dtype=np.uint16)
+    f = O.cvt_f16_f32(allh)
+    ref = allh.view(np.float16).astype(np.float32)
+    nan = np.isnan(ref)
+    assert np.array_equal(np.isnan(f), nan)
+    assert np.array_equal(f[~nan].view(np.uint32), ref[~nan].view(np.uint32))              # exact, signed zeros included
+    # every half survives the round trip
+    assert np.array_equal(O.cvt_f32_f16(f[~nan]), allh[~nan])
+
+    v = H.f16_boundary_values()
+    with np.errstate(over="ignore"):
+        assert np.array_equal(O.cvt_f32_f16(v), v.astype(np.float16).view(np.uint16))      # ties, subnormals, overflow
+        rnd = np.random.default_rng(5).integers(0, 2 ** 32, 2_000_000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+        rnd = rnd[~np.isnan(rnd)]
+        assert np.array_equal(O.cvt_f32_f16(rnd), rnd.astype(np.float16).view(np.uint16))
+    got = O.cvt_f32_f16(np.array([np.nan, -np.nan], np.float32)).view(np.float16)
+    assert np.isnan(got).all()
+
+
 def test_adam_matches_formula():
     n = 257
     w = H.normal(17, n); g = H.normal(18, n); m = H.normal(19, n, 0, 0.1); v = np.abs(H.normal(20, n, 0, 0.1))
