@@ -79,6 +79,7 @@ SIGNATURES = {
     "mi355_vocab_scatter_grads_dev": (_i, [_p, _p, _p, _i, _i, _i]),
     "mi355_gqa_tile_dev": (_i, [_p, _p, _i, _i, _i, _i, _i]),
     "mi355_gqa_reduce_dev": (_i, [_p, _p, _i, _i, _i, _i, _i]),
+    "mi355_sgemm_dev": (_i, [_i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _f, _p, _i]),
     "mi355_cvt_f32_f16_dev": (_i, [_p, _z, _p, _z, _z, _z]),
     "mi355_cvt_f16_f32_dev": (_i, [_p, _z, _p, _z, _z, _z]),
     "mi355_attn_grads_finish_dev": (_i, [_p, _p, _p, _p, _p, _p, _i, _z, _z, _z, _i, _i, _i, _i, _i, _p, _p]),

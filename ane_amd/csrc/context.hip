@@ -70,12 +70,14 @@ MI355_API int mi355_init(void) {
 
 void mi355_free_caches(void);   // rope tables, host drop-in staging (other translation units)
 void mi355_dw_free(void);       // queued weight-gradient reductions and their arena
+void mi355_blas_free(void);     // rocBLAS handle of mi355_sgemm_dev
 
 MI355_API void mi355_shutdown(void) {
     if (!g_ctx.ready) return;
     (void)hipDeviceSynchronize();
     mi355_free_caches();
     mi355_dw_free();
+    mi355_blas_free();
     if (g_ctx.ws) (void)hipFree(g_ctx.ws);
     g_ctx = Mi355Ctx{};
 }

@@ -477,13 +477,30 @@ def bench_aux(br, args):
                                                              0, 0, 0, heads, kvh, hd, S, B, cosd, sind))
                  for j, t in enumerate(trip)],
         3 * 2 * nq + 4 * nq + 2 * kb, len(trip))
+    # classifier products on the compact vocabulary (train.m:490-508), fp32 through rocBLAS: flops, not bytes
+    xf, dyc = A((D, S)), A((D, S))
+    br.check(br.lib.mi355_fill_normal_dev(xf.ptr, xf.size, 60, 0.0, 1.0))
+    logit, dlog = A((CV, S)), A((CV, S))
+    br.check(br.lib.mi355_fill_normal_dev(dlog.ptr, dlog.size, 61, 0.0, 1e-3))
+    gemms = []
+
+    def add_gemm(name, fn, flops):
+        for _ in range(max(args.warmup, 2)):
+            fn()
+        ms = time_region(br, fn, args.steps)
+        gemms.append(dict(op=name, ms=ms, gflop=flops / 1e9, tflops=flops / ms / 1e9, frac_fp32_mfma=flops / ms / 1e9 / 157.3))
+
+    fl = 2.0 * CV * D * S
+    add_gemm("sgemm logits[CV,S]=cembed.x", lambda: br.check(br.lib.mi355_sgemm_dev(0, 0, CV, S, D, 1.0, comp[0].ptr, D, xf.ptr, S, 0.0, logit.ptr, S)), fl)
+    add_gemm("sgemm dy[D,S]=cembed^T.dlogits", lambda: br.check(br.lib.mi355_sgemm_dev(1, 0, D, S, CV, 1.0, comp[0].ptr, D, dlog.ptr, S, 0.0, dyc.ptr, S)), fl)
+    add_gemm("sgemm gcembed[CV,D]+=dlogits.x^T", lambda: br.check(br.lib.mi355_sgemm_dev(0, 1, CV, D, S, 1.0, dlog.ptr, S, xf.ptr, S, 1.0, comp[1].ptr, D)), fl)
     total_ms = sum(r["ms"] for r in rows)
     print(json.dumps({"metric": "GQA tile/reduce, fp16 staging and vocabulary-compaction row copies at the Qwen3-0.6B shape",
                       "value": sum(r["alg_mb"] for r in rows) / total_ms, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
                       "warmup": args.warmup, "ms_per_step": total_ms, "higher_is_better": True, "scaling": "weak",
                       "vs_baseline": None, "dtype": "f32", "data": "synthetic",
                       "config": {"workload": "gqa 8->16 heads x 128 on 16x256 tokens; compact vocab 32000 of 151936 x 1024"},
-                      "ops": rows}))
+                      "ops": rows, "gemms": gemms}))
 
 
 def main():

@@ -245,6 +245,14 @@ int mi355_attn_grads_finish_dev(float *dq, float *dk, float *dv, const void *dq_
                                 int heads, int kv_heads, int hd, int S, int batch, const float *cos_dev,
                                 const float *sin_dev);
 
+/* cblas_sgemm(CblasRowMajor, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc) on device memory —
+ * the classifier products training/training_dynamic/train.m:490-491 (logits), :501-502 (dy), :507-508 (gcembed +=)
+ * and the weight-gradient products :577-581, :613, :681-685.  Same argument order and meaning as the cblas call
+ * without the layout argument (always row-major); trans flags take 0/1 or CblasNoTrans/CblasTrans (111/112).
+ * Runs on the bridge stream through rocBLAS, which is opened on the first call. */
+int mi355_sgemm_dev(int trans_a, int trans_b, int M, int N, int K, float alpha, const float *A, int lda,
+                    const float *B, int ldb, float beta, float *C, int ldc);
+
 /* Vocabulary compaction — training/training_dynamic/cpu_ops.h:127-148.  compact_to_full[CV] is the map that
  * vocab_map_build (cpu_ops.h:103-125, host code, unchanged) produces: distinct row numbers of the full table.
  *   compact_embed: compact[c] = full[map[c]]           (vocab_compact_embed, cpu_ops.h:127-132)

@@ -56,6 +56,8 @@ def _load():
         "orc_int8_dequant": (None, [_f32p, _i8p, C.c_size_t, C.c_float]),
         "orc_gqa_tile": (None, [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int]),
         "orc_gqa_reduce": (None, [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int]),
+        "orc_sgemm": (None, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, _f32p, C.c_int, _f32p, C.c_int,
+                             C.c_float, _f32p, C.c_int, C.c_int]),
         "orc_cvt_f32_f16": (None, [_u16p, C.c_size_t, _f32p, C.c_size_t, C.c_size_t, C.c_size_t]),
         "orc_cvt_f16_f32": (None, [_f32p, C.c_size_t, _u16p, C.c_size_t, C.c_size_t, C.c_size_t]),
         "orc_adam_update": (None, [_f32p, _f32p, _f32p, _f32p, C.c_size_t, C.c_int, C.c_float,
@@ -223,6 +225,17 @@ def int8_dequant(q, scale):
     x = np.empty(q.shape, np.float32)
     lib.orc_int8_dequant(x.reshape(-1), q.reshape(-1), q.size, scale)
     return x
+
+
+def sgemm(ta, tb, alpha, A, B, beta=0.0, Cin=None, threads=8):
+    """Row-major C = alpha*op(A)*op(B) + beta*C on 2-D arrays (leading dimensions = row lengths)."""
+    A = _f32(A); B = _f32(B)
+    M, K = (A.shape[1], A.shape[0]) if ta else A.shape
+    N = B.shape[0] if tb else B.shape[1]
+    out = np.zeros((M, N), np.float32) if Cin is None else _f32(Cin).copy()
+    lib.orc_sgemm(int(ta), int(tb), M, N, K, alpha, A.reshape(-1), A.shape[1], B.reshape(-1), B.shape[1], beta,
+                  out.reshape(-1), N, threads)
+    return out
 
 
 def cvt_f32_f16(x):

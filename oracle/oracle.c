@@ -399,6 +399,37 @@ ORC_API void orc_gqa_reduce(float *out, const float *in, int kv_heads, int ratio
 }
 
 /* ---------------------------------------------------------------------------------------------
+ * cblas_sgemm(CblasRowMajor, ...) — training/training_dynamic/train.m:490-508 and the dW products.  The
+ * reference's BLAS is Apple's (closed; its summation order is not documented), so this is the mathematical
+ * product: each C[i][j] accumulated in double over k ascending and rounded to float once.
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_sgemm(int ta, int tb, int M, int N, int K, float alpha, const float *A, int lda, const float *B,
+                       int ldb, float beta, float *C, int ldc, int threads) {
+    if (threads < 1) threads = 1;
+#pragma omp parallel num_threads(threads)
+    {
+        double *row = (double *)malloc((size_t)N * sizeof(double));
+#pragma omp for schedule(static)
+        for (int i = 0; i < M; i++) {
+            for (int j = 0; j < N; j++) row[j] = 0.0;
+            for (int k = 0; k < K; k++) {
+                const double a = ta ? A[(size_t)k * lda + i] : A[(size_t)i * lda + k];
+                if (!tb) {
+                    const float *b = B + (size_t)k * ldb;
+                    for (int j = 0; j < N; j++) row[j] += a * (double)b[j];
+                } else {
+                    for (int j = 0; j < N; j++) row[j] += a * (double)B[(size_t)j * ldb + k];
+                }
+            }
+            float *c = C + (size_t)i * ldc;
+            for (int j = 0; j < N; j++)
+                c[j] = (float)((double)alpha * row[j] + (beta == 0.0f ? 0.0 : (double)beta * (double)c[j]));
+        }
+        free(row);
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
  * fp32 <-> fp16 staging converts — training/training_dynamic/io.h:33-50.  The reference converts with the
  * ARM instructions behind vcvt_f16_f32 / vcvt_f32_f16 (and the scalar _Float16 casts for the tail), which are
  * IEEE 754 binary32 <-> binary16 conversions in the default rounding mode: nearest even, overflow to

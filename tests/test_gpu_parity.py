@@ -707,6 +707,47 @@ def test_staging_bad_arguments(br):
 
 
 # ---------------------------------------------------------------------------------------------
+# cblas_sgemm call sites (classifier, weight gradients)
+# ---------------------------------------------------------------------------------------------
+def test_sgemm_classifier_products(br):
+    """The three classifier products of train.m:490-508 at a compact-vocabulary shape."""
+    CV, D, S = 4096, 1024, 256
+    cembed = H.normal(160, (CV, D), 0, 0.02); x = H.normal(161, (D, S)); dlog = H.normal(162, (CV, S), 0, 1e-3)
+    g0 = H.normal(163, (CV, D), 0, 1e-3)
+    ed, xd, dd, gd = dev(br, cembed), dev(br, x), dev(br, dlog), dev(br, g0)
+    logits, dy = br.DevArray((CV, S)), br.DevArray((D, S))
+    br.check(br.lib.mi355_sgemm_dev(111, 111, CV, S, D, 1.0, ed.ptr, D, xd.ptr, S, 0.0, logits.ptr, S))
+    br.check(br.lib.mi355_sgemm_dev(112, 111, D, S, CV, 1.0, ed.ptr, D, dd.ptr, S, 0.0, dy.ptr, S))
+    br.check(br.lib.mi355_sgemm_dev(111, 112, CV, D, S, 1.0, dd.ptr, S, xd.ptr, S, 1.0, gd.ptr, D))
+    assert H.rel_err(logits.numpy(), O.sgemm(0, 0, 1.0, cembed, x)) <= TOL
+    assert H.rel_err(dy.numpy(), O.sgemm(1, 0, 1.0, cembed, dlog)) <= TOL
+    assert H.rel_err(gd.numpy(), O.sgemm(0, 1, 1.0, dlog, x, 1.0, g0)) <= TOL
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+def test_sgemm_pitched_operands(br, ta, tb):
+    M, N, K, pad = 45, 70, 33, 5
+    A = H.normal(170, ((K, M + pad) if ta else (M, K + pad))); B = H.normal(171, ((N, K + pad) if tb else (K, N + pad)))
+    C0 = H.normal(172, (M, N + pad))
+    ad, bd, cd = dev(br, A), dev(br, B), dev(br, C0)
+    br.check(br.lib.mi355_sgemm_dev(ta, tb, M, N, K, 0.5, ad.ptr, A.shape[1], bd.ptr, B.shape[1], 2.0, cd.ptr, N + pad))
+    Ao = A[:, :M] if ta else A[:, :K]; Bo = B[:, :K] if tb else B[:, :N]
+    want = C0.copy()
+    want[:, :N] = O.sgemm(ta, tb, 0.5, Ao, Bo, 2.0, C0[:, :N])
+    got = cd.numpy()
+    assert H.rel_err(got[:, :N], want[:, :N]) <= TOL
+    assert np.array_equal(got[:, N:], C0[:, N:])                          # padding columns untouched
+
+
+def test_sgemm_bad_arguments(br):
+    a = br.DevArray(64)
+    assert br.lib.mi355_sgemm_dev(0, 0, 4, 4, 4, 1.0, a.ptr, 3, a.ptr, 4, 0.0, a.ptr, 4) == -1
+    assert br.lib.mi355_sgemm_dev(2, 0, 4, 4, 4, 1.0, a.ptr, 4, a.ptr, 4, 0.0, a.ptr, 4) == -1
+    assert br.lib.mi355_sgemm_dev(0, 0, 0, 4, 4, 1.0, a.ptr, 4, a.ptr, 4, 0.0, a.ptr, 4) == -1
+    assert "sgemm" in br.last_error()
+
+
+# ---------------------------------------------------------------------------------------------
 # host-pointer drop-ins (reference signatures) and error behaviour
 # ---------------------------------------------------------------------------------------------
 def _p(a):

@@ -241,6 +241,17 @@ def test_fp16_converts_match_ieee_binary16():
     assert np.isnan(got).all()
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+def test_sgemm_is_the_row_major_product(ta, tb):
+    M, N, K = 37, 29, 53
+    A = H.normal(150, (K, M) if ta else (M, K)); B = H.normal(151, (N, K) if tb else (K, N)); C0 = H.normal(152, (M, N))
+    ref = 0.75 * ((A.T if ta else A).astype(np.float64) @ (B.T if tb else B).astype(np.float64)) - 0.5 * C0
+    got = O.sgemm(ta, tb, 0.75, A, B, -0.5, C0)
+    assert H.rel_err(got, ref) < 2e-7                                   # one rounding of the exact value
+    # beta = 0 must not read C (cblas semantics): NaNs in C are overwritten
+    assert np.isfinite(O.sgemm(ta, tb, 1.0, A, B, 0.0, np.full((M, N), np.nan, np.float32))).all()
+
+
 def test_adam_matches_formula():
     n = 257
     w = H.normal(17, n); g = H.normal(18, n); m = H.normal(19, n, 0, 0.1); v = np.abs(H.normal(20, n, 0, 0.1))
