@@ -724,6 +724,39 @@ def test_sgemm_classifier_products(br):
     assert H.rel_err(gd.numpy(), O.sgemm(0, 1, 1.0, dlog, x, 1.0, g0)) <= TOL
 
 
+def test_classifier_head_chain_stays_on_device(br):
+    """train.m:485-515 with every stage on the device: final RMSNorm, logits product, softmax-CE with the loss
+    scale folded in, the two backward products, RMSNorm backward.  Each stage is checked against the oracle fed
+    with the device result of the stage before it."""
+    CV, D, S, loss_scale = 4099, 768, 256, 256.0
+    x_cur = H.normal(180, (D, S)); w = H.normal(181, D, 1.0, 0.02); cembed = H.normal(182, (CV, D), 0, 0.02)
+    tgt = np.random.default_rng(183).integers(0, CV, S).astype(np.int32)
+    gce0 = H.normal(184, (CV, D), 0, 1e-3); grms0 = H.normal(185, D, 0, 1e-3)
+    xd, wd, ed, td, gced, grmsd = (dev(br, a) for a in (x_cur, w, cembed, tgt, gce0, grms0))
+    xf, logits, dlog, lossd = br.DevArray((D, S)), br.DevArray((CV, S)), br.DevArray((CV, S)), br.DevArray(1)
+    dy, dx = br.DevArray((D, S)), br.DevArray((D, S))
+    L = br.lib
+    br.check(L.mi355_rmsnorm_fwd_dev(xf.ptr, xd.ptr, wd.ptr, D, S, 1, 1e-5))
+    br.check(L.mi355_sgemm_dev(111, 111, CV, S, D, 1.0, ed.ptr, D, xf.ptr, S, 0.0, logits.ptr, S))
+    br.check(L.mi355_softmax_ce_dev(dlog.ptr, lossd.ptr, logits.ptr, td.ptr, CV, S, loss_scale))
+    br.check(L.mi355_sgemm_dev(112, 111, D, S, CV, 1.0, ed.ptr, D, dlog.ptr, S, 0.0, dy.ptr, S))
+    br.check(L.mi355_sgemm_dev(111, 112, CV, D, S, 1.0, dlog.ptr, S, xf.ptr, S, 1.0, gced.ptr, D))
+    br.check(L.mi355_rmsnorm_bwd_dev(dx.ptr, grmsd.ptr, dy.ptr, xd.ptr, wd.ptr, D, S, 1, 1e-5, 0))
+    g_xf, g_logits, g_dlog, g_dy = xf.numpy(), logits.numpy(), dlog.numpy(), dy.numpy()
+    assert H.rel_err(g_xf, O.rmsnorm(x_cur, w)) <= TOL
+    assert H.rel_err(g_logits, O.sgemm(0, 0, 1.0, cembed, g_xf)) <= TOL
+    r_loss, r_dlog = O.cross_entropy(g_logits, tgt, grad_scale=loss_scale)
+    assert abs(float(lossd.numpy()[0]) - r_loss) <= TOL * abs(r_loss) and H.rel_err(g_dlog, r_dlog) <= TOL
+    assert H.rel_err(g_dy, O.sgemm(1, 0, 1.0, cembed, g_dlog)) <= TOL
+    assert H.rel_err(gced.numpy(), O.sgemm(0, 1, 1.0, g_dlog, g_xf, 1.0, gce0)) <= TOL
+    r_dx, r_grms = O.rmsnorm_bwd(g_dy, x_cur, w, dw=grms0)
+    assert H.rel_err(dx.numpy(), r_dx) <= TOL and H.rel_err(grmsd.numpy(), r_grms) <= TOL
+    # end to end against the all-oracle chain: error compounds over six stages, so a looser bound
+    o_xf = O.rmsnorm(x_cur, w); o_loss, o_dlog = O.cross_entropy(O.sgemm(0, 0, 1.0, cembed, o_xf), tgt, grad_scale=loss_scale)
+    o_dx, _ = O.rmsnorm_bwd(O.sgemm(1, 0, 1.0, cembed, o_dlog), x_cur, w, dw=grms0)
+    assert H.rel_err(dx.numpy(), o_dx) <= 1e-4 and abs(float(lossd.numpy()[0]) - o_loss) <= 1e-5 * abs(o_loss)
+
+
 @pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
 def test_sgemm_pitched_operands(br, ta, tb):
     M, N, K, pad = 45, 70, 33, 5
