@@ -26,6 +26,20 @@ _p = C.c_void_p
 _i = C.c_int
 _f = C.c_float
 _z = C.c_size_t
+_u64 = C.c_uint64
+_s = C.c_char_p
+
+
+class CkptHdr(C.Structure):
+    """The 96-byte checkpoint header (``mi355_ckpt_hdr``)."""
+    _fields_ = ([(n, C.c_int) for n in ("magic", "version", "step", "total_steps", "n_layers", "vocab_size", "dim",
+                                         "hidden_dim", "n_heads", "seq_len")] +
+                [("lr", C.c_float), ("loss", C.c_float)] +
+                [(n, C.c_double) for n in ("cum_compile", "cum_train", "cum_wall")] +
+                [(n, C.c_int) for n in ("cum_steps", "cum_batches", "adam_t", "kv_heads", "head_dim", "q_dim")])
+
+
+CK_TENSORS = ("WQ", "WK", "WV", "WO", "W1", "W2", "W3", "RMS_ATT", "RMS_FFN", "RMS_FINAL", "EMBED")
 
 # name -> (restype, argtypes); every symbol include/mi355_bridge.h declares
 SIGNATURES = {
@@ -79,6 +93,12 @@ SIGNATURES = {
     "mi355_vocab_scatter_grads_dev": (_i, [_p, _p, _p, _i, _i, _i]),
     "mi355_gqa_tile_dev": (_i, [_p, _p, _i, _i, _i, _i, _i]),
     "mi355_gqa_reduce_dev": (_i, [_p, _p, _i, _i, _i, _i, _i]),
+    "mi355_ckpt_read_header": (_i, [_s, C.POINTER(CkptHdr)]),
+    "mi355_ckpt_locate": (_i, [C.POINTER(CkptHdr), _i, _i, _i, C.POINTER(_u64), C.POINTER(_u64)]),
+    "mi355_ckpt_file_bytes": (_u64, [C.POINTER(CkptHdr)]),
+    "mi355_ckpt_create": (_i, [_s, C.POINTER(CkptHdr)]),
+    "mi355_ckpt_load_dev": (_i, [_s, _u64, _p, _u64]),
+    "mi355_ckpt_store_dev": (_i, [_s, _u64, _p, _u64]),
     "mi355_sgemm_dev": (_i, [_i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _f, _p, _i]),
     "mi355_cvt_f32_f16_dev": (_i, [_p, _z, _p, _z, _z, _z]),
     "mi355_cvt_f16_f32_dev": (_i, [_p, _z, _p, _z, _z, _z]),

@@ -71,6 +71,7 @@ MI355_API int mi355_init(void) {
 void mi355_free_caches(void);   // rope tables, host drop-in staging (other translation units)
 void mi355_dw_free(void);       // queued weight-gradient reductions and their arena
 void mi355_blas_free(void);     // rocBLAS handle of mi355_sgemm_dev
+void mi355_ckpt_free(void);     // pinned staging buffer of the checkpoint reader/writer
 
 MI355_API void mi355_shutdown(void) {
     if (!g_ctx.ready) return;
@@ -78,6 +79,7 @@ MI355_API void mi355_shutdown(void) {
     mi355_free_caches();
     mi355_dw_free();
     mi355_blas_free();
+    mi355_ckpt_free();
     if (g_ctx.ws) (void)hipFree(g_ctx.ws);
     g_ctx = Mi355Ctx{};
 }

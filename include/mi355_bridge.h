@@ -253,6 +253,35 @@ int mi355_attn_grads_finish_dev(float *dq, float *dk, float *dv, const void *dq_
 int mi355_sgemm_dev(int trans_a, int trans_b, int M, int N, int K, float alpha, const float *A, int lda,
                     const float *B, int ldb, float beta, float *C, int ldc);
 
+/* Checkpoints of the two big loops — header CkptHdr training/stories_config.h:90-105 (version 2) and
+ * training/training_dynamic/config.h:78-86 (version 4: the trailing pad carries the GQA fields); tensor order of
+ * save_checkpoint / load_checkpoint training/train_large.m:110-181, training/training_dynamic/train.m:104-172
+ * (the dashboard reads the same layout, training/dashboard.py:141-174).  The struct below IS the 96 on-disk
+ * bytes.  read_header / locate / file_bytes / create are host-only and need no GPU; load / store move one
+ * tensor between the file and device memory on the bridge stream and return when it is done. */
+typedef struct mi355_ckpt_hdr {
+    int magic, version, step, total_steps;                 /* magic 0x424C5A54, version 2 or 4 */
+    int n_layers, vocab_size, dim, hidden_dim, n_heads, seq_len;
+    float lr, loss;
+    double cum_compile, cum_train, cum_wall;
+    int cum_steps, cum_batches, adam_t;
+    int kv_heads, head_dim, q_dim;                         /* version 4; zero padding in version 2 */
+} mi355_ckpt_hdr;
+enum { MI355_CK_WQ = 0, MI355_CK_WK, MI355_CK_WV, MI355_CK_WO, MI355_CK_W1, MI355_CK_W2, MI355_CK_W3,
+       MI355_CK_RMS_ATT, MI355_CK_RMS_FFN,                 /* per layer */
+       MI355_CK_RMS_FINAL, MI355_CK_EMBED };               /* once per file (layer argument ignored) */
+enum { MI355_CK_WEIGHT = 0, MI355_CK_ADAM_M = 1, MI355_CK_ADAM_V = 2 };
+/* 0, or -1 when the file is missing, short, or not a version 2 / 4 checkpoint (load_checkpoint's `return false`). */
+int mi355_ckpt_read_header(const char *path, mi355_ckpt_hdr *hdr);
+/* Byte offset in the file and element count of one tensor (part: the weight or its Adam m / v). */
+int mi355_ckpt_locate(const mi355_ckpt_hdr *hdr, int layer, int tensor, int part, uint64_t *byte_offset,
+                      uint64_t *count);
+uint64_t mi355_ckpt_file_bytes(const mi355_ckpt_hdr *hdr);                 /* 0 on a bad header */
+/* Writes the header and sizes the file; tensors are then stored in any order. */
+int mi355_ckpt_create(const char *path, const mi355_ckpt_hdr *hdr);
+int mi355_ckpt_load_dev(const char *path, uint64_t byte_offset, float *dst_dev, uint64_t count);
+int mi355_ckpt_store_dev(const char *path, uint64_t byte_offset, const float *src_dev, uint64_t count);
+
 /* Vocabulary compaction — training/training_dynamic/cpu_ops.h:127-148.  compact_to_full[CV] is the map that
  * vocab_map_build (cpu_ops.h:103-125, host code, unchanged) produces: distinct row numbers of the full table.
  *   compact_embed: compact[c] = full[map[c]]           (vocab_compact_embed, cpu_ops.h:127-132)

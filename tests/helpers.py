@@ -173,3 +173,54 @@ def f16_boundary_values():
                      np.float32)
     v = np.concatenate([h[np.isfinite(h)].astype(np.float32), near, extra])
     return np.concatenate([v, -v])
+
+
+# ---- checkpoints: the file as save_checkpoint writes it, and the offsets as the dashboard reads it ----
+CKPT_MAGIC = 0x424C5A54
+
+
+def ckpt_sizes(cfg):
+    """Element counts of the nine per-layer tensors in file order (train.m:118-122 of the dynamic loop)."""
+    dim, hid, qd, kvd = cfg["dim"], cfg["hidden"], cfg["q_dim"], cfg["kv_dim"]
+    return [qd * dim, kvd * dim, kvd * dim, dim * qd, hid * dim, dim * hid, hid * dim, dim, dim]
+
+
+def ckpt_header_bytes(cfg, version, step=7, total_steps=100, lr=3e-4, loss=2.5, adam_t=9):
+    import struct
+    tail = (cfg["kv_heads"], cfg["head_dim"], cfg["q_dim"]) if version == 4 else (0, 0, 0)
+    return struct.pack("<10i2f3d3i3i", CKPT_MAGIC, version, step, total_steps, cfg["layers"], cfg["vocab"], cfg["dim"],
+                       cfg["hidden"], cfg["heads"], cfg["seq"], lr, loss, 1.5, 2.5, 3.5, 11, 12, adam_t, *tail)
+
+
+def ckpt_write_like_reference(path, cfg, version, seed=0):
+    """Writes header + tensors with sequential writes in save_checkpoint's order; returns {(layer, tensor, part): array}."""
+    rng = np.random.default_rng(seed)
+    tensors = {}
+    with open(path, "wb") as f:
+        f.write(ckpt_header_bytes(cfg, version))
+        sizes = ckpt_sizes(cfg)
+        for L in range(cfg["layers"]):
+            for t, n in enumerate(sizes):                       # the nine weights
+                a = rng.standard_normal(n).astype(np.float32); tensors[(L, t, 0)] = a; f.write(a.tobytes())
+            for t, n in enumerate(sizes):                       # then (m, v) of each
+                for part in (1, 2):
+                    a = rng.standard_normal(n).astype(np.float32); tensors[(L, t, part)] = a; f.write(a.tobytes())
+        for t, n in ((9, cfg["dim"]), (10, cfg["vocab"] * cfg["dim"])):
+            for part in (0, 1, 2):
+                a = rng.standard_normal(n).astype(np.float32); tensors[(0, t, part)] = a; f.write(a.tobytes())
+    return tensors
+
+
+def ckpt_weight_offsets_like_dashboard(cfg):
+    """Byte offsets of the weights as training/dashboard.py:141-174 walks the file: 96-byte header, nine weights
+    per layer, a seek over the layer's Adam block, rms_final, a seek over its Adam pair, embed."""
+    sizes = ckpt_sizes(cfg)
+    adam_per_layer = 2 * sum(sizes)
+    off, out = 96, {}
+    for L in range(cfg["layers"]):
+        for t, n in enumerate(sizes):
+            out[(L, t)] = off; off += 4 * n
+        off += 4 * adam_per_layer
+    out[(0, 9)] = off; off += 4 * cfg["dim"] + 4 * 2 * cfg["dim"]
+    out[(0, 10)] = off
+    return out

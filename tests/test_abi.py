@@ -73,3 +73,64 @@ def test_product_does_not_touch_the_oracle():
                     if re.search(r"\boracle\b|liboracle|orc_", t):
                         bad.append(os.path.join(dp, fn))
     assert not bad, bad
+
+
+# ---- checkpoint header and index: host-only code, no GPU needed ----
+CK_GQA = dict(layers=3, vocab=101, dim=64, hidden=160, heads=4, kv_heads=2, head_dim=24, q_dim=96, kv_dim=48, seq=32)
+CK_MHA = dict(layers=2, vocab=77, dim=48, hidden=128, heads=4, kv_heads=4, head_dim=12, q_dim=48, kv_dim=48, seq=16)
+
+
+def _locate(br, hdr, layer, tensor, part):
+    off, cnt = ctypes.c_uint64(), ctypes.c_uint64()
+    assert br.lib.mi355_ckpt_locate(ctypes.byref(hdr), layer, tensor, part, ctypes.byref(off), ctypes.byref(cnt)) == 0
+    return off.value, cnt.value
+
+
+def test_checkpoint_header_and_index_match_the_reference_layout(tmp_path):
+    import ane_amd.bridge as br
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import helpers as H
+    assert ctypes.sizeof(br.CkptHdr) == 96 == len(H.ckpt_header_bytes(CK_GQA, 4))
+    for cfg, version in ((CK_GQA, 4), (CK_MHA, 2)):
+        path = str(tmp_path / ("ck%d.bin" % version))
+        tensors = H.ckpt_write_like_reference(path, cfg, version)
+        hdr = br.CkptHdr()
+        assert br.lib.mi355_ckpt_read_header(path.encode(), ctypes.byref(hdr)) == 0
+        assert (hdr.magic, hdr.version, hdr.step, hdr.total_steps, hdr.adam_t) == (H.CKPT_MAGIC, version, 7, 100, 9)
+        assert (hdr.n_layers, hdr.vocab_size, hdr.dim, hdr.hidden_dim, hdr.n_heads, hdr.seq_len) == \
+            (cfg["layers"], cfg["vocab"], cfg["dim"], cfg["hidden"], cfg["heads"], cfg["seq"])
+        assert abs(hdr.lr - 3e-4) < 1e-9 and hdr.loss == 2.5 and (hdr.cum_compile, hdr.cum_train, hdr.cum_wall) == (1.5, 2.5, 3.5)
+        assert (hdr.cum_steps, hdr.cum_batches) == (11, 12)
+        assert br.lib.mi355_ckpt_file_bytes(ctypes.byref(hdr)) == os.path.getsize(path)
+        raw = open(path, "rb").read()
+        for (L, t, part), a in tensors.items():                              # every tensor sits where locate says
+            off, cnt = _locate(br, hdr, L, t, part)
+            assert cnt == a.size and raw[off:off + 4 * cnt] == a.tobytes(), (L, t, part)
+        for (L, t), off in H.ckpt_weight_offsets_like_dashboard(cfg).items():   # and where the dashboard seeks
+            assert _locate(br, hdr, L, t, 0)[0] == off
+        # create: same header bytes, same file size
+        out = str(tmp_path / ("new%d.bin" % version))
+        assert br.lib.mi355_ckpt_create(out.encode(), ctypes.byref(hdr)) == 0
+        assert os.path.getsize(out) == os.path.getsize(path) and open(out, "rb").read(96) == raw[:96]
+
+
+def test_checkpoint_rejects_foreign_files(tmp_path):
+    import ane_amd.bridge as br
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import helpers as H
+    hdr = br.CkptHdr()
+    assert br.lib.mi355_ckpt_read_header(str(tmp_path / "missing.bin").encode(), ctypes.byref(hdr)) == -1
+    short = tmp_path / "short.bin"; short.write_bytes(b"\0" * 40)
+    assert br.lib.mi355_ckpt_read_header(str(short).encode(), ctypes.byref(hdr)) == -1
+    good = bytearray(H.ckpt_header_bytes(CK_GQA, 4))
+    for pos, val in ((0, b"\x01\x02\x03\x04"), (4, (3).to_bytes(4, "little"))):     # magic, version 3
+        bad = bytearray(good); bad[pos:pos + 4] = val
+        p = tmp_path / ("bad%d.bin" % pos); p.write_bytes(bytes(bad))
+        assert br.lib.mi355_ckpt_read_header(str(p).encode(), ctypes.byref(hdr)) == -1
+    assert "ckpt" in br.last_error()
+    assert br.lib.mi355_ckpt_file_bytes(ctypes.byref(br.CkptHdr())) == 0
+    hdr = br.CkptHdr.from_buffer_copy(bytes(good))
+    off, cnt = ctypes.c_uint64(), ctypes.c_uint64()
+    assert br.lib.mi355_ckpt_locate(ctypes.byref(hdr), 3, 0, 0, ctypes.byref(off), ctypes.byref(cnt)) == -1   # layer 3 of 3
+    assert br.lib.mi355_ckpt_locate(ctypes.byref(hdr), 0, 11, 0, ctypes.byref(off), ctypes.byref(cnt)) == -1
+    assert br.lib.mi355_ckpt_locate(ctypes.byref(hdr), 0, 0, 3, ctypes.byref(off), ctypes.byref(cnt)) == -1

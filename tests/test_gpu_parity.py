@@ -781,6 +781,34 @@ def test_sgemm_bad_arguments(br):
 
 
 # ---------------------------------------------------------------------------------------------
+# checkpoints: file <-> device memory
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("version", [4, 2])
+def test_checkpoint_load_store_round_trip(br, tmp_path, version):
+    import ctypes
+    cfg = dict(layers=2, vocab=300, dim=64, hidden=160, heads=4, kv_heads=2 if version == 4 else 4,
+               head_dim=24 if version == 4 else 16, q_dim=96 if version == 4 else 64, kv_dim=48 if version == 4 else 64,
+               seq=32)
+    src = str(tmp_path / "src.bin"); dst = str(tmp_path / "dst.bin")
+    tensors = H.ckpt_write_like_reference(src, cfg, version, seed=3)
+    hdr = br.CkptHdr()
+    br.check(br.lib.mi355_ckpt_read_header(src.encode(), ctypes.byref(hdr)))
+    br.check(br.lib.mi355_ckpt_create(dst.encode(), ctypes.byref(hdr)))
+    # every tensor: file -> device (compare with what the writer put there) -> new file, in reverse order
+    for (L, t, part), a in reversed(list(tensors.items())):
+        off, cnt = ctypes.c_uint64(), ctypes.c_uint64()
+        br.check(br.lib.mi355_ckpt_locate(ctypes.byref(hdr), L, t, part, ctypes.byref(off), ctypes.byref(cnt)))
+        d = br.DevArray(cnt.value)
+        br.check(br.lib.mi355_ckpt_load_dev(src.encode(), off.value, d.ptr, cnt.value))
+        assert d.numpy().tobytes() == a.tobytes(), (L, t, part)
+        br.check(br.lib.mi355_ckpt_store_dev(dst.encode(), off.value, d.ptr, cnt.value))
+    assert open(dst, "rb").read() == open(src, "rb").read()                  # byte-identical checkpoint
+    d = br.DevArray(16)
+    assert br.lib.mi355_ckpt_load_dev(src.encode(), os.path.getsize(src) - 8, d.ptr, 16) == -1   # runs off the end
+    assert br.lib.mi355_ckpt_store_dev(str(tmp_path / "absent.bin").encode(), 96, d.ptr, 16) == -1
+
+
+# ---------------------------------------------------------------------------------------------
 # host-pointer drop-ins (reference signatures) and error behaviour
 # ---------------------------------------------------------------------------------------------
 def _p(a):
