@@ -127,6 +127,7 @@ MI355_API int mi355_tune_set(const char *key, int value) {
         {"ew_unroll", &g_ctx.ew_unroll}, {"ew_threads", &g_ctx.ew_threads},
         {"ce_rows", &g_ctx.ce_rows}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
         {"gather_tile", &g_ctx.gather_tile}, {"nt_store", &g_ctx.nt_store},
+        {"gemm_splitk", &g_ctx.gemm_splitk},
     };
     for (auto &t : tab)
         if (strcmp(t.k, key) == 0) { *t.v = value; return 0; }

@@ -772,6 +772,26 @@ def test_sgemm_pitched_operands(br, ta, tb):
     assert np.array_equal(got[:, N:], C0[:, N:])                          # padding columns untouched
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
+def test_sgemm_long_inner_dimension_is_split_deterministically(br, ta, tb):
+    """Small output, long K (the dy = cembed^T . dlogits shape): the K-sliced path, including a ragged last slice."""
+    M, N, K = 96, 64, 9001
+    A = H.normal(190, (K, M) if ta else (M, K)); B = H.normal(191, (N, K) if tb else (K, N)); C0 = H.normal(192, (M, N))
+    ad, bd = dev(br, A), dev(br, B)
+    outs = []
+    for knob in (0, 7, 1):                                           # automatic, forced 7 slices, unsplit
+        br.tune("gemm_splitk", knob)
+        for beta in (0.0, -0.5):
+            cd = dev(br, C0)
+            br.check(br.lib.mi355_sgemm_dev(ta, tb, M, N, K, 0.75, ad.ptr, A.shape[1], bd.ptr, B.shape[1], beta, cd.ptr, N))
+            got = cd.numpy()
+            assert H.rel_err(got, O.sgemm(ta, tb, 0.75, A, B, beta, C0)) <= TOL, (knob, beta)
+            cd2 = dev(br, C0)
+            br.check(br.lib.mi355_sgemm_dev(ta, tb, M, N, K, 0.75, ad.ptr, A.shape[1], bd.ptr, B.shape[1], beta, cd2.ptr, N))
+            assert cd2.numpy().tobytes() == got.tobytes()            # same bits on a second run
+    br.tune("gemm_splitk", 0)
+
+
 def test_sgemm_bad_arguments(br):
     a = br.DevArray(64)
     assert br.lib.mi355_sgemm_dev(0, 0, 4, 4, 4, 1.0, a.ptr, 3, a.ptr, 4, 0.0, a.ptr, 4) == -1
