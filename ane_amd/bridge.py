@@ -99,6 +99,10 @@ SIGNATURES = {
     "mi355_ckpt_create": (_i, [_s, C.POINTER(CkptHdr)]),
     "mi355_ckpt_load_dev": (_i, [_s, _u64, _p, _u64]),
     "mi355_ckpt_store_dev": (_i, [_s, _u64, _p, _u64]),
+    "mi355_graph_begin": (_i, []),
+    "mi355_graph_end": (_p, []),
+    "mi355_graph_launch": (_i, [_p]),
+    "mi355_graph_free": (None, [_p]),
     "mi355_sgemm_dev": (_i, [_i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _f, _p, _i]),
     "mi355_cvt_f32_f16_dev": (_i, [_p, _z, _p, _z, _z, _z]),
     "mi355_cvt_f16_f32_dev": (_i, [_p, _z, _p, _z, _z, _z]),

@@ -22,6 +22,8 @@ struct Mi355Ctx {
     int device;
     int num_cu;
     hipStream_t stream;
+    unsigned alloc_epoch;      // bumped whenever a workspace that recorded graphs may point into is reallocated
+    bool capturing;            // between mi355_graph_begin and mi355_graph_end: `stream` is the capture stream
     void *ws;          // grow-only workspace
     size_t ws_bytes;
     // tuning knobs (0 = pick per shape)
@@ -33,6 +35,9 @@ extern Mi355Ctx g_ctx;
 int mi355_fail(const char *fmt, ...);
 // True when the context is usable; otherwise records the error.
 bool mi355_ready(const char *who);
+// False (with the error recorded) while a graph is being captured: for calls that allocate, free, copy to
+// or from the host, or wait.
+bool mi355_outside_capture(const char *who);
 // Workspace of at least `bytes` (256-byte aligned), NULL on failure.
 void *mi355_ws(size_t bytes);
 // Runs every queued weight-gradient reduction (dw_reduce.hip).

@@ -25,8 +25,16 @@ bool mi355_ready(const char *who) {
     return false;
 }
 
+bool mi355_outside_capture(const char *who) {
+    if (!g_ctx.capturing) return true;
+    mi355_fail("%s: not possible while a graph is being captured (it allocates, copies to the host or waits); "
+               "run the sequence once before capturing so that workspaces and tables exist", who);
+    return false;
+}
+
 void *mi355_ws(size_t bytes) {
     if (bytes <= g_ctx.ws_bytes && g_ctx.ws) return g_ctx.ws;
+    if (!mi355_outside_capture("workspace growth")) return nullptr;
     size_t want = (bytes + 0xFFFFF) & ~(size_t)0xFFFFF;   // 1 MiB granules
     if (g_ctx.ws) {
         (void)hipStreamSynchronize(g_ctx.stream);
@@ -42,6 +50,7 @@ void *mi355_ws(size_t bytes) {
     }
     g_ctx.ws = p;
     g_ctx.ws_bytes = want;
+    g_ctx.alloc_epoch++;
     return p;
 }
 
@@ -72,6 +81,7 @@ void mi355_free_caches(void);   // rope tables, host drop-in staging (other tran
 void mi355_dw_free(void);       // queued weight-gradient reductions and their arena
 void mi355_blas_free(void);     // rocBLAS handle of mi355_sgemm_dev
 void mi355_ckpt_free(void);     // pinned staging buffer of the checkpoint reader/writer
+void mi355_graph_shutdown(void);  // capture stream
 
 MI355_API void mi355_shutdown(void) {
     if (!g_ctx.ready) return;
@@ -80,6 +90,7 @@ MI355_API void mi355_shutdown(void) {
     mi355_dw_free();
     mi355_blas_free();
     mi355_ckpt_free();
+    mi355_graph_shutdown();
     if (g_ctx.ws) (void)hipFree(g_ctx.ws);
     g_ctx = Mi355Ctx{};
 }
@@ -103,6 +114,7 @@ MI355_API int mi355_device_info(char *name, size_t name_len, double *peak_hbm_gb
 
 MI355_API int mi355_set_stream(void *hip_stream) {
     if (!mi355_ready("set_stream")) return -1;
+    if (!mi355_outside_capture("set_stream")) return -1;
     if (mi355_dw_flush()) return -1;        // queued reductions belong to the old stream
     g_ctx.stream = (hipStream_t)hip_stream;
     return 0;
@@ -110,6 +122,7 @@ MI355_API int mi355_set_stream(void *hip_stream) {
 
 MI355_API int mi355_sync(void) {
     if (!mi355_ready("sync")) return -1;
+    if (!mi355_outside_capture("sync")) return -1;
     if (mi355_dw_flush()) return -1;
     HIP_OK(hipStreamSynchronize(g_ctx.stream));
     return 0;
@@ -145,6 +158,7 @@ struct mi355_buf {
 MI355_API mi355_buf *mi355_buf_alloc(size_t bytes) {
     if (!mi355_ready("buf_alloc")) return nullptr;
     if (bytes == 0) { mi355_fail("buf_alloc: zero bytes"); return nullptr; }
+    if (!mi355_outside_capture("buf_alloc")) return nullptr;
     void *p = nullptr;
     hipError_t e = hipMalloc(&p, bytes);
     if (e != hipSuccess) { mi355_fail("buf_alloc(%zu): %s", bytes, hipGetErrorString(e)); return nullptr; }
@@ -159,6 +173,7 @@ MI355_API mi355_buf *mi355_buf_alloc(size_t bytes) {
 
 MI355_API void mi355_buf_free(mi355_buf *b) {
     if (!b) return;
+    if (!mi355_outside_capture("buf_free")) return;
     if (g_ctx.ready && b->dev) {
         (void)hipStreamSynchronize(g_ctx.stream);
         (void)hipFree(b->dev);
@@ -171,6 +186,7 @@ MI355_API size_t mi355_buf_bytes(mi355_buf *b) { return b ? b->bytes : 0; }
 
 MI355_API void mi355_buf_write(mi355_buf *b, size_t offset, const void *src, size_t bytes) {
     if (!b || !src || !g_ctx.ready || offset > b->bytes || bytes > b->bytes - offset || bytes == 0) return;
+    if (!mi355_outside_capture("buf_write")) return;
     hipError_t e = hipMemcpyAsync((char *)b->dev + offset, src, bytes, hipMemcpyHostToDevice, g_ctx.stream);
     if (e == hipSuccess) e = hipStreamSynchronize(g_ctx.stream);
     if (e != hipSuccess) mi355_fail("buf_write: %s", hipGetErrorString(e));
@@ -178,6 +194,7 @@ MI355_API void mi355_buf_write(mi355_buf *b, size_t offset, const void *src, siz
 
 MI355_API void mi355_buf_read(mi355_buf *b, size_t offset, void *dst, size_t bytes) {
     if (!b || !dst || !g_ctx.ready || offset > b->bytes || bytes > b->bytes - offset || bytes == 0) return;
+    if (!mi355_outside_capture("buf_read")) return;
     (void)mi355_dw_flush();                 // a read may be of a gradient that is still queued
     hipError_t e = hipMemcpyAsync(dst, (const char *)b->dev + offset, bytes, hipMemcpyDeviceToHost, g_ctx.stream);
     if (e == hipSuccess) e = hipStreamSynchronize(g_ctx.stream);
@@ -295,4 +312,86 @@ MI355_API int mi355_fill_randint_dev(int32_t *p, size_t n, uint64_t seed, int32_
                        (uint32_t)(hi - lo));
     LAUNCH_OK("fill_randint");
     return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Graphs: a launch-bound sequence of ops recorded once and replayed as one submission.
+// Capture runs on a stream of the bridge's own (the default stream cannot be captured); replays go to the
+// bridge stream.  Nothing recorded may allocate, wait or touch the host, so the sequence has to have run once
+// before (workspaces sized, RoPE tables built).  No memset node is ever recorded: buffers are cleared by fill
+// kernels.
+// ---------------------------------------------------------------------------------------------
+struct mi355_graph {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+    unsigned epoch;     // g_ctx.alloc_epoch at capture: the recorded kernels hold workspace addresses of that time
+};
+
+static hipStream_t g_cap_stream = nullptr, g_saved_stream = nullptr;
+
+void mi355_graph_shutdown(void) {
+    if (g_cap_stream) (void)hipStreamDestroy(g_cap_stream);
+    g_cap_stream = nullptr;
+}
+
+MI355_API int mi355_graph_begin(void) {
+    if (!mi355_ready("graph_begin")) return -1;
+    if (g_ctx.capturing) return mi355_fail("graph_begin: a capture is already open");
+    if (mi355_dw_flush()) return -1;                       // queued reductions belong to the eager stream
+    HIP_OK(hipStreamSynchronize(g_ctx.stream));            // the recording starts from a quiet device
+    if (!g_cap_stream) HIP_OK(hipStreamCreate(&g_cap_stream));      // default flags and priority
+    HIP_OK(hipStreamBeginCapture(g_cap_stream, hipStreamCaptureModeThreadLocal));
+    g_saved_stream = g_ctx.stream;
+    g_ctx.stream = g_cap_stream;
+    g_ctx.capturing = true;
+    return 0;
+}
+
+MI355_API mi355_graph *mi355_graph_end(void) {
+    if (!g_ctx.ready || !g_ctx.capturing) { mi355_fail("graph_end: no capture is open"); return nullptr; }
+    const int flushed = mi355_dw_flush();                   // queued reductions become part of the graph
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(g_cap_stream, &graph);
+    g_ctx.stream = g_saved_stream;
+    g_ctx.capturing = false;
+    if (e != hipSuccess || !graph || flushed) {
+        if (graph) (void)hipGraphDestroy(graph);
+        (void)hipGetLastError();
+        if (e != hipSuccess || !graph) mi355_fail("graph_end: capture failed: %s", e == hipSuccess ? "empty graph" : hipGetErrorString(e));
+        return nullptr;
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        mi355_fail("graph_end: hipGraphInstantiate: %s", hipGetErrorString(e));
+        return nullptr;
+    }
+    mi355_graph *g = (mi355_graph *)malloc(sizeof(mi355_graph));
+    if (!g) { (void)hipGraphExecDestroy(exec); (void)hipGraphDestroy(graph); return nullptr; }
+    g->graph = graph;
+    g->exec = exec;
+    g->epoch = g_ctx.alloc_epoch;
+    return g;
+}
+
+MI355_API int mi355_graph_launch(mi355_graph *g) {
+    if (!mi355_ready("graph_launch")) return -1;
+    if (!g) return mi355_fail("graph_launch: NULL graph");
+    if (!mi355_outside_capture("graph_launch")) return -1;
+    if (g->epoch != g_ctx.alloc_epoch)
+        return mi355_fail("graph_launch: a workspace was reallocated after this graph was recorded; record it again");
+    if (mi355_dw_flush()) return -1;                        // keep eager reductions ahead of the replay
+    HIP_OK(hipGraphLaunch(g->exec, g_ctx.stream));
+    return 0;
+}
+
+MI355_API void mi355_graph_free(mi355_graph *g) {
+    if (!g) return;
+    if (g_ctx.ready) {
+        (void)hipStreamSynchronize(g_ctx.stream);
+        (void)hipGraphExecDestroy(g->exec);
+        (void)hipGraphDestroy(g->graph);
+    }
+    free(g);
 }

@@ -89,6 +89,7 @@ float *mi355_dw_partials(size_t floats, const float *out0, const float *out1) {
         if (launch_pending()) return nullptr;
     }
     if (floats > g_arena_floats) {
+        if (!mi355_outside_capture("growth of the weight-gradient arena")) return nullptr;
         size_t want = floats > ((size_t)32 << 20) ? floats : ((size_t)32 << 20);      // at least 128 MiB
         (void)hipStreamSynchronize(g_ctx.stream);
         if (g_arena) (void)hipFree(g_arena);
@@ -100,6 +101,7 @@ float *mi355_dw_partials(size_t floats, const float *out0, const float *out1) {
             return nullptr;
         }
         g_arena_floats = want;
+        g_ctx.alloc_epoch++;
     }
     float *p = g_arena + g_arena_used;
     g_arena_used += (floats + 63) & ~(size_t)63;
@@ -131,6 +133,7 @@ MI355_API int mi355_dw_flush(void) {
 
 MI355_API int mi355_dw_defer(int on) {
     if (!mi355_ready("dw_defer")) return -1;
+    if (!mi355_outside_capture("dw_defer")) return -1;
     if (launch_pending()) return -1;
     g_defer = on != 0;
     return 0;

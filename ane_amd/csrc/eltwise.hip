@@ -483,6 +483,7 @@ MI355_API int mi355_rope_tables_dev(const float **cos_dev, const float **sin_dev
             *sin_dev = g_rope[i].sin_d;
             return 0;
         }
+    if (!mi355_outside_capture("rope_tables_dev (first use of this S, head size and theta)")) return -1;
     if (g_rope_n == 64) return mi355_fail("rope_tables_dev: table cache full (64 distinct (S,hd,theta))");
     if (S <= 0 || hd <= 0 || (hd & 1) || !(theta > 0.f)) return mi355_fail("rope_tables_dev: bad S/hd/theta");
     const size_t n = (size_t)(hd / 2) * S;

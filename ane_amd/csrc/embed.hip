@@ -420,6 +420,7 @@ MI355_API int mi355_embed_gather_dev(float *x, const float *E, const int32_t *id
 MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, int V, int D, int S,
                                           int batch) {
     if (!mi355_ready("embed_scatter_add")) return -1;
+    if (!mi355_outside_capture("embed_scatter_add (its library sort may record memset nodes)")) return -1;
     if (!dE || !dx || !ids) return mi355_fail("embed_scatter_add: NULL pointer");
     if (V <= 0 || D <= 0 || S <= 0 || batch <= 0)
         return mi355_fail("embed_scatter_add: bad shape V=%d D=%d S=%d batch=%d", V, D, S, batch);

@@ -114,6 +114,7 @@ void mi355_blas_free(void) {
 MI355_API int mi355_sgemm_dev(int trans_a, int trans_b, int M, int N, int K, float alpha, const float *A, int lda,
                               const float *B, int ldb, float beta, float *C, int ldc) {
     if (!mi355_ready("sgemm")) return -1;
+    if (!mi355_outside_capture("sgemm (the GEMM library manages its own workspace)")) return -1;
     if (!A || !B || !C) return mi355_fail("sgemm: NULL pointer");
     const int ta = trans_flag(trans_a), tb = trans_flag(trans_b);
     if (ta < 0 || tb < 0) return mi355_fail("sgemm: transpose flags must be 0/1 (or CblasNoTrans/CblasTrans)");

@@ -515,6 +515,8 @@ def main():
     ap.add_argument("--fuse", action="store_true",
                     help="run each residual and the RMSNorm after it as one launch (mi355_residual_rmsnorm_fwd_dev)")
     ap.add_argument("--op-reps", type=int, default=3)
+    ap.add_argument("--graph", action="store_true",
+                    help="record one step as a graph and time its replays (pays off where the step is launch-bound)")
     ap.add_argument("--workload", default="qwen3", choices=["qwen3", "stories110m", "embed", "optimizer", "aux"],
                     help="qwen3 = the headline sweep (default); stories110m = the same sweep at the Stories110M shape "
                          "(BASELINE configs 0/1: one [C,256] sequence per op, 12 layers, RoPE without QK-norm); "
@@ -544,8 +546,19 @@ def main():
     for _ in range(args.warmup):
         wl.step()
     br.sync()
+    step = wl.step
+    if args.graph:
+        br.check(br.lib.mi355_graph_begin())
+        wl.step()
+        graph = br.lib.mi355_graph_end()
+        if not graph:
+            raise SystemExit("bench: graph capture failed: " + br.last_error())
+        step = lambda: br.check(br.lib.mi355_graph_launch(graph))
+        for _ in range(2):
+            step()
+        br.sync()
     t0 = time.perf_counter()
-    ms = time_region(br, wl.step, args.steps)
+    ms = time_region(br, step, args.steps)
     br.sync()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
@@ -580,7 +593,7 @@ def main():
                                    cfg["H"], cfg["heads"], cfg["kv_heads"], cfg["hd"],
                                    "QK-norm + RoPE" if cfg["qk_norm"] else "RoPE", cfg["V"], cfg["S"]),
                    "layers": args.layers, "tokens_per_step": tokens, "alg_gb_per_step": total_bytes / 1e9,
-                   "residual_fused_into_next_rmsnorm": wl.fuse,
+                   "residual_fused_into_next_rmsnorm": wl.fuse, "replayed_as_graph": bool(args.graph),
                    "weight_gradients": "reduced per op" if args.immediate_dw else "queued, reduced once per step"},
         "aggregate_gbs": total_bytes / ms / 1e6, "aggregate_frac_of_peak": total_bytes / ms / 1e6 / PEAK_HBM_GBS,
         "host_wall_ms_per_step": wall_ms,

@@ -70,6 +70,19 @@ void mi355_buf_write(mi355_buf *b, size_t offset, const void *src, size_t bytes)
 void mi355_buf_read(mi355_buf *b, size_t offset, void *dst, size_t bytes);
 int mi355_buf_zero(mi355_buf *b);                         /* asynchronous fill on the bridge stream */
 
+/* Graphs: record a launch-bound sequence of device-resident ops once, replay it as one submission.  No
+ * counterpart in the reference (its ops are synchronous CPU calls).  Between begin and end the *_dev ops are
+ * recorded instead of run; calls that allocate, wait or touch the host (buf_alloc/free/read/write, sync,
+ * set_stream, workspace growth, a first-time RoPE table, embed_scatter_add, sgemm, ckpt_*) fail with -1 and end
+ * in a failed capture, so run the sequence once eagerly first.  mi355_graph_launch enqueues the replay on the
+ * bridge stream; it fails if a workspace was reallocated since the recording (record again).  Accumulating ops
+ * (dw +=) accumulate on every replay. */
+typedef struct mi355_graph mi355_graph;
+int mi355_graph_begin(void);
+mi355_graph *mi355_graph_end(void);          /* NULL on failure */
+int mi355_graph_launch(mi355_graph *g);
+void mi355_graph_free(mi355_graph *g);       /* NULL-safe */
+
 /* Timing on the bridge stream (HIP events). */
 typedef struct mi355_event mi355_event;
 mi355_event *mi355_event_create(void);
