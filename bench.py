@@ -421,6 +421,56 @@ def bench_optimizer(br, args):
     print(json.dumps(out))
 
 
+def bench_host(br, args):
+    """The host-pointer drop-ins (reference signatures, operands in ordinary host memory) at the Stories110M
+    shape, each timed per call including both PCIe directions, beside the CPU oracle on the same arrays."""
+    import oracle as O
+    C, Hh, S, V, hd = 768, 2048, 256, 32000, 64
+    rng = np.random.default_rng(0)
+    f = lambda *sh: rng.standard_normal(sh).astype(np.float32)
+    P = lambda a: a.ctypes.data
+    x, dy, w, dw = f(C, S), f(C, S), (1 + 0.02 * f(C)).astype(np.float32), np.zeros(C, np.float32)
+    out, dx = np.empty_like(x), np.empty_like(x)
+    h1, h3, ds = f(Hh * S), f(Hh * S), f(Hh * S)
+    o1, o2 = np.empty_like(h1), np.empty_like(h1)
+    logits = (2 * f(V, S)).astype(np.float32); dl = np.empty_like(logits)
+    tg = rng.integers(0, V, S).astype(np.uint16)
+    E = (0.02 * f(V, C)).astype(np.float32); tok = zipf_ids(1, S, V).astype(np.uint16); xe = np.zeros((C, S), np.float32)
+    dE = np.zeros((V, C), np.float32)
+    L = br.lib
+    cases = [
+        ("rmsnorm", lambda: L.mi355_rmsnorm(P(out), P(x), P(w), C, S), lambda: O.rmsnorm(x, w), 2 * x.nbytes),
+        ("rmsnorm_bwd", lambda: L.mi355_rmsnorm_bwd(P(dx), P(dw), P(dy), P(x), P(w), C, S), lambda: O.rmsnorm_bwd(dy, x, w), 3 * x.nbytes),
+        ("swiglu_fwd", lambda: L.mi355_swiglu_fwd(P(o1), P(h1), P(h3), h1.size), lambda: O.swiglu_fwd(h1, h3), 3 * h1.nbytes),
+        ("swiglu_bwd", lambda: L.mi355_swiglu_bwd(P(o1), P(o2), P(ds), P(h1), P(h3), h1.size), lambda: O.swiglu_bwd(ds, h1, h3), 5 * h1.nbytes),
+        ("axpby (vsma)", lambda: L.mi355_axpby(P(out), P(x), P(dy), 2.2134, x.size, 0), lambda: O.axpby(x, dy, 2.2134, 0), 3 * x.nbytes),
+        ("rope_backward_inplace", lambda: L.mi355_rope_backward_inplace(P(dx), S, C, hd), lambda: O.rope(dx, hd, 10000.0, -1), 2 * x.nbytes),
+        ("cross_entropy_loss", lambda: L.mi355_cross_entropy_loss(P(dl), P(logits), P(tg), V, S), lambda: O.cross_entropy(logits, tg.astype(np.int32)), 2 * logits.nbytes),
+        ("embed_lookup (table resident)", lambda: L.mi355_embed_lookup(P(xe), P(E), P(tok), V, C, S), lambda: O.embed_lookup(E, tok.astype(np.int32).reshape(1, S)), xe.nbytes),
+    ]
+    rows = []
+    for name, gpu, cpu, pcie in cases:
+        for _ in range(3):
+            gpu()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            gpu()
+        g_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        cpu()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            cpu()
+        c_ms = (time.perf_counter() - t0) * 1e3 / 3
+        rows.append(dict(op=name, gpu_ms_per_call=round(g_ms, 4), cpu_oracle_ms_per_call=round(c_ms, 4),
+                         host_bytes_mb=pcie / 1e6, pcie_inclusive_gbs=round(pcie / g_ms / 1e6, 2)))
+    tot = sum(r["gpu_ms_per_call"] for r in rows)
+    print(json.dumps({"metric": "host-pointer drop-ins at the Stories110M shape, per call including PCIe both ways",
+                      "value": S / (tot / 1e3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": 3,
+                      "ms_per_step": tot, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+                      "data": "synthetic", "config": {"workload": "host-pointer drop-ins, C 768, H 2048, S 256, V 32000"},
+                      "ops": rows}))
+
+
 def bench_aux(br, args):
     """The helpers either side of the hot path at the Qwen3-0.6B shape: GQA tile / reduce
     (training/training_dynamic/io.h:330-351) on 16 x 256 tokens, and the vocabulary-compaction row copies
@@ -517,7 +567,7 @@ def main():
     ap.add_argument("--op-reps", type=int, default=3)
     ap.add_argument("--graph", action="store_true",
                     help="record one step as a graph and time its replays (pays off where the step is launch-bound)")
-    ap.add_argument("--workload", default="qwen3", choices=["qwen3", "stories110m", "embed", "optimizer", "aux"],
+    ap.add_argument("--workload", default="qwen3", choices=["qwen3", "stories110m", "embed", "optimizer", "aux", "host"],
                     help="qwen3 = the headline sweep (default); stories110m = the same sweep at the Stories110M shape "
                          "(BASELINE configs 0/1: one [C,256] sequence per op, 12 layers, RoPE without QK-norm); "
                          "embed = BASELINE config 2; optimizer = the Adam tail (each prints its own JSON line)")
@@ -535,6 +585,8 @@ def main():
         return bench_optimizer(br, args)
     if args.workload == "aux":
         return bench_aux(br, args)
+    if args.workload == "host":
+        return bench_host(br, args)
     cfg = dict(S110 if args.workload == "stories110m" else Q3)
     if args.batch > 0:
         cfg["batch"] = args.batch
