@@ -99,6 +99,13 @@ SIGNATURES = {
     "mi355_ckpt_create": (_i, [_s, C.POINTER(CkptHdr)]),
     "mi355_ckpt_load_dev": (_i, [_s, _u64, _p, _u64]),
     "mi355_ckpt_store_dev": (_i, [_s, _u64, _p, _u64]),
+    "mi355_cvt_f32_bf16_dev": (_i, [_p, _z, _p, _z, _z, _z]),
+    "mi355_cvt_bf16_f32_dev": (_i, [_p, _z, _p, _z, _z, _z]),
+    "mi355_rmsnorm_fwd_bf16_dev": (_i, [_p, _p, _p, _i, _i, _i, _f]),
+    "mi355_rmsnorm_bwd_bf16_dev": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _f, _i]),
+    "mi355_swiglu_fwd_bf16_dev": (_i, [_p, _p, _p, _z]),
+    "mi355_swiglu_bwd_bf16_dev": (_i, [_p, _p, _p, _p, _p, _z]),
+    "mi355_axpby_bf16_dev": (_i, [_p, _p, _p, _f, _z, _i]),
     "mi355_graph_begin": (_i, []),
     "mi355_graph_end": (_p, []),
     "mi355_graph_launch": (_i, [_p]),

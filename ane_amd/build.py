@@ -10,7 +10,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmi355_ops.so")
 
 SOURCES = ["context.hip", "dw_reduce.hip", "norm.hip", "eltwise.hip", "qknorm_rope.hip", "embed.hip", "softmax_ce.hip", "optim.hip",
-           "staging.hip", "gemm.hip", "ckpt.hip", "host_dropins.hip"]
+           "staging.hip", "bf16_ops.hip", "gemm.hip", "ckpt.hip", "host_dropins.hip"]
 
 # -ffp-contract=off: products and sums round separately, as the reference's sequences of vDSP calls do;
 # the packed-fp32 feature is disabled because some packed forms have given wrong results on this hardware.

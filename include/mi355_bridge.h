@@ -70,6 +70,21 @@ void mi355_buf_write(mi355_buf *b, size_t offset, const void *src, size_t bytes)
 void mi355_buf_read(mi355_buf *b, size_t offset, void *dst, size_t bytes);
 int mi355_buf_zero(mi355_buf *b);                         /* asynchronous fill on the bridge stream */
 
+/* Optional bfloat16-storage variants (no counterpart in the reference, whose CPU ops are fp32): the same
+ * arithmetic in fp32 registers, activations in device memory as bfloat16 bit patterns (uint16_t, the upper half
+ * of the fp32 pattern), results rounded to nearest even on store; norm weights and weight gradients stay fp32.
+ * They agree with the fp32 entry points run on the same bf16-representable inputs to within 5e-3.
+ * Arguments as the fp32 entry points of the same name. */
+int mi355_cvt_f32_bf16_dev(uint16_t *dst, size_t dst_ld, const float *src, size_t src_ld, size_t rows, size_t cols);
+int mi355_cvt_bf16_f32_dev(float *dst, size_t dst_ld, const uint16_t *src, size_t src_ld, size_t rows, size_t cols);
+int mi355_rmsnorm_fwd_bf16_dev(uint16_t *y, const uint16_t *x, const float *w, int C, int S, int batch, float eps);
+int mi355_rmsnorm_bwd_bf16_dev(uint16_t *dx, float *dw, const uint16_t *dy, const uint16_t *x, const float *w, int C,
+                               int S, int batch, float eps, int variant);
+int mi355_swiglu_fwd_bf16_dev(uint16_t *out, const uint16_t *h1, const uint16_t *h3, size_t n);
+int mi355_swiglu_bwd_bf16_dev(uint16_t *dh1, uint16_t *dh3, const uint16_t *dsilu, const uint16_t *h1,
+                              const uint16_t *h3, size_t n);
+int mi355_axpby_bf16_dev(uint16_t *y, const uint16_t *a, const uint16_t *b, float alpha, size_t n, int mode);
+
 /* Graphs: record a launch-bound sequence of device-resident ops once, replay it as one submission.  No
  * counterpart in the reference (its ops are synchronous CPU calls).  Between begin and end the *_dev ops are
  * recorded instead of run; calls that allocate, wait or touch the host (buf_alloc/free/read/write, sync,

@@ -58,6 +58,8 @@ def _load():
         "orc_gqa_reduce": (None, [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int]),
         "orc_sgemm": (None, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, _f32p, C.c_int, _f32p, C.c_int,
                              C.c_float, _f32p, C.c_int, C.c_int]),
+        "orc_cvt_f32_bf16": (None, [_u16p, _f32p, C.c_size_t]),
+        "orc_cvt_bf16_f32": (None, [_f32p, _u16p, C.c_size_t]),
         "orc_cvt_f32_f16": (None, [_u16p, C.c_size_t, _f32p, C.c_size_t, C.c_size_t, C.c_size_t]),
         "orc_cvt_f16_f32": (None, [_f32p, C.c_size_t, _u16p, C.c_size_t, C.c_size_t, C.c_size_t]),
         "orc_adam_update": (None, [_f32p, _f32p, _f32p, _f32p, C.c_size_t, C.c_int, C.c_float,
@@ -235,6 +237,21 @@ def sgemm(ta, tb, alpha, A, B, beta=0.0, Cin=None, threads=8):
     out = np.zeros((M, N), np.float32) if Cin is None else _f32(Cin).copy()
     lib.orc_sgemm(int(ta), int(tb), M, N, K, alpha, A.reshape(-1), A.shape[1], B.reshape(-1), B.shape[1], beta,
                   out.reshape(-1), N, threads)
+    return out
+
+
+def cvt_f32_bf16(x):
+    """fp32 -> bfloat16 bit patterns (uint16), round to nearest even."""
+    x = _f32(x)
+    out = np.empty(x.shape, np.uint16)
+    lib.orc_cvt_f32_bf16(out.reshape(-1), x.reshape(-1), x.size)
+    return out
+
+
+def cvt_bf16_f32(h):
+    h = np.ascontiguousarray(h, np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib.orc_cvt_bf16_f32(out.reshape(-1), h.reshape(-1), h.size)
     return out
 
 

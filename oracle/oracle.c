@@ -480,6 +480,26 @@ ORC_API void orc_cvt_f16_f32(float *dst, size_t dst_ld, const uint16_t *src, siz
 }
 
 /* ---------------------------------------------------------------------------------------------
+ * bfloat16 <-> fp32 (for the optional bf16-storage variants; the reference has none).  bfloat16 is the upper
+ * half of the binary32 pattern; narrowing rounds to nearest even, NaN stays NaN.
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_cvt_f32_bf16(uint16_t *dst, const float *src, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        uint32_t u;
+        memcpy(&u, &src[i], 4);
+        if ((u & 0x7fffffffu) > 0x7f800000u) dst[i] = (uint16_t)((u >> 16) | 0x40u);
+        else dst[i] = (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+    }
+}
+
+ORC_API void orc_cvt_bf16_f32(float *dst, const uint16_t *src, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        uint32_t u = (uint32_t)src[i] << 16;
+        memcpy(&dst[i], &u, 4);
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
  * Adam / AdamW — training/stories_cpu_ops.h:55-63 (wd = 0) and training_dynamic/cpu_ops.h:56-64.
  * ------------------------------------------------------------------------------------------- */
 ORC_API void orc_adam_update(float *w, const float *g, float *m, float *v, size_t n, int t,

@@ -1,0 +1,92 @@
+"""Optional bfloat16-storage variants: parity with the fp32 oracle run on the same bf16-representable inputs,
+within 5e-3 (the tolerance stated for bf16 variants); the converts themselves are bit-exact."""
+import numpy as np
+import pytest
+
+import helpers as H
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL16 = 5e-3
+
+
+def bf(a):
+    """fp32 array -> (bf16 bit patterns, the fp32 values they stand for)."""
+    bits = O.cvt_f32_bf16(a)
+    return bits, O.cvt_bf16_f32(bits)
+
+
+def dev(br, a):
+    return br.DevArray.from_numpy(a)
+
+
+def back(d):
+    return O.cvt_bf16_f32(d.numpy())
+
+
+@pytest.mark.parametrize("rows,cols,dst_ld,src_ld", [(1, 1 << 20, 1 << 20, 1 << 20), (7, 13, 19, 13), (5, 16, 16, 24)])
+def test_bf16_converts_bit_exact(br, rows, cols, dst_ld, src_ld):
+    src = H.normal(200, (rows, src_ld), 0, 30.0)
+    if cols >= 4096:
+        b = H.f16_boundary_values()
+        ties = (np.arange(0x3f80, 0x4080, dtype=np.uint32) << 16 | 0x8000).view(np.float32)
+        src[0, :b.size] = b; src[0, b.size:b.size + ties.size] = ties
+    dst0 = np.random.default_rng(201).integers(0, 65536, (rows, dst_ld)).astype(np.uint16)
+    sd, dd = dev(br, src), dev(br, dst0)
+    br.check(br.lib.mi355_cvt_f32_bf16_dev(dd.ptr, dst_ld, sd.ptr, src_ld, rows, cols))
+    want = dst0.copy(); want[:, :cols] = O.cvt_f32_bf16(src[:, :cols])
+    assert np.array_equal(dd.numpy(), want)
+    b0 = H.normal(202, (rows, src_ld)); bd = dev(br, b0)
+    br.check(br.lib.mi355_cvt_bf16_f32_dev(bd.ptr, src_ld, dd.ptr, dst_ld, rows, cols))
+    wb = b0.copy(); wb[:, :cols] = O.cvt_bf16_f32(want[:, :cols])
+    assert np.array_equal(bd.numpy().view(np.uint32), wb.view(np.uint32))
+
+
+@pytest.mark.parametrize("n", [16 * 3072 * 256, 2048 * 256, 1003, 8])
+def test_swiglu_and_residual_bf16(br, n):
+    print("[case] bf16 swiglu/axpby n=%d" % n, flush=True)
+    (h1b, h1), (h3b, h3), (db, d) = bf(H.normal(210, n)), bf(H.normal(211, n)), bf(H.normal(212, n))
+    h1d, h3d, dd = dev(br, h1b), dev(br, h3b), dev(br, db)
+    out, o1, o3 = (br.DevArray(n, np.uint16) for _ in range(3))
+    br.check(br.lib.mi355_swiglu_fwd_bf16_dev(out.ptr, h1d.ptr, h3d.ptr, n))
+    assert H.rel_err(back(out), O.swiglu_fwd(h1, h3)) <= TOL16
+    br.check(br.lib.mi355_swiglu_bwd_bf16_dev(o1.ptr, o3.ptr, dd.ptr, h1d.ptr, h3d.ptr, n))
+    r1, r3 = O.swiglu_bwd(d, h1, h3)
+    assert H.rel_err(back(o1), r1) <= TOL16 and H.rel_err(back(o3), r3) <= TOL16
+    # the stored values are the correctly rounded fp32 results: identical to rounding the oracle's output
+    assert np.mean(out.numpy() == O.cvt_f32_bf16(O.swiglu_fwd(h1, h3))) > 0.999
+    al = np.float32(24 ** 0.25)
+    for mode, ref in ((0, O.axpby(h1, h3, al, 0)), (1, O.axpby(h1, None, al, 1)), (2, O.axpby(h1, h3, 0.0, 2))):
+        y = br.DevArray(n, np.uint16)
+        br.check(br.lib.mi355_axpby_bf16_dev(y.ptr, h1d.ptr, None if mode == 1 else h3d.ptr, al, n, mode))
+        assert np.array_equal(y.numpy(), O.cvt_f32_bf16(ref))          # exact fp32 arithmetic, one rounding
+    br.check(br.lib.mi355_axpby_bf16_dev(h1d.ptr, h1d.ptr, h3d.ptr, al, n, 0))          # in place
+    assert np.array_equal(h1d.numpy(), O.cvt_f32_bf16(O.axpby(h1, h3, al, 0)))
+
+
+@pytest.mark.parametrize("B,C,S", [(16, 1024, 256), (1, 768, 256), (2, 100, 37), (3, 48, 24), (2, 5000, 64), (5, 128, 256),
+                                   (2, 300, 16), (1, 2048, 8), (1, 1, 8)])
+def test_rmsnorm_bf16(br, B, C, S):
+    print("[case] bf16 rmsnorm B=%d C=%d S=%d" % (B, C, S), flush=True)
+    (xb, x), (dyb, dy) = bf(H.normal(220, (B, C, S))), bf(H.normal(221, (B, C, S)))
+    w = H.normal(222, C, 1.0, 0.02); dw0 = H.normal(223, C)
+    xd, dyd, wd = dev(br, xb), dev(br, dyb), dev(br, w)
+    y, dx = br.DevArray(x.shape, np.uint16), br.DevArray(x.shape, np.uint16)
+    br.check(br.lib.mi355_rmsnorm_fwd_bf16_dev(y.ptr, xd.ptr, wd.ptr, C, S, B, 1e-5))
+    assert H.rel_err(back(y), O.rmsnorm(x, w)) <= TOL16
+    for variant in (0, 1):
+        dwd = dev(br, dw0)
+        br.check(br.lib.mi355_rmsnorm_bwd_bf16_dev(dx.ptr, dwd.ptr, dyd.ptr, xd.ptr, wd.ptr, C, S, B, 1e-5, variant))
+        rdx, rdw = O.rmsnorm_bwd(dy, x, w, variant=variant, dw=dw0)
+        assert H.rel_err(back(dx), rdx) <= TOL16
+        assert H.rel_err(dwd.numpy(), rdw) <= 1e-5                      # fp32 in, fp32 sums, fp32 out
+
+
+def test_bf16_bad_arguments(br):
+    a = br.DevArray(64, np.uint16); w = br.DevArray(8)
+    assert br.lib.mi355_rmsnorm_fwd_bf16_dev(a.ptr, a.ptr, None, 8, 8, 1, 1e-5) == -1
+    assert br.lib.mi355_rmsnorm_bwd_bf16_dev(a.ptr, w.ptr, a.ptr, a.ptr, w.ptr, 8, 8, 1, 1e-5, 2) == -1
+    assert br.lib.mi355_swiglu_fwd_bf16_dev(a.ptr, a.ptr, a.ptr, 0) == -1
+    assert br.lib.mi355_axpby_bf16_dev(a.ptr, a.ptr, None, 1.0, 64, 0) == -1
+    assert br.lib.mi355_cvt_f32_bf16_dev(a.ptr, 4, w.ptr, 8, 1, 8) == -1
+    assert "bf16" in br.last_error()

@@ -252,6 +252,24 @@ def test_sgemm_is_the_row_major_product(ta, tb):
     assert np.isfinite(O.sgemm(ta, tb, 1.0, A, B, 0.0, np.full((M, N), np.nan, np.float32))).all()
 
 
+def test_bf16_converts_match_an_independent_implementation():
+    """torch's bfloat16 is an independent round-to-nearest-even implementation."""
+    import torch
+    v = np.concatenate([H.f16_boundary_values(),
+                        np.random.default_rng(8).integers(0, 2 ** 32, 1_000_000, dtype=np.uint64).astype(np.uint32).view(np.float32)])
+    # exact ties of bf16: patterns ending in 0x8000, both parities of the kept part
+    ties = (np.arange(0x3f80, 0x4080, dtype=np.uint32) << 16 | 0x8000).view(np.float32)
+    v = np.concatenate([v, ties, -ties, np.array([3.3895314e38, 3.4028235e38, np.inf, -np.inf, 0.0, -0.0, 1e-45], np.float32)])
+    v = v[~np.isnan(v)]
+    ref = torch.from_numpy(v.copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = O.cvt_f32_bf16(v)
+    assert np.array_equal(got, ref)
+    allb = np.arange(65536, dtype=np.uint16)
+    back = O.cvt_bf16_f32(allb)
+    assert np.array_equal(back.view(np.uint32), allb.astype(np.uint32) << 16)
+    assert np.isnan(O.cvt_bf16_f32(O.cvt_f32_bf16(np.array([np.nan], np.float32)))).all()
+
+
 def test_adam_matches_formula():
     n = 257
     w = H.normal(17, n); g = H.normal(18, n); m = H.normal(19, n, 0, 0.1); v = np.abs(H.normal(20, n, 0, 0.1))
