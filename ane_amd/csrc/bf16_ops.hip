@@ -55,6 +55,48 @@ __device__ __forceinline__ void stb(bf16_t *p, const float (&r)[VEC]) {
     }
 }
 
+// Register tiles keep the bf16 words packed (half the registers of an fp32 tile) and widen them at each use.
+template <int VEC> struct RawT { typedef unsigned type; };
+template <> struct RawT<8> { typedef v4u type; };
+template <int VEC, bool NT>
+__device__ __forceinline__ typename RawT<VEC>::type ld_raw(const bf16_t *p) {
+    if constexpr (VEC == 8) {
+        const v4u *q = reinterpret_cast<const v4u *>(p);
+        return NT ? __builtin_nontemporal_load(q) : *q;
+    } else {
+        return (unsigned)*p;
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void unpack(float (&r)[VEC], const typename RawT<VEC>::type &w) {
+    if constexpr (VEC == 8) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            r[2 * j] = bf_to_f(w[j] & 0xffffu);
+            r[2 * j + 1] = bf_to_f(w[j] >> 16);
+        }
+    } else {
+        r[0] = bf_to_f(w);
+    }
+}
+// Tells the compiler nothing about the words' contents from here on, so that the widened copies made before a
+// reduction are dropped instead of being kept alive across it (they would double the register tile).
+template <int VEC>
+__device__ __forceinline__ void forget(typename RawT<VEC>::type &w) {
+    if constexpr (VEC == 8) {
+        unsigned a = w[0], b = w[1], c = w[2], d = w[3];
+        asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+        w[0] = a; w[1] = b; w[2] = c; w[3] = d;
+    } else {
+        asm volatile("" : "+v"(w));
+    }
+}
+template <int VEC>
+__device__ __forceinline__ typename RawT<VEC>::type raw_zero() {
+    if constexpr (VEC == 8) { v4u z = {0u, 0u, 0u, 0u}; return z; }
+    else return 0u;
+}
+
 // ---- converts (rectangles, as the fp16 staging converts) ----
 template <int VEC>
 __global__ __launch_bounds__(BT) void cvt_f32_bf16_kernel(bf16_t *__restrict__ dst, size_t dst_ld,
@@ -164,24 +206,25 @@ __global__ __launch_bounds__(THREADS) void rms_fwd_bf16_kernel(bf16_t *__restric
 #pragma unroll
     for (int j = 0; j < VEC; j++) acc[0][j] = 0.f;
     if constexpr (CAP > 0) {
-        float xv[CAP][VEC], wv[CAP];
+        typename RawT<VEC>::type xr[CAP];
+        float wv[CAP];
 #pragma unroll
         for (int k = 0; k < CAP; k++) {
             const int c = row0 + k * RPS;
-            if (c < C && col_ok) {
-                ldb<VEC, true>(xv[k], x + base + (size_t)c * S);
-                wv[k] = w[c];
-            } else {
-#pragma unroll
-                for (int j = 0; j < VEC; j++) xv[k][j] = 0.f;
-                wv[k] = 0.f;
-            }
+            const bool ok = c < C && col_ok;
+            xr[k] = ok ? ld_raw<VEC, true>(x + base + (size_t)c * S) : raw_zero<VEC>();
+            wv[k] = ok ? w[c] : 0.f;
         }
 #pragma unroll
-        for (int k = 0; k < CAP; k++)
+        for (int k = 0; k < CAP; k++) {
+            float xv[VEC];
+            unpack<VEC>(xv, xr[k]);
 #pragma unroll
-            for (int j = 0; j < VEC; j++) acc[0][j] += xv[k][j] * xv[k][j];
+            for (int j = 0; j < VEC; j++) acc[0][j] += xv[j] * xv[j];
+        }
         strip_reduce<VEC, LPR, THREADS, 1>(acc, lds);
+#pragma unroll
+        for (int k = 0; k < CAP; k++) forget<VEC>(xr[k]);
         float rr[VEC];
 #pragma unroll
         for (int j = 0; j < VEC; j++) rr[j] = 1.0f / sqrtf(acc[0][j] * invC + eps);
@@ -189,9 +232,10 @@ __global__ __launch_bounds__(THREADS) void rms_fwd_bf16_kernel(bf16_t *__restric
         for (int k = 0; k < CAP; k++) {
             const int c = row0 + k * RPS;
             if (c < C && col_ok) {
-                float o[VEC];
+                float xv[VEC], o[VEC];
+                unpack<VEC>(xv, xr[k]);
 #pragma unroll
-                for (int j = 0; j < VEC; j++) o[j] = (xv[k][j] * rr[j]) * wv[k];
+                for (int j = 0; j < VEC; j++) o[j] = (xv[j] * rr[j]) * wv[k];
                 stb<VEC>(y + base + (size_t)c * S, o);
             }
         }
@@ -257,28 +301,30 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_bf16_kernel(bf16_t *dx, float
     };
 
     if constexpr (CAP > 0) {
-        float xv[CAP][VEC], dv[CAP][VEC], wv[CAP];
+        typename RawT<VEC>::type xr[CAP], dr[CAP];
+        float wv[CAP];
 #pragma unroll
         for (int k = 0; k < CAP; k++) {
             const int c = row0 + k * RPS;
-            if (c < C && col_ok) {
-                ldb<VEC, true>(xv[k], x + base + (size_t)c * S);
-                ldb<VEC, true>(dv[k], dy + base + (size_t)c * S);
-                wv[k] = w[c];
-            } else {
-#pragma unroll
-                for (int j = 0; j < VEC; j++) xv[k][j] = dv[k][j] = 0.f;
-                wv[k] = 0.f;
-            }
+            const bool ok = c < C && col_ok;
+            xr[k] = ok ? ld_raw<VEC, true>(x + base + (size_t)c * S) : raw_zero<VEC>();
+            dr[k] = ok ? ld_raw<VEC, true>(dy + base + (size_t)c * S) : raw_zero<VEC>();
+            wv[k] = ok ? w[c] : 0.f;
         }
 #pragma unroll
-        for (int k = 0; k < CAP; k++)
+        for (int k = 0; k < CAP; k++) {
+            float xv[VEC], dv[VEC];
+            unpack<VEC>(xv, xr[k]);
+            unpack<VEC>(dv, dr[k]);
 #pragma unroll
             for (int j = 0; j < VEC; j++) {
-                acc[0][j] += xv[k][j] * xv[k][j];
-                acc[1][j] += (dv[k][j] * xv[k][j]) * wv[k];
+                acc[0][j] += xv[j] * xv[j];
+                acc[1][j] += (dv[j] * xv[j]) * wv[k];
             }
+        }
         strip_reduce<VEC, LPR, THREADS, 2>(acc, lds);
+#pragma unroll
+        for (int k = 0; k < CAP; k++) { forget<VEC>(xr[k]); forget<VEC>(dr[k]); }
         float rr[VEC], dotn[VEC];
 #pragma unroll
         for (int j = 0; j < VEC; j++) {
@@ -288,7 +334,12 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_bf16_kernel(bf16_t *dx, float
 #pragma unroll
         for (int k = 0; k < CAP; k++) {
             const int c = row0 + k * RPS;
-            if (c < C) row_out(c, xv[k], dv[k], wv[k], rr, dotn);      // uniform per group of LPR lanes
+            if (c < C) {                                                  // uniform per group of LPR lanes
+                float xv[VEC], dv[VEC];
+                unpack<VEC>(xv, xr[k]);
+                unpack<VEC>(dv, dr[k]);
+                row_out(c, xv, dv, wv[k], rr, dotn);
+            }
         }
     } else {
         if (col_ok)
@@ -324,19 +375,274 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_bf16_kernel(bf16_t *dx, float
     }
 }
 
+// ---- RoPE and per-head QK-RMSNorm + RoPE ----
+// fp32 table row -> VEC floats (tables are shared by all heads and sequences: cached loads)
+template <int VEC>
+__device__ __forceinline__ void ldtab(float (&r)[VEC], const float *p) {
+    if constexpr (VEC == 8) {
+        const v4f a = ld4(p), b = ld4(p + 4);
+#pragma unroll
+        for (int j = 0; j < 4; j++) { r[j] = a[j]; r[4 + j] = b[j]; }
+    } else {
+        r[0] = *p;
+    }
+}
+
+// one lane = one interleaved row pair of one head x VEC columns; Q pair rows first, then K
+template <int VEC>
+__global__ __launch_bounds__(BT) void rope_bf16_kernel(bf16_t *q_out, bf16_t *k_out, const bf16_t *q_in,
+                                                       const bf16_t *k_in, int heads, int kv_heads, int hd, int S,
+                                                       int batch, const float *__restrict__ cos_t,
+                                                       const float *__restrict__ sin_t, float sgn, size_t total) {
+    const size_t idx = (size_t)blockIdx.x * BT + threadIdx.x;
+    if (idx >= total) return;
+    const int cols = S / VEC;
+    const int cg = (int)(idx % cols);
+    size_t pr = idx / cols;
+    const int half = hd >> 1;
+    const size_t q_rows = (size_t)batch * heads * half;
+    const bf16_t *in = q_in;
+    bf16_t *out = q_out;
+    if (pr >= q_rows) { pr -= q_rows; in = k_in; out = k_out; }
+    const int i = (int)(pr % half);
+    const size_t row = (pr / half) * hd + 2 * i;
+    const int s = cg * VEC;
+    const size_t o0 = row * S + s;
+    float v0[VEC], v1[VEC], c[VEC], sn[VEC], r0[VEC], r1[VEC];
+    ldb<VEC, true>(v0, in + o0);
+    ldb<VEC, true>(v1, in + o0 + S);
+    ldtab<VEC>(c, cos_t + (size_t)i * S + s);
+    ldtab<VEC>(sn, sin_t + (size_t)i * S + s);
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        const float sj = sn[j] * sgn;
+        r0[j] = v0[j] * c[j] - v1[j] * sj;
+        r1[j] = v0[j] * sj + v1[j] * c[j];
+    }
+    stb<VEC>(out + o0, r0);
+    stb<VEC>(out + o0 + S, r1);
+}
+
+template <int VEC, int LPR, int THREADS, int CAP>
+__global__ __launch_bounds__(THREADS) void qknorm_rope_fwd_bf16_kernel(
+    bf16_t *__restrict__ q_out, bf16_t *__restrict__ k_out, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k,
+    const float *__restrict__ wq, const float *__restrict__ wk, int hd, int S, int strips, int nq,
+    const float *__restrict__ cos_t, const float *__restrict__ sin_t, float eps, float invhd) {
+    constexpr int PPS = THREADS / LPR;   // row pairs per step
+    constexpr int NW = THREADS / 64;
+    __shared__ float lds[NW * (LPR < 64 ? LPR : 64) * VEC];
+    int blk = blockIdx.x;
+    const bf16_t *in = q;
+    const float *w = wq;
+    bf16_t *out = q_out;
+    if (blk >= nq) { blk -= nq; in = k; out = k_out; w = wk; }
+    const int slab = blk / strips, strip = blk - slab * strips;
+    const int lc = threadIdx.x % LPR, p0 = threadIdx.x / LPR;
+    const int col = (strip * LPR + lc) * VEC;
+    const bool col_ok = col < S;
+    const int half = hd >> 1;
+    const size_t base = (size_t)slab * hd * S + col;
+    typename RawT<VEC>::type r0[CAP], r1[CAP];
+    float w0[CAP], w1[CAP];
+    float acc[1][VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc[0][j] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < CAP; kk++) {
+        const int rp = p0 + kk * PPS;
+        const bool ok = rp < half && col_ok;
+        r0[kk] = ok ? ld_raw<VEC, true>(in + base + (size_t)(2 * rp) * S) : raw_zero<VEC>();
+        r1[kk] = ok ? ld_raw<VEC, true>(in + base + (size_t)(2 * rp + 1) * S) : raw_zero<VEC>();
+        w0[kk] = ok ? w[2 * rp] : 0.f;
+        w1[kk] = ok ? w[2 * rp + 1] : 0.f;
+        float x0[VEC], x1[VEC];
+        unpack<VEC>(x0, r0[kk]);
+        unpack<VEC>(x1, r1[kk]);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            acc[0][j] += x0[j] * x0[j];
+            acc[0][j] += x1[j] * x1[j];
+        }
+    }
+    strip_reduce<VEC, LPR, THREADS, 1>(acc, lds);
+#pragma unroll
+    for (int kk = 0; kk < CAP; kk++) { forget<VEC>(r0[kk]); forget<VEC>(r1[kk]); }
+    float rr[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) rr[j] = 1.0f / sqrtf(acc[0][j] * invhd + eps);
+#pragma unroll
+    for (int kk = 0; kk < CAP; kk++) {
+        const int rp = p0 + kk * PPS;
+        if (rp < half && col_ok) {
+            float x0[VEC], x1[VEC], cs[VEC], sn[VEC], o0[VEC], o1[VEC];
+            unpack<VEC>(x0, r0[kk]);
+            unpack<VEC>(x1, r1[kk]);
+            ldtab<VEC>(cs, cos_t + (size_t)rp * S + col);
+            ldtab<VEC>(sn, sin_t + (size_t)rp * S + col);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                const float y0 = (x0[j] * rr[j]) * w0[kk], y1 = (x1[j] * rr[j]) * w1[kk];
+                o0[j] = y0 * cs[j] - y1 * sn[j];
+                o1[j] = y0 * sn[j] + y1 * cs[j];
+            }
+            stb<VEC>(out + base + (size_t)(2 * rp) * S, o0);
+            stb<VEC>(out + base + (size_t)(2 * rp + 1) * S, o1);
+        }
+    }
+}
+
+template <int VEC, int LPR, int THREADS, int CAP>
+__global__ __launch_bounds__(THREADS) void qknorm_rope_bwd_bf16_kernel(
+    bf16_t *dq, bf16_t *dk, float *__restrict__ part, const bf16_t *dq_out, const bf16_t *dk_out,
+    const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const float *__restrict__ wq,
+    const float *__restrict__ wk, int hd, int S, int strips, int nq, const float *__restrict__ cos_t,
+    const float *__restrict__ sin_t, float eps, float invhd, int variant) {
+    constexpr int PPS = THREADS / LPR;
+    constexpr int NW = THREADS / 64;
+    constexpr int G = LPR < 64 ? LPR : 64;
+    __shared__ float lds[NW * 2 * G * VEC];
+    int blk = blockIdx.x;
+    float *prt = part + (size_t)blk * hd;
+    const bf16_t *gin = dq_out, *xin = q;
+    const float *w = wq;
+    bf16_t *out = dq;
+    if (blk >= nq) { blk -= nq; gin = dk_out; xin = k; out = dk; w = wk; }
+    const int slab = blk / strips, strip = blk - slab * strips;
+    const int lc = threadIdx.x % LPR, p0 = threadIdx.x / LPR;
+    const int col = (strip * LPR + lc) * VEC;
+    const bool col_ok = col < S;
+    const int half = hd >> 1;
+    const size_t base = (size_t)slab * hd * S + col;
+    typename RawT<VEC>::type rx0[CAP], rx1[CAP], rg0[CAP], rg1[CAP];
+    float w0[CAP], w1[CAP];
+    float acc[2][VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc[0][j] = acc[1][j] = 0.f;
+
+    // un-rotated upstream gradient of pair kk (training/training_dynamic/cpu_ops.h:179-180); zero where masked
+    auto unrotate = [&](int kk, int rp, float (&d0)[VEC], float (&d1)[VEC]) {
+        float g0[VEC], g1[VEC], c[VEC], sn[VEC];
+        unpack<VEC>(g0, rg0[kk]);
+        unpack<VEC>(g1, rg1[kk]);
+        if (rp < half && col_ok) {
+            ldtab<VEC>(c, cos_t + (size_t)rp * S + col);
+            ldtab<VEC>(sn, sin_t + (size_t)rp * S + col);
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) c[j] = sn[j] = 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            d0[j] = g0[j] * c[j] + g1[j] * sn[j];
+            d1[j] = (-g0[j]) * sn[j] + g1[j] * c[j];
+        }
+    };
+
+#pragma unroll
+    for (int kk = 0; kk < CAP; kk++) {
+        const int rp = p0 + kk * PPS;
+        const bool ok = rp < half && col_ok;
+        const size_t o = base + (size_t)(2 * rp) * S;
+        rx0[kk] = ok ? ld_raw<VEC, true>(xin + o) : raw_zero<VEC>();
+        rx1[kk] = ok ? ld_raw<VEC, true>(xin + o + S) : raw_zero<VEC>();
+        rg0[kk] = ok ? ld_raw<VEC, true>(gin + o) : raw_zero<VEC>();
+        rg1[kk] = ok ? ld_raw<VEC, true>(gin + o + S) : raw_zero<VEC>();
+        w0[kk] = ok ? w[2 * rp] : 0.f;
+        w1[kk] = ok ? w[2 * rp + 1] : 0.f;
+        float x0[VEC], x1[VEC], d0[VEC], d1[VEC];
+        unpack<VEC>(x0, rx0[kk]);
+        unpack<VEC>(x1, rx1[kk]);
+        unrotate(kk, rp, d0, d1);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            acc[0][j] += x0[j] * x0[j];
+            acc[0][j] += x1[j] * x1[j];
+            acc[1][j] += (d0[j] * x0[j]) * w0[kk];
+            acc[1][j] += (d1[j] * x1[j]) * w1[kk];
+        }
+    }
+    strip_reduce<VEC, LPR, THREADS, 2>(acc, lds);
+#pragma unroll
+    for (int kk = 0; kk < CAP; kk++) { forget<VEC>(rx0[kk]); forget<VEC>(rx1[kk]); forget<VEC>(rg0[kk]); forget<VEC>(rg1[kk]); }
+    float rr[VEC], dotn[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        rr[j] = 1.0f / sqrtf(acc[0][j] * invhd + eps);
+        dotn[j] = acc[1][j] * ((rr[j] * rr[j]) * invhd);
+    }
+#pragma unroll
+    for (int kk = 0; kk < CAP; kk++) {
+        const int rp = p0 + kk * PPS;
+        if (rp < half) {   // uniform over each group of LPR lanes
+            float x0[VEC], x1[VEC], d0[VEC], d1[VEC], o0[VEC], o1[VEC];
+            unpack<VEC>(x0, rx0[kk]);
+            unpack<VEC>(x1, rx1[kk]);
+            unrotate(kk, rp, d0, d1);
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                if (variant == 0) {
+                    o0[j] = ((d0[j] - x0[j] * dotn[j]) * rr[j]) * w0[kk];
+                    o1[j] = ((d1[j] - x1[j] * dotn[j]) * rr[j]) * w1[kk];
+                } else {
+                    o0[j] = (d0[j] * w0[kk]) * rr[j] - (x0[j] * dotn[j]) * rr[j];
+                    o1[j] = (d1[j] * w1[kk]) * rr[j] - (x1[j] * dotn[j]) * rr[j];
+                }
+                s0 += (d0[j] * x0[j]) * rr[j];
+                s1 += (d1[j] * x1[j]) * rr[j];
+            }
+            if (col_ok) {
+                stb<VEC>(out + base + (size_t)(2 * rp) * S, o0);
+                stb<VEC>(out + base + (size_t)(2 * rp + 1) * S, o1);
+            }
+            s0 = group_sum<G>(s0);
+            s1 = group_sum<G>(s1);
+            if (lc == 0) {
+                prt[2 * rp] = s0;
+                prt[2 * rp + 1] = s1;
+            }
+        }
+    }
+}
+
+struct QkBf {
+    int vec, lpr, threads, cap;
+};
+
+// Row pairs must fit the register tile: at most two pairs per lane with 8-column lanes, four with 1-column lanes.
+bool pick_qk_bf(int hd, bool vec_ok, bool backward, QkBf &cfg) {
+    const int half = hd / 2;
+    if (!vec_ok) {
+        cfg = QkBf{1, 64, 1024, 4};
+        return half <= 64;
+    }
+    const int thr = backward ? 512 : 256;
+    for (int cap : {1, 2})
+        if ((thr / 4) * cap >= half) { cfg = QkBf{8, 4, thr, cap}; return true; }
+    if (512 >= half) { cfg = QkBf{8, 4, 1024, 2}; return true; }      // one pair per lane spills with 16 waves
+    return false;
+}
+
+#define QKBF_DISPATCH(KERNEL, cfg, grid, ...)                                                                            do {                                                                                                                     const int key = (cfg).vec * 100000 + (cfg).threads * 10 + (cfg).cap;                                                 switch (key) {                                                                                                           case 110244: hipLaunchKernelGGL((KERNEL<1, 64, 1024, 4>), grid, dim3(1024), 0, g_ctx.stream, __VA_ARGS__); break;              case 802561: hipLaunchKernelGGL((KERNEL<8, 4, 256, 1>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;                 case 802562: hipLaunchKernelGGL((KERNEL<8, 4, 256, 2>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;                 case 805121: hipLaunchKernelGGL((KERNEL<8, 4, 512, 1>), grid, dim3(512), 0, g_ctx.stream, __VA_ARGS__); break;                 case 805122: hipLaunchKernelGGL((KERNEL<8, 4, 512, 2>), grid, dim3(512), 0, g_ctx.stream, __VA_ARGS__); break;                 case 810241: hipLaunchKernelGGL((KERNEL<8, 4, 1024, 1>), grid, dim3(1024), 0, g_ctx.stream, __VA_ARGS__); break;               case 810242: hipLaunchKernelGGL((KERNEL<8, 4, 1024, 2>), grid, dim3(1024), 0, g_ctx.stream, __VA_ARGS__); break;               default: return mi355_fail("bf16 qknorm_rope: no kernel for tile key %d", key);                                  }                                                                                                                } while (0)
+
+int qk_shape(const char *who, int heads, int kv_heads, int hd, int S, int batch) {
+    if (hd <= 0 || (hd & 1) || S <= 0 || batch <= 0 || heads < 0 || kv_heads < 0 || heads + kv_heads == 0)
+        return mi355_fail("%s: bad shape heads=%d kv_heads=%d hd=%d S=%d batch=%d", who, heads, kv_heads, hd, S, batch);
+    return 0;
+}
+
 struct BfCfg {
     int vec, lpr, threads, cap;
 };
 
 // 8-column lanes when the rows allow 128-bit accesses; 4 lanes (64 bytes) per strip row; rows in registers
 // when one workgroup can hold them.
-BfCfg pick_bf(int C, bool vec_ok, bool backward) {
+BfCfg pick_bf(int C, bool vec_ok) {
     if (!vec_ok) return BfCfg{1, 64, 256, 0};
     const int threads = C >= 512 ? 1024 : 256;
     const int rps = threads / 4;
-    const int max_cap = backward ? 4 : 8;            // 8 floats per row and operand: 2 x 4 x 8 data registers backward
     for (int cap : {2, 4, 8})
-        if (cap <= max_cap && rps * cap >= C) return BfCfg{8, 4, threads, cap};
+        if (rps * cap >= C) return BfCfg{8, 4, threads, cap};
     return BfCfg{8, 4, threads, 0};
 }
 
@@ -446,7 +752,7 @@ MI355_API int mi355_rmsnorm_fwd_bf16_dev(uint16_t *y, const uint16_t *x, const f
     if (!mi355_ready("rmsnorm_fwd_bf16")) return -1;
     if (!y || !x || !w) return mi355_fail("rmsnorm_fwd_bf16: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_fwd_bf16: bad shape C=%d S=%d batch=%d", C, S, batch);
-    const BfCfg cfg = pick_bf(C, S % 8 == 0 && aligned16(x) && aligned16(y), false);
+    const BfCfg cfg = pick_bf(C, S % 8 == 0 && aligned16(x) && aligned16(y));
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
     BF_DISPATCH(rms_fwd_bf16_kernel, cfg, nblk, y, x, w, C, S, strips, nblk, eps, 1.0f / (float)C);
@@ -460,7 +766,7 @@ MI355_API int mi355_rmsnorm_bwd_bf16_dev(uint16_t *dx, float *dw, const uint16_t
     if (!dx || !dw || !dy || !x || !w) return mi355_fail("rmsnorm_bwd_bf16: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_bwd_bf16: bad shape C=%d S=%d batch=%d", C, S, batch);
     if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd_bf16: variant must be 0 or 1");
-    const BfCfg cfg = pick_bf(C, S % 8 == 0 && aligned16(x) && aligned16(dy) && aligned16(dx), true);
+    const BfCfg cfg = pick_bf(C, S % 8 == 0 && aligned16(x) && aligned16(dy) && aligned16(dx));
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
     float *part = mi355_dw_partials((size_t)nblk * C, dw, nullptr);
@@ -468,5 +774,74 @@ MI355_API int mi355_rmsnorm_bwd_bf16_dev(uint16_t *dx, float *dw, const uint16_t
     BF_DISPATCH(rms_bwd_bf16_kernel, cfg, nblk, dx, part, dy, x, w, C, S, strips, nblk, eps, 1.0f / (float)C, variant);
     LAUNCH_OK("rmsnorm_bwd_bf16");
     if (mi355_dw_submit(dw, part, nblk, C)) return -1;
+    return mi355_dw_op_end();
+}
+
+MI355_API int mi355_rope_bf16_dev(uint16_t *q_out, uint16_t *k_out, const uint16_t *q_in, const uint16_t *k_in, int heads,
+                                  int kv_heads, int hd, int S, int batch, const float *cos_dev, const float *sin_dev,
+                                  int dir) {
+    if (!mi355_ready("rope_bf16")) return -1;
+    if (qk_shape("rope_bf16", heads, kv_heads, hd, S, batch)) return -1;
+    if (!cos_dev || !sin_dev || (heads > 0 && (!q_out || !q_in)) || (kv_heads > 0 && (!k_out || !k_in)))
+        return mi355_fail("rope_bf16: NULL pointer");
+    if (dir != 1 && dir != -1) return mi355_fail("rope_bf16: dir must be +1 or -1");
+    const bool vec = S % 8 == 0 && aligned16(cos_dev) && aligned16(sin_dev) &&
+                     (heads == 0 || (aligned16(q_in) && aligned16(q_out))) &&
+                     (kv_heads == 0 || (aligned16(k_in) && aligned16(k_out)));
+    const size_t pair_rows = (size_t)batch * (heads + kv_heads) * (hd / 2);
+    const size_t total = pair_rows * (size_t)(vec ? S / 8 : S);
+    if (vec) hipLaunchKernelGGL(rope_bf16_kernel<8>, dim3(blocks_for(total)), dim3(BT), 0, g_ctx.stream, q_out, k_out, q_in, k_in, heads, kv_heads, hd, S, batch, cos_dev, sin_dev, (float)dir, total);
+    else hipLaunchKernelGGL(rope_bf16_kernel<1>, dim3(blocks_for(total)), dim3(BT), 0, g_ctx.stream, q_out, k_out, q_in, k_in, heads, kv_heads, hd, S, batch, cos_dev, sin_dev, (float)dir, total);
+    LAUNCH_OK("rope_bf16");
+    return 0;
+}
+
+MI355_API int mi355_qknorm_rope_fwd_bf16_dev(uint16_t *q_out, uint16_t *k_out, const uint16_t *q, const uint16_t *k,
+                                             const float *wq, const float *wk, int heads, int kv_heads, int hd, int S,
+                                             int batch, const float *cos_dev, const float *sin_dev, float eps) {
+    if (!mi355_ready("qknorm_rope_fwd_bf16")) return -1;
+    if (qk_shape("qknorm_rope_fwd_bf16", heads, kv_heads, hd, S, batch)) return -1;
+    if (!cos_dev || !sin_dev || (heads > 0 && (!q_out || !q || !wq)) || (kv_heads > 0 && (!k_out || !k || !wk)))
+        return mi355_fail("qknorm_rope_fwd_bf16: NULL pointer");
+    const bool vec_ok = S % 8 == 0 && aligned16(cos_dev) && aligned16(sin_dev) &&
+                        (heads == 0 || (aligned16(q) && aligned16(q_out))) &&
+                        (kv_heads == 0 || (aligned16(k) && aligned16(k_out)));
+    QkBf cfg;
+    if (!pick_qk_bf(hd, vec_ok, false, cfg))
+        return mi355_fail("qknorm_rope_fwd_bf16: head size %d does not fit the register tile for this layout", hd);
+    const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
+    const int nq = batch * heads * strips, nk = batch * kv_heads * strips;
+    QKBF_DISPATCH(qknorm_rope_fwd_bf16_kernel, cfg, dim3(nq + nk), q_out, k_out, q, k, wq, wk, hd, S, strips, nq, cos_dev,
+                  sin_dev, eps, 1.0f / (float)hd);
+    LAUNCH_OK("qknorm_rope_fwd_bf16");
+    return 0;
+}
+
+MI355_API int mi355_qknorm_rope_bwd_bf16_dev(uint16_t *dq, uint16_t *dk, float *dwq, float *dwk, const uint16_t *dq_out,
+                                             const uint16_t *dk_out, const uint16_t *q, const uint16_t *k,
+                                             const float *wq, const float *wk, int heads, int kv_heads, int hd, int S,
+                                             int batch, const float *cos_dev, const float *sin_dev, float eps,
+                                             int variant) {
+    if (!mi355_ready("qknorm_rope_bwd_bf16")) return -1;
+    if (qk_shape("qknorm_rope_bwd_bf16", heads, kv_heads, hd, S, batch)) return -1;
+    if (variant != 0 && variant != 1) return mi355_fail("qknorm_rope_bwd_bf16: variant must be 0 or 1");
+    if (!cos_dev || !sin_dev || (heads > 0 && (!dq || !dwq || !dq_out || !q || !wq)) ||
+        (kv_heads > 0 && (!dk || !dwk || !dk_out || !k || !wk)))
+        return mi355_fail("qknorm_rope_bwd_bf16: NULL pointer");
+    const bool vec_ok = S % 8 == 0 && aligned16(cos_dev) && aligned16(sin_dev) &&
+                        (heads == 0 || (aligned16(q) && aligned16(dq) && aligned16(dq_out))) &&
+                        (kv_heads == 0 || (aligned16(k) && aligned16(dk) && aligned16(dk_out)));
+    QkBf cfg;
+    if (!pick_qk_bf(hd, vec_ok, true, cfg))
+        return mi355_fail("qknorm_rope_bwd_bf16: head size %d does not fit the register tile for this layout", hd);
+    const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
+    const int nq = batch * heads * strips, nk = batch * kv_heads * strips;
+    float *part = mi355_dw_partials((size_t)(nq + nk) * hd, nq > 0 ? dwq : nullptr, nk > 0 ? dwk : nullptr);
+    if (!part) return -1;
+    QKBF_DISPATCH(qknorm_rope_bwd_bf16_kernel, cfg, dim3(nq + nk), dq, dk, part, dq_out, dk_out, q, k, wq, wk, hd, S,
+                  strips, nq, cos_dev, sin_dev, eps, 1.0f / (float)hd, variant);
+    LAUNCH_OK("qknorm_rope_bwd_bf16");
+    if (nq > 0 && mi355_dw_submit(dwq, part, nq, hd)) return -1;
+    if (nk > 0 && mi355_dw_submit(dwk, part + (size_t)nq * hd, nk, hd)) return -1;
     return mi355_dw_op_end();
 }

@@ -84,6 +84,17 @@ int mi355_swiglu_fwd_bf16_dev(uint16_t *out, const uint16_t *h1, const uint16_t 
 int mi355_swiglu_bwd_bf16_dev(uint16_t *dh1, uint16_t *dh3, const uint16_t *dsilu, const uint16_t *h1,
                               const uint16_t *h3, size_t n);
 int mi355_axpby_bf16_dev(uint16_t *y, const uint16_t *a, const uint16_t *b, float alpha, size_t n, int mode);
+int mi355_rope_bf16_dev(uint16_t *q_out, uint16_t *k_out, const uint16_t *q_in, const uint16_t *k_in, int heads,
+                        int kv_heads, int hd, int S, int batch, const float *cos_dev, const float *sin_dev, int dir);
+/* The head size must fit the register tile: hd <= 1024 with rows of a multiple of 8 columns and 16-byte aligned
+ * pointers, hd <= 128 otherwise (the fp32 entry points have no such limit). */
+int mi355_qknorm_rope_fwd_bf16_dev(uint16_t *q_out, uint16_t *k_out, const uint16_t *q, const uint16_t *k,
+                                   const float *wq, const float *wk, int heads, int kv_heads, int hd, int S, int batch,
+                                   const float *cos_dev, const float *sin_dev, float eps);
+int mi355_qknorm_rope_bwd_bf16_dev(uint16_t *dq, uint16_t *dk, float *dwq, float *dwk, const uint16_t *dq_out,
+                                   const uint16_t *dk_out, const uint16_t *q, const uint16_t *k, const float *wq,
+                                   const float *wk, int heads, int kv_heads, int hd, int S, int batch,
+                                   const float *cos_dev, const float *sin_dev, float eps, int variant);
 
 /* Graphs: record a launch-bound sequence of device-resident ops once, replay it as one submission.  No
  * counterpart in the reference (its ops are synchronous CPU calls).  Between begin and end the *_dev ops are

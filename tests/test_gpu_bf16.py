@@ -90,3 +90,45 @@ def test_bf16_bad_arguments(br):
     assert br.lib.mi355_axpby_bf16_dev(a.ptr, a.ptr, None, 1.0, 64, 0) == -1
     assert br.lib.mi355_cvt_f32_bf16_dev(a.ptr, 4, w.ptr, 8, 1, 8) == -1
     assert "bf16" in br.last_error()
+
+
+@pytest.mark.parametrize("B,heads,kvh,hd,S", [(16, 16, 8, 128, 256), (2, 12, 12, 64, 256), (2, 3, 2, 16, 24), (1, 2, 1, 8, 10),
+                                              (1, 2, 1, 512, 16), (2, 4, 2, 256, 32), (1, 1, 1, 1024, 8), (1, 4, 0, 32, 16)])
+def test_rope_and_qknorm_rope_bf16(br, B, heads, kvh, hd, S):
+    print("[case] bf16 qknorm_rope B=%d heads=%d/%d hd=%d S=%d" % (B, heads, kvh, hd, S), flush=True)
+    theta = 1e6
+    kv = max(kvh, 1)
+    (qb, q), (kb, k) = bf(H.normal(230, (B, heads * hd, S))), bf(H.normal(231, (B, kv * hd, S)))
+    (gqb, gq), (gkb, gk) = bf(H.normal(232, q.shape)), bf(H.normal(233, k.shape))
+    wq = H.normal(234, hd, 1.0, 0.02); wk = H.normal(235, hd, 1.0, 0.02)
+    dwq0 = H.normal(236, hd); dwk0 = H.normal(237, hd)
+    cd, sd = br.rope_tables_dev(S, hd, theta)
+    qd, kd, gqd, gkd, wqd, wkd = (dev(br, a) for a in (qb, kb, gqb, gkb, wq, wk))
+    K = lambda a: a.ptr if kvh else None
+    # stand-alone rotation, both directions
+    for direction in (+1, -1):
+        qo, ko = br.DevArray(q.shape, np.uint16), br.DevArray(k.shape, np.uint16)
+        br.check(br.lib.mi355_rope_bf16_dev(qo.ptr, K(ko), qd.ptr, K(kd), heads, kvh, hd, S, B, cd, sd, direction))
+        assert H.rel_err(back(qo), O.rope(q, hd, theta, direction)) <= TOL16
+        if kvh:
+            assert H.rel_err(back(ko), O.rope(k, hd, theta, direction)) <= TOL16
+    small = hd / 2 > 64 and S % 8 != 0          # beyond the scalar-column register tile: refused
+    qo, ko = br.DevArray(q.shape, np.uint16), br.DevArray(k.shape, np.uint16)
+    rc = br.lib.mi355_qknorm_rope_fwd_bf16_dev(qo.ptr, K(ko), qd.ptr, K(kd), wqd.ptr, K(wkd), heads, kvh, hd, S, B, cd, sd, 1e-5)
+    assert rc == (-1 if small else 0)
+    if small:
+        return
+    assert H.rel_err(back(qo), O.qknorm_rope_fwd(q, wq, hd, theta)) <= TOL16
+    if kvh:
+        assert H.rel_err(back(ko), O.qknorm_rope_fwd(k, wk, hd, theta)) <= TOL16
+    for variant in (0, 1):
+        dq, dk = br.DevArray(q.shape, np.uint16), br.DevArray(k.shape, np.uint16)
+        dwq, dwk = dev(br, dwq0), dev(br, dwk0)
+        br.check(br.lib.mi355_qknorm_rope_bwd_bf16_dev(dq.ptr, K(dk), dwq.ptr, K(dwk), gqd.ptr, K(gkd), qd.ptr, K(kd), wqd.ptr,
+                                                       K(wkd), heads, kvh, hd, S, B, cd, sd, 1e-5, variant))
+        rdq, rdwq = O.qknorm_rope_bwd(gq, q, wq, hd, theta, variant=variant, dw=dwq0)
+        tol = TOL16 if hd >= 16 else 2e-2
+        assert H.rel_err(back(dq), rdq) <= tol and H.rel_err(dwq.numpy(), rdwq) <= 1e-5
+        if kvh:
+            rdk, rdwk = O.qknorm_rope_bwd(gk, k, wk, hd, theta, variant=variant, dw=dwk0)
+            assert H.rel_err(back(dk), rdk) <= tol and H.rel_err(dwk.numpy(), rdwk) <= 1e-5
