@@ -106,6 +106,7 @@ SIGNATURES = {
     "mi355_swiglu_fwd_bf16_dev": (_i, [_p, _p, _p, _z]),
     "mi355_swiglu_bwd_bf16_dev": (_i, [_p, _p, _p, _p, _p, _z]),
     "mi355_axpby_bf16_dev": (_i, [_p, _p, _p, _f, _z, _i]),
+    "mi355_softmax_ce_bf16_dev": (_i, [_p, _p, _p, _p, _i, _i, _f]),
     "mi355_rope_bf16_dev": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _i]),
     "mi355_qknorm_rope_fwd_bf16_dev": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _f]),
     "mi355_qknorm_rope_bwd_bf16_dev": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _f, _i]),

@@ -44,10 +44,60 @@ __device__ __forceinline__ void ld_cols_nt(float (&r)[VEC], const float *p) {
     }
 }
 
-// grid: (row blocks, column strips of 64*VEC)
+// bfloat16 logits (the optional bf16-storage variant): four columns = one 64-bit access; widened to fp32 here,
+// so everything below is the same arithmetic for both storage types.
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float bf_widen(unsigned bits16) { return __uint_as_float(bits16 << 16); }
+__device__ __forceinline__ unsigned bf_narrow(float f) {       // round to nearest even; NaN stays NaN
+    const unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
 template <int VEC>
+__device__ __forceinline__ void ld_cols(float (&r)[VEC], const uint16_t *p) {
+    if constexpr (VEC == 4) {
+        const v2u w = *reinterpret_cast<const v2u *>(p);
+        r[0] = bf_widen(w[0] & 0xffffu); r[1] = bf_widen(w[0] >> 16);
+        r[2] = bf_widen(w[1] & 0xffffu); r[3] = bf_widen(w[1] >> 16);
+    } else {
+        r[0] = bf_widen(*p);
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void ld_cols_nt(float (&r)[VEC], const uint16_t *p) {
+    if constexpr (VEC == 4) {
+        const v2u w = __builtin_nontemporal_load(reinterpret_cast<const v2u *>(p));
+        r[0] = bf_widen(w[0] & 0xffffu); r[1] = bf_widen(w[0] >> 16);
+        r[2] = bf_widen(w[1] & 0xffffu); r[3] = bf_widen(w[1] >> 16);
+    } else {
+        r[0] = bf_widen(*p);
+    }
+}
+__device__ __forceinline__ float ld_one(const float *p) { return *p; }
+__device__ __forceinline__ float ld_one(const uint16_t *p) { return bf_widen(*p); }
+template <int VEC>
+__device__ __forceinline__ void st_cols(float *p, const float (&o)[VEC]) {
+    if constexpr (VEC == 4) {
+        v4f t = {o[0], o[1], o[2], o[3]};
+        st4_nt(p, t);
+    } else {
+        *p = o[0];
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void st_cols(uint16_t *p, const float (&o)[VEC]) {
+    if constexpr (VEC == 4) {
+        v2u w = {bf_narrow(o[0]) | (bf_narrow(o[1]) << 16), bf_narrow(o[2]) | (bf_narrow(o[3]) << 16)};
+        __builtin_nontemporal_store(w, reinterpret_cast<v2u *>(p));
+    } else {
+        *p = (uint16_t)bf_narrow(o[0]);
+    }
+}
+
+// grid: (row blocks, column strips of 64*VEC)
+template <int VEC, typename T>
 __global__ __launch_bounds__(CE_THREADS) void ce_partial_kernel(float *__restrict__ pm, float *__restrict__ pl,
-                                                                const float *__restrict__ logits, int V, int S,
+                                                                const T *__restrict__ logits, int V, int S,
                                                                 int rows_per_block) {
     __shared__ float sm[CE_WAVES][64 * VEC], sl[CE_WAVES][64 * VEC];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -109,10 +159,11 @@ __global__ __launch_bounds__(CE_THREADS) void ce_partial_kernel(float *__restric
 
 // One workgroup per 64 columns: 16 groups of threads each merge an interleaved subset of the row
 // blocks, then the 16 partial results are merged in order.
+template <typename T>
 __global__ __launch_bounds__(1024) void ce_combine_kernel(float *__restrict__ colM, float *__restrict__ colInv,
                                                           float *__restrict__ colLoss, const float *__restrict__ pm,
                                                           const float *__restrict__ pl,
-                                                          const float *__restrict__ logits,
+                                                          const T *__restrict__ logits,
                                                           const int32_t *__restrict__ targets, int V, int S,
                                                           int nblk) {
     __shared__ float sm[16][64], sl[16][64];
@@ -154,15 +205,15 @@ __global__ __launch_bounds__(1024) void ce_combine_kernel(float *__restrict__ co
         const int tgt = targets[t];
         float loss = 0.f;
         if (tgt >= 0 && tgt < V) {
-            const float p = exp_neg(logits[(size_t)tgt * S + t] - M) * inv;
+            const float p = exp_neg(ld_one(logits + (size_t)tgt * S + t) - M) * inv;
             loss = -logf(p + 1e-10f);
         }
         colLoss[t] = loss;
     }
 }
 
-template <int VEC>
-__global__ __launch_bounds__(CE_THREADS) void ce_grad_kernel(float *dlogits, const float *logits,
+template <int VEC, typename T>
+__global__ __launch_bounds__(CE_THREADS) void ce_grad_kernel(T *dlogits, const T *logits,
                                                              const float *__restrict__ colM,
                                                              const float *__restrict__ colInv,
                                                              const int32_t *__restrict__ targets, int V, int S,
@@ -219,35 +270,30 @@ __global__ __launch_bounds__(CE_THREADS) void ce_grad_kernel(float *dlogits, con
                     if (grad_scale != 1.0f) p = p * grad_scale;
                     o[j] = p;
                 }
-                float *dst = dlogits + (size_t)v * S + col;
-                if constexpr (VEC == 4) {
-                    v4f t = {o[0], o[1], o[2], o[3]};
-                    st4_nt(dst, t);
-                } else {
-                    *dst = o[0];
-                }
+                st_cols<VEC>(dlogits + (size_t)v * S + col, o);
             }
         }
     }
 }
 
-}   // namespace
-
-MI355_API int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float *logits, const int32_t *targets, int V,
-                                   int S, float grad_scale) {
-    if (!mi355_ready("softmax_ce")) return -1;
-    if (!dlogits || !loss_dev || !logits || !targets) return mi355_fail("softmax_ce: NULL pointer");
-    if (V <= 0 || S <= 0) return mi355_fail("softmax_ce: bad shape V=%d S=%d", V, S);
+template <typename T>
+int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const int32_t *targets, int V, int S,
+           float grad_scale) {
+    if (!mi355_ready(who)) return -1;
+    if (!dlogits || !loss_dev || !logits || !targets) return mi355_fail("%s: NULL pointer", who);
+    if (V <= 0 || S <= 0) return mi355_fail("%s: bad shape V=%d S=%d", who, V, S);
     // rows per workgroup: about 600 workgroups per column strip (2+ per compute unit), between one and
     // four 64-row register tiles; 256 rows measured best at V = 151936
     int rpb = g_ctx.ce_rows > 0 ? g_ctx.ce_rows : (int)ceil_div((size_t)V, 600);
     rpb = (int)ceil_div((size_t)rpb, CE_TILE_ROWS) * CE_TILE_ROWS;
     if (g_ctx.ce_rows <= 0 && rpb > 4 * CE_TILE_ROWS) rpb = 4 * CE_TILE_ROWS;
     const int nblk = (int)ceil_div((size_t)V, (size_t)rpb);
-    const bool vec_ok = (S % 4 == 0) && aligned16(logits) && aligned16(dlogits);
+    // four columns per lane: 16 bytes of fp32, 8 bytes of bf16
+    const uintptr_t mask = 4 * sizeof(T) - 1;
+    const bool vec_ok = (S % 4 == 0) && (((uintptr_t)logits | (uintptr_t)dlogits) & mask) == 0;
     const int vec = vec_ok ? 4 : 1;
     const int strips = (int)ceil_div((size_t)S, (size_t)64 * vec);
-    if (strips > 65535) return mi355_fail("softmax_ce: S too large");
+    if (strips > 65535) return mi355_fail("%s: S too large", who);
 
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
     const size_t part_b = al((size_t)nblk * S * sizeof(float)), col_b = al((size_t)S * sizeof(float));
@@ -258,18 +304,31 @@ MI355_API int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float 
     float *colLoss = (float *)(ws + 2 * part_b + 2 * col_b);
 
     const dim3 grid((unsigned)nblk, (unsigned)strips);
-    if (vec_ok) hipLaunchKernelGGL((ce_partial_kernel<4>), grid, dim3(CE_THREADS), 0, g_ctx.stream, pm, pl, logits, V, S, rpb);
-    else hipLaunchKernelGGL((ce_partial_kernel<1>), grid, dim3(CE_THREADS), 0, g_ctx.stream, pm, pl, logits, V, S, rpb);
+    if (vec_ok) hipLaunchKernelGGL((ce_partial_kernel<4, T>), grid, dim3(CE_THREADS), 0, g_ctx.stream, pm, pl, logits, V, S, rpb);
+    else hipLaunchKernelGGL((ce_partial_kernel<1, T>), grid, dim3(CE_THREADS), 0, g_ctx.stream, pm, pl, logits, V, S, rpb);
     LAUNCH_OK("softmax_ce partial");
-    hipLaunchKernelGGL(ce_combine_kernel, dim3((unsigned)ceil_div((size_t)S, 64)), dim3(1024), 0, g_ctx.stream, colM,
+    hipLaunchKernelGGL(ce_combine_kernel<T>, dim3((unsigned)ceil_div((size_t)S, 64)), dim3(1024), 0, g_ctx.stream, colM,
                        colInv, colLoss, pm, pl, logits, targets, V, S, nblk);
     LAUNCH_OK("softmax_ce combine");
     if (vec_ok)
-        hipLaunchKernelGGL((ce_grad_kernel<4>), grid, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
+        hipLaunchKernelGGL((ce_grad_kernel<4, T>), grid, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
                            targets, V, S, rpb, 1.0f / (float)S, grad_scale, loss_dev, colLoss);
     else
-        hipLaunchKernelGGL((ce_grad_kernel<1>), grid, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
+        hipLaunchKernelGGL((ce_grad_kernel<1, T>), grid, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
                            targets, V, S, rpb, 1.0f / (float)S, grad_scale, loss_dev, colLoss);
     LAUNCH_OK("softmax_ce grad");
     return 0;
+}
+
+}   // namespace
+
+MI355_API int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float *logits, const int32_t *targets, int V,
+                                   int S, float grad_scale) {
+    return ce_run<float>("softmax_ce", dlogits, loss_dev, logits, targets, V, S, grad_scale);
+}
+
+// bfloat16 logits and gradient (bit patterns as uint16_t); the loss and every intermediate stay fp32.
+MI355_API int mi355_softmax_ce_bf16_dev(uint16_t *dlogits, float *loss_dev, const uint16_t *logits, const int32_t *targets,
+                                        int V, int S, float grad_scale) {
+    return ce_run<uint16_t>("softmax_ce_bf16", dlogits, loss_dev, logits, targets, V, S, grad_scale);
 }

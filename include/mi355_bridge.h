@@ -84,6 +84,8 @@ int mi355_swiglu_fwd_bf16_dev(uint16_t *out, const uint16_t *h1, const uint16_t 
 int mi355_swiglu_bwd_bf16_dev(uint16_t *dh1, uint16_t *dh3, const uint16_t *dsilu, const uint16_t *h1,
                               const uint16_t *h3, size_t n);
 int mi355_axpby_bf16_dev(uint16_t *y, const uint16_t *a, const uint16_t *b, float alpha, size_t n, int mode);
+int mi355_softmax_ce_bf16_dev(uint16_t *dlogits, float *loss_dev, const uint16_t *logits, const int32_t *targets,
+                              int V, int S, float grad_scale);
 int mi355_rope_bf16_dev(uint16_t *q_out, uint16_t *k_out, const uint16_t *q_in, const uint16_t *k_in, int heads,
                         int kv_heads, int hd, int S, int batch, const float *cos_dev, const float *sin_dev, int dir);
 /* The head size must fit the register tile: hd <= 1024 with rows of a multiple of 8 columns and 16-byte aligned

@@ -132,3 +132,21 @@ def test_rope_and_qknorm_rope_bf16(br, B, heads, kvh, hd, S):
         if kvh:
             rdk, rdwk = O.qknorm_rope_bwd(gk, k, wk, hd, theta, variant=variant, dw=dwk0)
             assert H.rel_err(back(dk), rdk) <= tol and H.rel_err(dwk.numpy(), rdwk) <= 1e-5
+
+
+@pytest.mark.parametrize("V,S", [(32000, 256), (151936, 256), (37, 12), (1000, 5), (300, 1024)])
+def test_softmax_ce_bf16(br, V, S):
+    print("[case] bf16 softmax_ce V=%d S=%d" % (V, S), flush=True)
+    lb, logits = bf(H.normal(240, (V, S), 0, 2.0))
+    tgt = np.random.default_rng(241).integers(0, V, S).astype(np.int32)
+    if S > 8:
+        tgt[3] = V; tgt[5] = -1                                         # out-of-range targets are skipped
+    ld, td = dev(br, lb), dev(br, tgt)
+    for scale in (1.0, 256.0):
+        dl, lossd = br.DevArray((V, S), np.uint16), br.DevArray(1)
+        br.check(br.lib.mi355_softmax_ce_bf16_dev(dl.ptr, lossd.ptr, ld.ptr, td.ptr, V, S, scale))
+        rl, rd = O.cross_entropy(logits, tgt, grad_scale=scale)
+        assert abs(float(lossd.numpy()[0]) - rl) <= 1e-5 * abs(rl)        # fp32 all the way
+        assert H.rel_err(back(dl), rd) <= TOL16
+    br.check(br.lib.mi355_softmax_ce_bf16_dev(ld.ptr, lossd.ptr, ld.ptr, td.ptr, V, S, 1.0))     # in place
+    assert H.rel_err(back(ld), O.cross_entropy(logits, tgt)[1]) <= TOL16
