@@ -609,7 +609,9 @@ struct QkBf {
     int vec, lpr, threads, cap;
 };
 
-// Row pairs must fit the register tile: at most two pairs per lane with 8-column lanes, four with 1-column lanes.
+// Widest strip whose row pairs fit the (packed) register tile: 16 lanes x 8 columns = 256-byte row segments first;
+// 64-byte segments run at little more than half the rate.  One-column lanes (ragged S, unaligned pointers) hold
+// at most four pairs.
 bool pick_qk_bf(int hd, bool vec_ok, bool backward, QkBf &cfg) {
     const int half = hd / 2;
     if (!vec_ok) {
@@ -617,13 +619,34 @@ bool pick_qk_bf(int hd, bool vec_ok, bool backward, QkBf &cfg) {
         return half <= 64;
     }
     const int thr = backward ? 512 : 256;
-    for (int cap : {1, 2})
-        if ((thr / 4) * cap >= half) { cfg = QkBf{8, 4, thr, cap}; return true; }
-    if (512 >= half) { cfg = QkBf{8, 4, 1024, 2}; return true; }      // one pair per lane spills with 16 waves
+    for (int lpr : {16, 8, 4})
+        for (int cap : {1, 2, 4})
+            if ((thr / lpr) * cap >= half) { cfg = QkBf{8, lpr, thr, cap}; return true; }
+    if (512 >= half) { cfg = QkBf{8, 4, 1024, 2}; return true; }
     return false;
 }
 
-#define QKBF_DISPATCH(KERNEL, cfg, grid, ...)                                                                            do {                                                                                                                     const int key = (cfg).vec * 100000 + (cfg).threads * 10 + (cfg).cap;                                                 switch (key) {                                                                                                           case 110244: hipLaunchKernelGGL((KERNEL<1, 64, 1024, 4>), grid, dim3(1024), 0, g_ctx.stream, __VA_ARGS__); break;              case 802561: hipLaunchKernelGGL((KERNEL<8, 4, 256, 1>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;                 case 802562: hipLaunchKernelGGL((KERNEL<8, 4, 256, 2>), grid, dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;                 case 805121: hipLaunchKernelGGL((KERNEL<8, 4, 512, 1>), grid, dim3(512), 0, g_ctx.stream, __VA_ARGS__); break;                 case 805122: hipLaunchKernelGGL((KERNEL<8, 4, 512, 2>), grid, dim3(512), 0, g_ctx.stream, __VA_ARGS__); break;                 case 810241: hipLaunchKernelGGL((KERNEL<8, 4, 1024, 1>), grid, dim3(1024), 0, g_ctx.stream, __VA_ARGS__); break;               case 810242: hipLaunchKernelGGL((KERNEL<8, 4, 1024, 2>), grid, dim3(1024), 0, g_ctx.stream, __VA_ARGS__); break;               default: return mi355_fail("bf16 qknorm_rope: no kernel for tile key %d", key);                                  }                                                                                                                } while (0)
+#define QKBF_CASE(KERNEL, V, L, T, CP, grid, ...)                                                                    \
+    case (V) * 1000000 + (L) * 10000 + ((T) / 256) * 100 + (CP):                                                     \
+        hipLaunchKernelGGL((KERNEL<V, L, T, CP>), grid, dim3(T), 0, g_ctx.stream, __VA_ARGS__);                      \
+        break;
+#define QKBF_DISPATCH(KERNEL, cfg, grid, ...)                                                                        \
+    do {                                                                                                             \
+        switch ((cfg).vec * 1000000 + (cfg).lpr * 10000 + ((cfg).threads / 256) * 100 + (cfg).cap) {                 \
+            QKBF_CASE(KERNEL, 1, 64, 1024, 4, grid, __VA_ARGS__)                                                     \
+            QKBF_CASE(KERNEL, 8, 16, 256, 1, grid, __VA_ARGS__) QKBF_CASE(KERNEL, 8, 16, 256, 2, grid, __VA_ARGS__)  \
+            QKBF_CASE(KERNEL, 8, 16, 256, 4, grid, __VA_ARGS__) QKBF_CASE(KERNEL, 8, 16, 512, 1, grid, __VA_ARGS__)  \
+            QKBF_CASE(KERNEL, 8, 16, 512, 2, grid, __VA_ARGS__) QKBF_CASE(KERNEL, 8, 16, 512, 4, grid, __VA_ARGS__)  \
+            QKBF_CASE(KERNEL, 8, 8, 256, 1, grid, __VA_ARGS__) QKBF_CASE(KERNEL, 8, 8, 256, 2, grid, __VA_ARGS__)    \
+            QKBF_CASE(KERNEL, 8, 8, 256, 4, grid, __VA_ARGS__) QKBF_CASE(KERNEL, 8, 8, 512, 1, grid, __VA_ARGS__)    \
+            QKBF_CASE(KERNEL, 8, 8, 512, 2, grid, __VA_ARGS__) QKBF_CASE(KERNEL, 8, 8, 512, 4, grid, __VA_ARGS__)    \
+            QKBF_CASE(KERNEL, 8, 4, 256, 1, grid, __VA_ARGS__) QKBF_CASE(KERNEL, 8, 4, 256, 2, grid, __VA_ARGS__)    \
+            QKBF_CASE(KERNEL, 8, 4, 256, 4, grid, __VA_ARGS__) QKBF_CASE(KERNEL, 8, 4, 512, 1, grid, __VA_ARGS__)    \
+            QKBF_CASE(KERNEL, 8, 4, 512, 2, grid, __VA_ARGS__) QKBF_CASE(KERNEL, 8, 4, 512, 4, grid, __VA_ARGS__)    \
+            QKBF_CASE(KERNEL, 8, 4, 1024, 2, grid, __VA_ARGS__)                                                      \
+            default: return mi355_fail("bf16 qknorm_rope: no kernel for this tile");                                 \
+        }                                                                                                            \
+    } while (0)
 
 int qk_shape(const char *who, int heads, int kv_heads, int hd, int S, int batch) {
     if (hd <= 0 || (hd & 1) || S <= 0 || batch <= 0 || heads < 0 || kv_heads < 0 || heads + kv_heads == 0)
@@ -635,31 +658,36 @@ struct BfCfg {
     int vec, lpr, threads, cap;
 };
 
-// 8-column lanes when the rows allow 128-bit accesses; 4 lanes (64 bytes) per strip row; rows in registers
-// when one workgroup can hold them.
+// 8-column lanes when the rows allow 128-bit accesses; rows in (packed) registers when one workgroup can hold
+// them, else two sweeps.  The rms_lpr / rms_threads knobs override the strip width and workgroup size.
 BfCfg pick_bf(int C, bool vec_ok) {
     if (!vec_ok) return BfCfg{1, 64, 256, 0};
-    const int threads = C >= 512 ? 1024 : 256;
-    const int rps = threads / 4;
+    int lpr = g_ctx.rms_lpr == 8 ? 8 : 4;
+    int threads = g_ctx.rms_threads == 256 || g_ctx.rms_threads == 512 || g_ctx.rms_threads == 1024
+                      ? g_ctx.rms_threads
+                      : (C >= 512 ? 1024 : 256);   // measured at C = 1024, 16 x 256 columns: 11.0 / 20.5 us forward / backward with
+                                                   // 16 waves, 12.6 / 23.0 with 8, 15.1 / 25.7 with 128-byte strips
+    const int rps = threads / lpr;
     for (int cap : {2, 4, 8})
-        if (rps * cap >= C) return BfCfg{8, 4, threads, cap};
-    return BfCfg{8, 4, threads, 0};
+        if (rps * cap >= C) return BfCfg{8, lpr, threads, cap};
+    return BfCfg{8, lpr, threads, 0};
 }
 
+#define BF_CASE(KERNEL, V, L, T, CP, nblk, ...)                                                                      \
+    case (V) * 1000000 + (L) * 10000 + ((T) / 256) * 100 + (CP):                                                     \
+        hipLaunchKernelGGL((KERNEL<V, L, T, CP>), dim3(nblk), dim3(T), 0, g_ctx.stream, __VA_ARGS__);                \
+        break;
+#define BF_CASES4(KERNEL, L, T, nblk, ...)                                                                           \
+    BF_CASE(KERNEL, 8, L, T, 0, nblk, __VA_ARGS__) BF_CASE(KERNEL, 8, L, T, 2, nblk, __VA_ARGS__)                    \
+    BF_CASE(KERNEL, 8, L, T, 4, nblk, __VA_ARGS__) BF_CASE(KERNEL, 8, L, T, 8, nblk, __VA_ARGS__)
 #define BF_DISPATCH(KERNEL, cfg, nblk, ...)                                                                          \
     do {                                                                                                             \
-        const int key = (cfg).vec * 100000 + (cfg).threads * 10 + (cfg).cap;                                         \
-        switch (key) {                                                                                               \
-            case 102560: hipLaunchKernelGGL((KERNEL<1, 64, 256, 0>), dim3(nblk), dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;   \
-            case 802560: hipLaunchKernelGGL((KERNEL<8, 4, 256, 0>), dim3(nblk), dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;    \
-            case 802562: hipLaunchKernelGGL((KERNEL<8, 4, 256, 2>), dim3(nblk), dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;    \
-            case 802564: hipLaunchKernelGGL((KERNEL<8, 4, 256, 4>), dim3(nblk), dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;    \
-            case 802568: hipLaunchKernelGGL((KERNEL<8, 4, 256, 8>), dim3(nblk), dim3(256), 0, g_ctx.stream, __VA_ARGS__); break;    \
-            case 810240: hipLaunchKernelGGL((KERNEL<8, 4, 1024, 0>), dim3(nblk), dim3(1024), 0, g_ctx.stream, __VA_ARGS__); break;  \
-            case 810242: hipLaunchKernelGGL((KERNEL<8, 4, 1024, 2>), dim3(nblk), dim3(1024), 0, g_ctx.stream, __VA_ARGS__); break;  \
-            case 810244: hipLaunchKernelGGL((KERNEL<8, 4, 1024, 4>), dim3(nblk), dim3(1024), 0, g_ctx.stream, __VA_ARGS__); break;  \
-            case 810248: hipLaunchKernelGGL((KERNEL<8, 4, 1024, 8>), dim3(nblk), dim3(1024), 0, g_ctx.stream, __VA_ARGS__); break;  \
-            default: return mi355_fail("bf16 rmsnorm: no kernel for tile key %d", key);                              \
+        switch ((cfg).vec * 1000000 + (cfg).lpr * 10000 + ((cfg).threads / 256) * 100 + (cfg).cap) {                 \
+            BF_CASE(KERNEL, 1, 64, 256, 0, nblk, __VA_ARGS__)                                                        \
+            BF_CASES4(KERNEL, 4, 256, nblk, __VA_ARGS__) BF_CASES4(KERNEL, 4, 512, nblk, __VA_ARGS__)                \
+            BF_CASES4(KERNEL, 4, 1024, nblk, __VA_ARGS__) BF_CASES4(KERNEL, 8, 256, nblk, __VA_ARGS__)               \
+            BF_CASES4(KERNEL, 8, 512, nblk, __VA_ARGS__) BF_CASES4(KERNEL, 8, 1024, nblk, __VA_ARGS__)               \
+            default: return mi355_fail("bf16 rmsnorm: no kernel for this tile");                                     \
         }                                                                                                            \
     } while (0)
 

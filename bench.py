@@ -41,43 +41,78 @@ S110 = dict(C=768, H=2048, heads=12, kv_heads=12, hd=64, S=256, batch=1, layers=
             int8_shape=(1024, 4096), qk_norm=False, name="stories110m")
 
 
-def alg_bytes(cfg):
-    """Algorithmic bytes per launch of each op (fp32 = 4 B; St = batch*S columns)."""
+def alg_bytes(cfg, a=4):
+    """Algorithmic bytes per launch of each op (a = bytes per activation: 4 for fp32, 2 for bf16 storage; norm
+    weights and weight gradients are always fp32; St = batch*S columns)."""
     C, H, S, B = cfg["C"], cfg["H"], cfg["S"], cfg["batch"]
     St = B * S
     qkd = (cfg["heads"] + cfg["kv_heads"]) * cfg["hd"]
     V = cfg["V"]
     n8 = cfg["int8_shape"][0] * cfg["int8_shape"][1]
     return {
-        "rmsnorm_fwd": 8 * C * St + 4 * C,
-        "rmsnorm_bwd": 12 * C * St + 12 * C,
-        "qknorm_rope_fwd": 8 * qkd * St,
-        "qknorm_rope_bwd": (12 if cfg["qk_norm"] else 8) * qkd * St,
-        "swiglu_fwd": 12 * H * St,
-        "swiglu_bwd": 20 * H * St,
-        "residual": 12 * C * St,
-        "scale_copy": 8 * H * St,        # y = alpha*a over an [H,St] tensor: a plain copy-shaped stream (train.m:523,595)
+        "rmsnorm_fwd": 2 * a * C * St + 4 * C,
+        "rmsnorm_bwd": 3 * a * C * St + 12 * C,
+        "qknorm_rope_fwd": 2 * a * qkd * St,
+        "qknorm_rope_bwd": (3 if cfg["qk_norm"] else 2) * a * qkd * St,
+        "swiglu_fwd": 3 * a * H * St,
+        "swiglu_bwd": 5 * a * H * St,
+        "residual": 3 * a * C * St,
+        "scale_copy": 2 * a * H * St,        # y = alpha*a over an [H,St] tensor: a plain copy-shaped stream (train.m:523,595)
         # residual + the RMSNorm after it in one launch; as two ops the same work is 12CSt + 8CSt + 4C
-        "residual_rmsnorm_fwd": 16 * C * St + 4 * C,
-        "softmax_ce": 8 * V * S,
+        "residual_rmsnorm_fwd": 4 * a * C * St + 4 * C,
+        "softmax_ce": 2 * a * V * S,
         "int8_scale": 4 * n8,
         "int8_quant": 5 * n8,
         "int8_dequant": 5 * n8,
     }
 
 
+class Bf16Lib:
+    """Routes the ops that have a bfloat16-storage variant to it (mi355_X_dev -> mi355_X_bf16_dev)."""
+    HAVE = {"mi355_rmsnorm_fwd_dev", "mi355_rmsnorm_bwd_dev", "mi355_swiglu_fwd_dev", "mi355_swiglu_bwd_dev",
+            "mi355_axpby_dev", "mi355_rope_dev", "mi355_qknorm_rope_fwd_dev", "mi355_qknorm_rope_bwd_dev",
+            "mi355_softmax_ce_dev"}
+
+    # fp32 entry points that the sweep may still call in bf16 mode: they never see an activation buffer
+    FP32_OK = {"mi355_dw_flush", "mi355_int8_scale_dev", "mi355_int8_quant_dev", "mi355_int8_dequant_dev"}
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def __getattr__(self, name):
+        if name in self.HAVE:
+            return getattr(self._lib, name[:-4] + "_bf16_dev")
+        if name not in self.FP32_OK:
+            # an fp32 kernel on half-size bf16 buffers would run off their end
+            raise AttributeError("%s has no bf16-storage variant" % name)
+        return getattr(self._lib, name)
+
+
 class Workload:
-    def __init__(self, br, cfg, layers, fuse=False):
-        self.br, self.cfg, self.L, self.fuse = br, cfg, layers, fuse
+    def __init__(self, br, cfg, layers, fuse=False, bf16=False):
+        self.br, self.cfg, self.L, self.fuse, self.bf16 = br, cfg, layers, fuse, bf16
+        self.lib = Bf16Lib(br.lib) if bf16 else br.lib
         C, H, S, B = cfg["C"], cfg["H"], cfg["S"], cfg["batch"]
         qd, kd = cfg["heads"] * cfg["hd"], cfg["kv_heads"] * cfg["hd"]
-        A = br.DevArray
         seed = [1]
 
+        def A(shape, dtype=None):
+            """Activations (two or more dimensions) take the storage type; vectors (weights, dw) stay fp32."""
+            shape = shape if hasattr(shape, "__len__") else (shape,)
+            if dtype is None:
+                dtype = np.uint16 if bf16 and len(shape) >= 2 else np.float32
+            return br.DevArray(shape, dtype)
+
         def rnd(*shape, std=1.0, mean=0.0):
-            a = A(shape)
+            a = br.DevArray(shape)
             br.check(br.lib.mi355_fill_normal_dev(a.ptr, a.size, seed[0], mean, std))
             seed[0] += 1
+            if bf16 and len(shape) >= 2:
+                b = br.DevArray(shape, np.uint16)
+                br.check(br.lib.mi355_cvt_f32_bf16_dev(b.ptr, a.size, a.ptr, a.size, 1, a.size))
+                br.sync()
+                a.free()
+                return b
             return a
 
         self.lay = []
@@ -103,7 +138,7 @@ class Workload:
         br.check(br.lib.mi355_fill_randint_dev(self.targets.ptr, S, 999, 0, V))
         self.loss = A(1)
         n8 = cfg["int8_shape"][0] * cfg["int8_shape"][1]
-        self.x8 = rnd(n8)
+        self.x8 = rnd(n8)                      # the INT8 ops take fp32 in both modes
         self.q8 = A(n8, np.int8)
         self.y8 = A(n8)
         self.scale8 = A(1)
@@ -113,9 +148,17 @@ class Workload:
         self.alpha = float(np.float32((2.0 * 12) ** 0.25 if not cfg["qk_norm"] else 1.0 / np.sqrt(2.0 * cfg["layers"])))
         br.sync()
 
+    def host(self, a):
+        """Device array -> fp32 numpy (bf16 storage is widened; exact)."""
+        h = a.numpy()
+        if h.dtype == np.uint16:
+            import oracle as O
+            return O.cvt_bf16_f32(h)
+        return h
+
     # ---- single ops on layer buffers d -------------------------------------------------------
     def op(self, name, d):
-        lib, c, ck = self.br.lib, self.cfg, self.br.check
+        lib, c, ck = self.lib, self.cfg, self.br.check
         C, H, S, B, hd = c["C"], c["H"], c["S"], c["batch"], c["hd"]
         n_c, n_h = B * C * S, B * H * S
         if name == "rmsnorm_fwd":
@@ -173,7 +216,7 @@ class Workload:
     BWD = ["swiglu_bwd", "rmsnorm_bwd2", "qknorm_rope_bwd", "rmsnorm_bwd"]
 
     def ce(self):
-        self.br.check(self.br.lib.mi355_softmax_ce_dev(self.dlogits.ptr, self.loss.ptr, self.logits.ptr,
+        self.br.check(self.lib.mi355_softmax_ce_dev(self.dlogits.ptr, self.loss.ptr, self.logits.ptr,
                                                        self.targets.ptr, self.cfg["V"], self.cfg["S"], 1.0))
 
     def int8(self, which=("scale", "quant", "dequant")):
@@ -213,11 +256,13 @@ def time_region(br, fn, reps=1):
 def per_op_table(br, wl, reps):
     """Average launch time of each op over all layer buffers (cold operands), HIP events on the
     bridge stream."""
-    ab = alg_bytes(wl.cfg)
+    ab = alg_bytes(wl.cfg, 2 if wl.bf16 else 4)
     names = {"rmsnorm_fwd": "rmsnorm_fwd", "rmsnorm_bwd": "rmsnorm_bwd", "qknorm_rope_fwd": "qknorm_rope_fwd",
              "qknorm_rope_bwd": "qknorm_rope_bwd", "swiglu_fwd": "swiglu_fwd", "swiglu_bwd": "swiglu_bwd",
              "residual1": "residual", "res_rms1": "residual_rmsnorm_fwd", "scale_copy": "scale_copy"}
     table = []
+    if wl.bf16:
+        del names["res_rms1"]          # the fused residual + RMSNorm exists for fp32 storage only
     for opname, key in names.items():
         def run():
             for d in wl.lay:
@@ -244,7 +289,7 @@ def cpu_baseline(br, wl, sample_layers, threads_mt):
     now = time.perf_counter
 
     def layer_time(d, threads):
-        h = {k: v.numpy() for k, v in d.items() if k in ("x", "w_att", "q", "k", "wq", "wk", "o", "w_ffn", "h1", "h3",
+        h = {k: wl.host(v) for k, v in d.items() if k in ("x", "w_att", "q", "k", "wq", "wk", "o", "w_ffn", "h1", "h3",
                                                          "f", "dsilu", "dx_ffn", "dy", "gq", "gk", "dx_attn")}
         out = {}
         t0 = now()
@@ -256,13 +301,15 @@ def cpu_baseline(br, wl, sample_layers, threads_mt):
             out["q_rot"] = O.rope(h["q"], hd, c["theta"], +1, threads=threads)
             out["k_rot"] = O.rope(h["k"], hd, c["theta"], +1, threads=threads)
         out["x2"] = O.axpby(h["x"], h["o"], wl.alpha, 0, threads=threads)
-        out["x2n"] = O.rmsnorm(out["x2"], h["w_ffn"], threads=threads)
+        # with bf16 storage the device's x2 is a rounded copy: the ops that consume it are checked on that copy
+        x2 = wl.host(d["x2"]) if wl.bf16 else out["x2"]
+        out["x2n"] = O.rmsnorm(x2, h["w_ffn"], threads=threads)
         out["gate"] = O.swiglu_fwd(h["h1"], h["h3"], threads=threads)
-        out["x_next"] = O.axpby(out["x2"], h["f"], wl.alpha, 0, threads=threads)
+        out["x_next"] = O.axpby(x2, h["f"], wl.alpha, 0, threads=threads)
         if wl.fuse:
             out["xn_next"] = O.rmsnorm(out["x_next"], h["w_att"], threads=threads)
         out["dh1"], out["dh3"] = O.swiglu_bwd(h["dsilu"], h["h1"], h["h3"], threads=threads)
-        out["dx2"], out["dw_ffn"] = O.rmsnorm_bwd(h["dx_ffn"], out["x2"], h["w_ffn"], threads=threads)
+        out["dx2"], out["dw_ffn"] = O.rmsnorm_bwd(h["dx_ffn"], x2, h["w_ffn"], threads=threads)
         if c["qk_norm"]:
             out["dq"], out["dwq"] = O.qknorm_rope_bwd(h["gq"], h["q"], h["wq"], hd, c["theta"], threads=threads)
             out["dk"], out["dwk"] = O.qknorm_rope_bwd(h["gk"], h["k"], h["wk"], hd, c["theta"], threads=threads)
@@ -285,10 +332,10 @@ def cpu_baseline(br, wl, sample_layers, threads_mt):
         if i == 0:
             # dw buffers accumulate over steps on the GPU; compare the assigned tensors only
             for k in ("xn", "q_rot", "k_rot", "x2", "x2n", "gate", "x_next", "dh1", "dh3", "dx2", "dq", "dk", "dx1"):
-                parity = max(parity, rel(wl.lay[0][k].numpy(), out[k]))
-    logits = wl.logits.numpy(); tg = wl.targets.numpy()
+                parity = max(parity, rel(wl.host(wl.lay[0][k]), out[k]))
+    logits = wl.host(wl.logits); tg = wl.targets.numpy()
     t0 = now(); loss, dl = O.cross_entropy(logits, tg); t_ce = now() - t0
-    parity = max(parity, rel(wl.dlogits.numpy(), dl), abs(float(wl.loss.numpy()[0]) - loss) / abs(loss))
+    parity = max(parity, rel(wl.host(wl.dlogits), dl), abs(float(wl.loss.numpy()[0]) - loss) / abs(loss))
     del dl, logits
     x8 = wl.x8.numpy()
     t0 = now(); sc = O.int8_scale(x8); q = O.int8_quant(x8, sc, 0); y = O.int8_dequant(q, sc); t_i8 = now() - t0
@@ -565,6 +612,9 @@ def main():
     ap.add_argument("--fuse", action="store_true",
                     help="run each residual and the RMSNorm after it as one launch (mi355_residual_rmsnorm_fwd_dev)")
     ap.add_argument("--op-reps", type=int, default=3)
+    ap.add_argument("--storage", default="f32", choices=["f32", "bf16"],
+                    help="activation storage: f32 (the reference's, default) or the optional bf16 variants "
+                         "(arithmetic stays f32; parity bound 5e-3 instead of 1e-5)")
     ap.add_argument("--graph", action="store_true",
                     help="record one step as a graph and time its replays (pays off where the step is launch-bound)")
     ap.add_argument("--workload", default="qwen3", choices=["qwen3", "stories110m", "embed", "optimizer", "aux", "host"],
@@ -592,7 +642,10 @@ def main():
         cfg["batch"] = args.batch
     if args.layers <= 0:
         args.layers = cfg["layers"]
-    wl = Workload(br, cfg, args.layers, fuse=args.fuse)
+    bf16 = args.storage == "bf16"
+    if bf16 and args.fuse:
+        raise SystemExit("bench.py: the fused residual + RMSNorm has no bf16-storage variant; drop --fuse")
+    wl = Workload(br, cfg, args.layers, fuse=args.fuse, bf16=bf16)
     br.check(br.lib.mi355_dw_defer(0 if args.immediate_dw else 1))
 
     for _ in range(args.warmup):
@@ -614,7 +667,7 @@ def main():
     br.sync()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    ab = alg_bytes(cfg)
+    ab = alg_bytes(cfg, 2 if bf16 else 4)
     # algorithmic bytes of the work done, op by op as the unfused definitions count it
     per_layer = (2 * ab["rmsnorm_fwd"] + 2 * ab["rmsnorm_bwd"] + ab["qknorm_rope_fwd"] + ab["qknorm_rope_bwd"] +
                  ab["swiglu_fwd"] + ab["swiglu_bwd"] + 2 * ab["residual"])
@@ -628,7 +681,7 @@ def main():
                                                                ("softmax_ce", "int8_scale", "int8_quant", "int8_dequant") else 1))
     roofline = dict(bound="hbm", kernel=dom["op"], achieved=dom["gbs"], peak=PEAK_HBM_GBS, unit="GB/s",
                     frac=dom["gbs"] / PEAK_HBM_GBS,
-                    traffic=MEASURED_TRAFFIC_BYTES.get(dom["op"]) if (cfg["name"], cfg["batch"]) == ("qwen3-0.6b", 16) else None,
+                    traffic=MEASURED_TRAFFIC_BYTES.get(dom["op"]) if (cfg["name"], cfg["batch"], bf16) == ("qwen3-0.6b", 16, False) else None,
                     traffic_source="profiles/qwen3_sweep_pmc_fetch_write.md", alg_bytes_per_launch=ab[dom["op"]],
                     avg_launch_ms=dom["ms"])
 
@@ -646,6 +699,7 @@ def main():
                                    "QK-norm + RoPE" if cfg["qk_norm"] else "RoPE", cfg["V"], cfg["S"]),
                    "layers": args.layers, "tokens_per_step": tokens, "alg_gb_per_step": total_bytes / 1e9,
                    "residual_fused_into_next_rmsnorm": wl.fuse, "replayed_as_graph": bool(args.graph),
+                   "activation_storage": args.storage,
                    "weight_gradients": "reduced per op" if args.immediate_dw else "queued, reduced once per step"},
         "aggregate_gbs": total_bytes / ms / 1e6, "aggregate_frac_of_peak": total_bytes / ms / 1e6 / PEAK_HBM_GBS,
         "host_wall_ms_per_step": wall_ms,
