@@ -115,7 +115,7 @@ __global__ __launch_bounds__(CE_THREADS) void ce_partial_kernel(float *__restric
 #pragma unroll
         for (int k = 0; k < CE_CAP; k++) {
             const int v = base + k * CE_WAVES + wave;
-            if (v < v_hi && col_ok) ld_cols<VEC>(x[k], logits + (size_t)v * S + col);
+            if (v < v_hi && col_ok) ld_cols<VEC>(x[k], logits + (size_t)v * S + col);   // cached: pass 2 re-reads these rows (non-temporal here costs 30 %)
             else {
 #pragma unroll
                 for (int j = 0; j < VEC; j++) x[k][j] = -INFINITY;
@@ -157,8 +157,10 @@ __global__ __launch_bounds__(CE_THREADS) void ce_partial_kernel(float *__restric
     }
 }
 
-// One workgroup per 64 columns: 16 groups of threads each merge an interleaved subset of the row
-// blocks, then the 16 partial results are merged in order.
+// One workgroup per 16 columns: 64 groups of threads each merge an interleaved subset of the row blocks (few
+// rounds of loads per thread, S/16 workgroups in flight), then the 64 partial results are merged by a fixed
+// tree.  The merge of two (max, sum) pairs is the online-softmax rescaling.
+constexpr int CB_COLS = 16, CB_GROUPS = 1024 / CB_COLS;
 template <typename T>
 __global__ __launch_bounds__(1024) void ce_combine_kernel(float *__restrict__ colM, float *__restrict__ colInv,
                                                           float *__restrict__ colLoss, const float *__restrict__ pm,
@@ -166,21 +168,21 @@ __global__ __launch_bounds__(1024) void ce_combine_kernel(float *__restrict__ co
                                                           const T *__restrict__ logits,
                                                           const int32_t *__restrict__ targets, int V, int S,
                                                           int nblk) {
-    __shared__ float sm[16][64], sl[16][64];
-    const int cl = threadIdx.x & 63, g = threadIdx.x >> 6;
-    const int t = blockIdx.x * 64 + cl;
+    __shared__ float sm[CB_GROUPS][CB_COLS], sl[CB_GROUPS][CB_COLS];
+    const int cl = threadIdx.x % CB_COLS, g = threadIdx.x / CB_COLS;
+    const int t = blockIdx.x * CB_COLS + cl;
     float m = -INFINITY, l = 0.f;
     if (t < S)
-        for (int r0 = g; r0 < nblk; r0 += 16 * 8) {
-            float mr[8], lr[8];
+        for (int r0 = g; r0 < nblk; r0 += CB_GROUPS * 4) {
+            float mr[4], lr[4];
 #pragma unroll
-            for (int u = 0; u < 8; u++) {     // eight independent loads in flight
-                const int r = r0 + 16 * u;
+            for (int u = 0; u < 4; u++) {     // four independent loads in flight
+                const int r = r0 + CB_GROUPS * u;
                 mr[u] = r < nblk ? pm[(size_t)r * S + t] : -INFINITY;
                 lr[u] = r < nblk ? pl[(size_t)r * S + t] : 0.f;
             }
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
+            for (int u = 0; u < 4; u++) {
                 const float nm = fmaxf(m, mr[u]);
                 if (nm > -INFINITY) {
                     l = l * exp_neg(m - nm) + lr[u] * exp_neg(mr[u] - nm);
@@ -191,15 +193,20 @@ __global__ __launch_bounds__(1024) void ce_combine_kernel(float *__restrict__ co
     sm[g][cl] = m;
     sl[g][cl] = l;
     __syncthreads();
+    for (int half = CB_GROUPS / 2; half > 0; half >>= 1) {
+        if (g < half) {
+            const float m0 = sm[g][cl], m1 = sm[g + half][cl];
+            const float nm = fmaxf(m0, m1);
+            if (nm > -INFINITY) {
+                sl[g][cl] = sl[g][cl] * exp_neg(m0 - nm) + sl[g + half][cl] * exp_neg(m1 - nm);
+                sm[g][cl] = nm;
+            }
+        }
+        __syncthreads();
+    }
     if (g == 0 && t < S) {
-        float M = sm[0][cl];
-#pragma unroll
-        for (int k = 1; k < 16; k++) M = fmaxf(M, sm[k][cl]);
-        float L = 0.f;
-#pragma unroll
-        for (int k = 0; k < 16; k++)
-            if (sm[k][cl] > -INFINITY) L += sl[k][cl] * exp_neg(sm[k][cl] - M);
-        const float inv = 1.0f / L;
+        const float M = sm[0][cl];
+        const float inv = 1.0f / sl[0][cl];
         colM[t] = M;
         colInv[t] = inv;
         const int tgt = targets[t];
@@ -307,7 +314,7 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
     if (vec_ok) hipLaunchKernelGGL((ce_partial_kernel<4, T>), grid, dim3(CE_THREADS), 0, g_ctx.stream, pm, pl, logits, V, S, rpb);
     else hipLaunchKernelGGL((ce_partial_kernel<1, T>), grid, dim3(CE_THREADS), 0, g_ctx.stream, pm, pl, logits, V, S, rpb);
     LAUNCH_OK("softmax_ce partial");
-    hipLaunchKernelGGL(ce_combine_kernel<T>, dim3((unsigned)ceil_div((size_t)S, 64)), dim3(1024), 0, g_ctx.stream, colM,
+    hipLaunchKernelGGL(ce_combine_kernel<T>, dim3((unsigned)ceil_div((size_t)S, CB_COLS)), dim3(1024), 0, g_ctx.stream, colM,
                        colInv, colLoss, pm, pl, logits, targets, V, S, nblk);
     LAUNCH_OK("softmax_ce combine");
     if (vec_ok)
