@@ -89,7 +89,7 @@ class Bf16Lib:
 
 
 class Workload:
-    def __init__(self, br, cfg, layers, fuse=False, bf16=False):
+    def __init__(self, br, cfg, layers, fuse=False, bf16=False, share=False):
         self.br, self.cfg, self.L, self.fuse, self.bf16 = br, cfg, layers, fuse, bf16
         self.lib = Bf16Lib(br.lib) if bf16 else br.lib
         C, H, S, B = cfg["C"], cfg["H"], cfg["S"], cfg["batch"]
@@ -116,7 +116,7 @@ class Workload:
             return a
 
         self.lay = []
-        for _ in range(layers):
+        for _ in range(1 if share else layers):
             d = dict(
                 x=rnd(B, C, S), w_att=rnd(C, std=0.02, mean=1.0), xn=A((B, C, S)),
                 q=rnd(B, qd, S), k=rnd(B, kd, S), wq=rnd(cfg["hd"], std=0.02, mean=1.0),
@@ -131,6 +131,8 @@ class Workload:
                 dwk=A(cfg["hd"]), dx_attn=rnd(B, C, S), dx1=A((B, C, S)), dw_att=A(C), dy_out=A((B, C, S)),
             )
             self.lay.append(d)
+        if share:       # every layer runs on the same buffers: operands are as warm as the last-level cache keeps them
+            self.lay = self.lay * layers
         V = cfg["V"]
         self.logits = rnd(V, S, std=2.0)
         self.dlogits = A((V, S))
@@ -615,6 +617,8 @@ def main():
     ap.add_argument("--storage", default="f32", choices=["f32", "bf16"],
                     help="activation storage: f32 (the reference's, default) or the optional bf16 variants "
                          "(arithmetic stays f32; parity bound 5e-3 instead of 1e-5)")
+    ap.add_argument("--share-buffers", action="store_true",
+                    help="run every layer on one set of buffers (warm operands) instead of one set per layer (cold, default)")
     ap.add_argument("--graph", action="store_true",
                     help="record one step as a graph and time its replays (pays off where the step is launch-bound)")
     ap.add_argument("--workload", default="qwen3", choices=["qwen3", "stories110m", "embed", "optimizer", "aux", "host"],
@@ -645,7 +649,7 @@ def main():
     bf16 = args.storage == "bf16"
     if bf16 and args.fuse:
         raise SystemExit("bench.py: the fused residual + RMSNorm has no bf16-storage variant; drop --fuse")
-    wl = Workload(br, cfg, args.layers, fuse=args.fuse, bf16=bf16)
+    wl = Workload(br, cfg, args.layers, fuse=args.fuse, bf16=bf16, share=args.share_buffers)
     br.check(br.lib.mi355_dw_defer(0 if args.immediate_dw else 1))
 
     for _ in range(args.warmup):
@@ -700,6 +704,7 @@ def main():
                    "layers": args.layers, "tokens_per_step": tokens, "alg_gb_per_step": total_bytes / 1e9,
                    "residual_fused_into_next_rmsnorm": wl.fuse, "replayed_as_graph": bool(args.graph),
                    "activation_storage": args.storage,
+                   "operands": "warm: one buffer set shared by all layers" if args.share_buffers else "cold: one buffer set per layer",
                    "weight_gradients": "reduced per op" if args.immediate_dw else "queued, reduced once per step"},
         "aggregate_gbs": total_bytes / ms / 1e6, "aggregate_frac_of_peak": total_bytes / ms / 1e6 / PEAK_HBM_GBS,
         "host_wall_ms_per_step": wall_ms,
