@@ -685,6 +685,8 @@ ORC_API void orc_embed_backward_batched(float *d_embed, const float *dx, const i
  *   recipe 0: training/test_rmsnorm_bwd.m:26-33   x=(2u-1)*0.5, dy=(2u-1)*0.1 interleaved; w=0.5u+0.75
  *   recipe 1: training/test_classifier.m:25-27    x=2u-1; w=0.5u+0.75   (dy untouched)
  *   recipe 2: training/test_classifier.m:132-134  x=10u-5               (w, dy untouched)
+ *   recipe 3: training/test_classifier.m:60-62    x=(2u-1)*0.1 (n values), then w=(2u-1)*0.02 (d values)
+ *   recipe 4: training/test_classifier.m:205-207  x=(2u-1)*0.01 (n values), then w=(2u-1)*0.02 (d values)
  * ------------------------------------------------------------------------------------------- */
 ORC_API void orc_recipe_drand48(int recipe, long seed, float *x, float *dy, float *w, size_t n,
                                 int d) {
@@ -698,8 +700,12 @@ ORC_API void orc_recipe_drand48(int recipe, long seed, float *x, float *dy, floa
     } else if (recipe == 1) {
         for (size_t i = 0; i < n; i++) x[i] = (float)(drand48() * 2 - 1);
         for (int i = 0; i < d; i++) w[i] = (float)(drand48() * 0.5 + 0.75);
-    } else {
+    } else if (recipe == 2) {
         for (size_t i = 0; i < n; i++) x[i] = (float)(drand48() * 10 - 5);
+    } else {
+        const float sx = recipe == 3 ? 0.1f : 0.01f;
+        for (size_t i = 0; i < n; i++) x[i] = (float)(drand48() * 2 - 1) * sx;
+        for (int i = 0; i < d; i++) w[i] = (float)(drand48() * 2 - 1) * 0.02f;
     }
 }
 

@@ -757,6 +757,25 @@ def test_classifier_head_chain_stays_on_device(br):
     assert H.rel_err(dx.numpy(), o_dx) <= 1e-4 and abs(float(lossd.numpy()[0]) - o_loss) <= 1e-5 * abs(o_loss)
 
 
+def test_sgemm_reference_test_recipes(br):
+    """The inputs of the reference's own classifier tests at their own size (VOCAB 32000, DIM 768, SEQ 256):
+    forward training/test_classifier.m:60-69 (srand48(123)), backward :205-214 (srand48(456)).  The reference
+    compares against an fp16 accelerator at 0.05-1.0 absolute; here the product is checked at 1e-5."""
+    V, D, S = 32000, 768, 256
+    x, _, emb = O.recipe_drand48(3, 123, D * S, V * D)
+    x = x.reshape(D, S); emb = emb.reshape(V, D)
+    xd, ed = dev(br, x), dev(br, emb)
+    logits = br.DevArray((V, S))
+    br.check(br.lib.mi355_sgemm_dev(111, 111, V, S, D, 1.0, ed.ptr, D, xd.ptr, S, 0.0, logits.ptr, S))
+    assert H.rel_err(logits.numpy(), O.sgemm(0, 0, 1.0, emb, x)) <= TOL
+    dlog, _, emb2 = O.recipe_drand48(4, 456, V * S, V * D)
+    dlog = dlog.reshape(V, S); emb2 = emb2.reshape(V, D)
+    dd, e2d = dev(br, dlog), dev(br, emb2)
+    dx = br.DevArray((D, S))
+    br.check(br.lib.mi355_sgemm_dev(112, 111, D, S, V, 1.0, e2d.ptr, D, dd.ptr, S, 0.0, dx.ptr, S))
+    assert H.rel_err(dx.numpy(), O.sgemm(1, 0, 1.0, emb2, dlog)) <= TOL
+
+
 @pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (0, 1), (1, 1)])
 def test_sgemm_pitched_operands(br, ta, tb):
     M, N, K, pad = 45, 70, 33, 5

@@ -32,6 +32,12 @@ def test_drand48_recipes_match_the_posix_lcg():
     x2, _, _ = O.recipe_drand48(2, 999, 16, 0)
     g = H.Drand48(999)
     assert np.array_equal(x2, np.array([np.float32(g.next() * 10 - 5) for _ in range(16)], np.float32))
+    # training/test_classifier.m:60-62 and :205-207 — one array, then the next, from the same stream
+    for recipe, seed, sx in ((3, 123, 0.1), (4, 456, 0.01)):
+        x3, _, w3 = O.recipe_drand48(recipe, seed, 10, 7)
+        g = H.Drand48(seed)
+        assert np.array_equal(x3, np.array([np.float32(g.next() * 2 - 1) * np.float32(sx) for _ in range(10)], np.float32))
+        assert np.array_equal(w3, np.array([np.float32(g.next() * 2 - 1) * np.float32(0.02) for _ in range(7)], np.float32))
 
 
 # ---------------------------------------------------------------------------------------------
