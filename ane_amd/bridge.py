@@ -110,6 +110,7 @@ SIGNATURES = {
     "mi355_rope_bf16_dev": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _i]),
     "mi355_qknorm_rope_fwd_bf16_dev": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _f]),
     "mi355_qknorm_rope_bwd_bf16_dev": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _f, _i]),
+    "mi355_workspace_size": (_z, []),
     "mi355_graph_begin": (_i, []),
     "mi355_graph_end": (_p, []),
     "mi355_graph_launch": (_i, [_p]),

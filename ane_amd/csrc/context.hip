@@ -133,13 +133,14 @@ MI355_API int mi355_workspace_reserve(size_t bytes) {
     return mi355_ws(bytes) ? 0 : -1;
 }
 
+MI355_API size_t mi355_workspace_size(void) { return g_ctx.ready ? g_ctx.ws_bytes : 0; }
+
 MI355_API int mi355_tune_set(const char *key, int value) {
     if (!key) return -1;
     struct { const char *k; int *v; } tab[] = {
         {"rms_lpr", &g_ctx.rms_lpr}, {"rms_threads", &g_ctx.rms_threads},
-        {"ew_unroll", &g_ctx.ew_unroll}, {"ew_threads", &g_ctx.ew_threads},
+        {"ew_unroll", &g_ctx.ew_unroll},
         {"ce_rows", &g_ctx.ce_rows}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
-        {"gather_tile", &g_ctx.gather_tile}, {"nt_store", &g_ctx.nt_store},
         {"gemm_splitk", &g_ctx.gemm_splitk},
     };
     for (auto &t : tab)

@@ -50,8 +50,12 @@ int mi355_sync(void);
 /* Grow the internal workspace (sort buffers, reduction partials) to at least `bytes` now, so
  * that later calls of up to that need allocate nothing. */
 int mi355_workspace_reserve(size_t bytes);
-/* Tuning knob for experiments: named integer settings ("rms_lpr", "ew_unroll", ...); unknown
- * names return -1.  Defaults are chosen per shape when a knob is 0. */
+/* Present size of that workspace: run a step once, read this, reserve as much at the next start. */
+size_t mi355_workspace_size(void);
+/* Tuning knobs for experiments; 0 = choose per shape (the default), unknown names return -1:
+ * "rms_lpr" (lanes per strip row, 4/8/16) and "rms_threads" (256/512/1024) of the RMSNorm tiles, "qk_lpr" and
+ * "qk_threads" (256/512) of the QK-norm + RoPE tiles, "ew_unroll" (accesses per lane of the streaming ops, 1/2/4),
+ * "ce_rows" (rows of logits per workgroup), "gemm_splitk" (K slices of mi355_sgemm_dev; 1 = never split). */
 int mi355_tune_set(const char *key, int value);
 
 /* ------------------------------------------------------------------------------------------

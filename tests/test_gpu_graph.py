@@ -93,7 +93,7 @@ def test_graph_replays_equal_eager_runs(br, defer):
             br.check(L.mi355_axpby_dev(eager["scratch"].ptr, eager["scratch"].ptr, None, 1.5, 4096, 1))
             br.sync()
         # a workspace reallocated after the recording invalidates it
-        br.check(L.mi355_workspace_reserve((3 + defer) << 30))       # larger than any earlier reservation
+        br.check(L.mi355_workspace_reserve(L.mi355_workspace_size() + (1 << 20)))
         assert L.mi355_graph_launch(g) == -1 and "record it again" in br.last_error()
         L.mi355_graph_free(g)
     finally:
