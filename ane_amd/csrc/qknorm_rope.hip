@@ -35,7 +35,7 @@ __global__ __launch_bounds__(THREADS) void qknorm_rope_fwd_kernel(
     const int half = hd >> 1;
     const size_t base = (size_t)slab * hd * S + col;
 
-    v4f x0[CAP], x1[CAP], cs[CAP], sn[CAP];
+    v4f x0[CAP], x1[CAP];
     float w0[CAP], w1[CAP];
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -45,12 +45,10 @@ __global__ __launch_bounds__(THREADS) void qknorm_rope_fwd_kernel(
             const float *px = in + base + (size_t)(2 * rp) * S;
             x0[kk] = ld4_nt(px);
             x1[kk] = ld4_nt(px + S);
-            cs[kk] = ld4(cos_t + (size_t)rp * S + col);
-            sn[kk] = ld4(sin_t + (size_t)rp * S + col);
             w0[kk] = w[2 * rp];
             w1[kk] = w[2 * rp + 1];
         } else {
-            x0[kk] = x1[kk] = cs[kk] = sn[kk] = zero;
+            x0[kk] = x1[kk] = zero;
             w0[kk] = w1[kk] = 0.f;
         }
     }
@@ -70,11 +68,14 @@ __global__ __launch_bounds__(THREADS) void qknorm_rope_fwd_kernel(
     for (int kk = 0; kk < CAP; kk++) {
         const int rp = p0 + kk * PPS;
         if (rp < half && col_ok) {
+            // the tables are shared by every head and sequence (cache-resident): read here, after the reduction,
+            // rather than held in registers across it
+            const v4f cs = ld4(cos_t + (size_t)rp * S + col), sn = ld4(sin_t + (size_t)rp * S + col);
             const v4f y0 = (x0[kk] * rr) * w0[kk];
             const v4f y1 = (x1[kk] * rr) * w1[kk];
             float *po = out + base + (size_t)(2 * rp) * S;
-            st4_nt(po, y0 * cs[kk] - y1 * sn[kk]);
-            st4_nt(po + S, y0 * sn[kk] + y1 * cs[kk]);
+            st4_nt(po, y0 * cs - y1 * sn);
+            st4_nt(po + S, y0 * sn + y1 * cs);
         }
     }
 }
