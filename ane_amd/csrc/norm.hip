@@ -248,7 +248,6 @@ __global__ __launch_bounds__(THREADS) void res_rms_fwd_kernel(float *y, float *_
 #pragma unroll
         for (int k = 0; k < CAP; k++) {
             const int c = row0 + k * RPS;
-            if (c < C && col_ok) stv_nt<VEC>(y + base + (size_t)c * S, yv[k]);
 #pragma unroll
             for (int j = 0; j < VEC; j++) acc[0][j] += yv[k][j] * yv[k][j];
         }
@@ -263,6 +262,7 @@ __global__ __launch_bounds__(THREADS) void res_rms_fwd_kernel(float *y, float *_
                 float o[VEC];
 #pragma unroll
                 for (int j = 0; j < VEC; j++) o[j] = (yv[k][j] * rr[j]) * wv[k];
+                stv_nt<VEC>(y + base + (size_t)c * S, yv[k]);
                 stv_nt<VEC>(yn + base + (size_t)c * S, o);
             }
         }
