@@ -106,15 +106,12 @@ __global__ __launch_bounds__(256) void gather_kernel(float *__restrict__ x, cons
 // ---------------------------------------------------------------------------------------------
 // Scatter-add
 // ---------------------------------------------------------------------------------------------
-__global__ void prep_keys_kernel(int *keys, int *vals, int *meta, const int32_t *ids, int N, int V) {
-    const int n = blockIdx.x * blockDim.x + threadIdx.x;
-    if (n == 0) { meta[0] = 0; meta[1] = 0; meta[2] = N; }
-    if (n < N) {
-        const int id = ids[n];
-        keys[n] = (id < 0 || id >= V) ? V : id;   // out-of-range ids sort last and are skipped
-        vals[n] = n;
-    }
-}
+// Sort key of a token id: the id itself, or V for an id outside [0,V) so that those sort last and are skipped.
+// The sort reads ids through this functor and takes 0,1,2,... as the values, so no staging pass is needed.
+struct ClampId {
+    int V;
+    __host__ __device__ int operator()(int32_t id) const { return (id < 0 || id >= V) ? V : id; }
+};
 
 // meta[0] = number of segments, meta[2] = number of valid (in-range) entries.
 //
@@ -158,7 +155,10 @@ __global__ __launch_bounds__(PLAN_T) void plan_flags_kernel(int *__restrict__ ra
         const int kp = i > 0 ? keys[i - 1] : -1;
         rank[vals[i]] = i;
         head = (k < V && k != kp) ? 1 : 0;
-        if (k >= V && kp < V) meta[2] = i;          // first out-of-range key: at most one thread writes
+        // number of valid entries: the index of the first out-of-range key, or N when the last key is valid
+        // (exactly one thread of the grid meets one of the two conditions)
+        if (k >= V && kp < V) meta[2] = i;
+        if (i == N - 1 && k < V) meta[2] = N;
     }
     int total;
     (void)block_excl_scan_1024(head, lds, total);
@@ -430,32 +430,29 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     const int bits = key_bits(V);
 
     size_t temp_bytes = 0;
-    hipError_t e = rocprim::radix_sort_pairs(nullptr, temp_bytes, (int *)nullptr, (int *)nullptr, (int *)nullptr,
-                                             (int *)nullptr, (size_t)N, 0, bits, g_ctx.stream);
+    hipError_t e = rocprim::radix_sort_pairs(nullptr, temp_bytes, rocprim::make_transform_iterator(ids, ClampId{V}),
+                                             (int *)nullptr, rocprim::counting_iterator<int>(0), (int *)nullptr,
+                                             (size_t)N, 0, bits, g_ctx.stream);
     if (e != hipSuccess) return mi355_fail("embed_scatter_add: sort sizing: %s", hipGetErrorString(e));
 
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
     const size_t nb = al((size_t)N * sizeof(int));
     const int nplan = (int)ceil_div((size_t)N, PLAN_T);
-    const size_t off_keys_in = 0, off_vals_in = nb, off_keys = 2 * nb, off_vals = 3 * nb, off_rank = 4 * nb;
-    const size_t off_seg = 5 * nb, off_cnt = off_seg + al((size_t)(N + 1) * sizeof(int));
+    const size_t off_keys = 0, off_vals = nb, off_rank = 2 * nb;
+    const size_t off_seg = 3 * nb, off_cnt = off_seg + al((size_t)(N + 1) * sizeof(int));
     const size_t off_boff = off_cnt + al((size_t)nplan * sizeof(int));
     const size_t off_meta = off_boff + al((size_t)nplan * sizeof(int)), off_temp = off_meta + 256;
     const size_t off_rows = off_temp + al(temp_bytes);
     const size_t total = off_rows + al((size_t)N * D * sizeof(float));
     char *ws = (char *)mi355_ws(total);
     if (!ws) return -1;
-    int *keys_in = (int *)(ws + off_keys_in), *vals_in = (int *)(ws + off_vals_in);
     int *keys = (int *)(ws + off_keys), *vals = (int *)(ws + off_vals), *rank = (int *)(ws + off_rank);
     int *seg_start = (int *)(ws + off_seg), *blk_count = (int *)(ws + off_cnt), *blk_off = (int *)(ws + off_boff);
     int *meta = (int *)(ws + off_meta);
     float *rows = (float *)(ws + off_rows);
 
-    hipLaunchKernelGGL(prep_keys_kernel, dim3((unsigned)ceil_div((size_t)N, 256)), dim3(256), 0, g_ctx.stream, keys_in,
-                       vals_in, meta, ids, N, V);
-    LAUNCH_OK("embed_scatter_add prep");
-    e = rocprim::radix_sort_pairs(ws + off_temp, temp_bytes, keys_in, keys, vals_in, vals, (size_t)N, 0, bits,
-                                  g_ctx.stream);
+    e = rocprim::radix_sort_pairs(ws + off_temp, temp_bytes, rocprim::make_transform_iterator(ids, ClampId{V}), keys,
+                                  rocprim::counting_iterator<int>(0), vals, (size_t)N, 0, bits, g_ctx.stream);
     if (e != hipSuccess) return mi355_fail("embed_scatter_add: sort: %s", hipGetErrorString(e));
     hipLaunchKernelGGL(plan_flags_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, rank, blk_count, meta, keys, vals,
                        N, V);

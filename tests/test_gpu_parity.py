@@ -354,6 +354,8 @@ def test_embed_gather_bit_exact(br, V, D, B, S, oob):
     (64, 768, 8, 256, 0),         # tiny vocabulary: every segment is long
     (70, 4, 1, 1, 0),
     (40, 130, 2, 100, 1),
+    (3000, 24, 160, 256, 3),      # 40960 positions: beyond the single-launch segment planner
+    (900, 16, 128, 256, 0),       # 32768 positions: its upper limit
 ])
 def test_embed_scatter_add_bit_exact_and_deterministic(br, V, D, B, S, oob):
     say("scatter_add V=%d D=%d B=%d S=%d" % (V, D, B, S))
