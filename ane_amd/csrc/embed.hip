@@ -293,17 +293,24 @@ __global__ __launch_bounds__(1024) void seg_sum_kernel(float *__restrict__ dE, c
                 const int tok = keys[lo];
                 float acc = 0.f;
                 if (wave == 0 && d_ok) acc = dE[(size_t)tok * D + d];
-                for (int base = lo; base < hi; base += STAGE_ROWS) {
+                // Software pipeline: the rows of stage s+1 are already on their way into registers while wave 0
+                // adds the rows of stage s out of LDS.
+                float v[STAGE_PER_WAVE];
+                auto fetch = [&](int base) {
                     const int nrow = min(STAGE_ROWS, hi - base);
-                    float v[STAGE_PER_WAVE];
 #pragma unroll
                     for (int j = 0; j < STAGE_PER_WAVE; j++) {
                         const int rl = wave * STAGE_PER_WAVE + j;
                         v[j] = (rl < nrow && d_ok) ? __builtin_nontemporal_load(rows + (size_t)(base + rl) * D + d) : 0.f;
                     }
+                };
+                fetch(lo);
+                for (int base = lo; base < hi; base += STAGE_ROWS) {
+                    const int nrow = min(STAGE_ROWS, hi - base);
 #pragma unroll
                     for (int j = 0; j < STAGE_PER_WAVE; j++) stage[wave * STAGE_PER_WAVE + j][lane] = v[j];
                     __syncthreads();
+                    if (base + STAGE_ROWS < hi) fetch(base + STAGE_ROWS);
                     if (wave == 0) {
                         int rl = 0;
                         for (; rl + 16 <= nrow; rl += 16) {
