@@ -141,7 +141,7 @@ MI355_API int mi355_tune_set(const char *key, int value) {
         {"rms_lpr", &g_ctx.rms_lpr}, {"rms_threads", &g_ctx.rms_threads},
         {"ew_unroll", &g_ctx.ew_unroll},
         {"ce_rows", &g_ctx.ce_rows}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
-        {"gemm_splitk", &g_ctx.gemm_splitk},
+        {"gemm_splitk", &g_ctx.gemm_splitk}, {"scatter_tree", &g_ctx.scatter_tree},
     };
     for (auto &t : tab)
         if (strcmp(t.k, key) == 0) { *t.v = value; return 0; }

@@ -262,6 +262,7 @@ __global__ __launch_bounds__(256) void transpose_sorted_kernel(float *__restrict
 //    from memory, eight loads in flight.
 // Either way every (row of dE, d) is written by exactly one lane, sequentially in position order,
 // starting from the value already in dE.
+template <bool TREE>
 __global__ __launch_bounds__(1024) void seg_sum_kernel(float *__restrict__ dE, const float *__restrict__ rows,
                                                        const int *__restrict__ seg_start, const int *__restrict__ keys,
                                                        const int *__restrict__ meta, int D, int nchunk,
@@ -307,6 +308,23 @@ __global__ __launch_bounds__(1024) void seg_sum_kernel(float *__restrict__ dE, c
                 fetch(lo);
                 for (int base = lo; base < hi; base += STAGE_ROWS) {
                     const int nrow = min(STAGE_ROWS, hi - base);
+                    if constexpr (TREE) {
+                        // fixed tree instead of the reference's chain (opt-in, "scatter_tree" knob): every wave sums
+                        // its 15 rows in order, wave 0 adds the 16 partial rows in wave order.  Deterministic, 8x
+                        // shorter chain, but rounded differently from the CPU loop.  Rows past the end are zeros.
+                        float p = v[0];
+#pragma unroll
+                        for (int j = 1; j < STAGE_PER_WAVE; j++) p += v[j];
+                        stage[wave][lane] = p;
+                        __syncthreads();
+                        if (base + STAGE_ROWS < hi) fetch(base + STAGE_ROWS);
+                        if (wave == 0) {
+#pragma unroll
+                            for (int q = 0; q < 16; q++) acc += stage[q][lane];
+                        }
+                        __syncthreads();
+                        continue;
+                    }
 #pragma unroll
                     for (int j = 0; j < STAGE_PER_WAVE; j++) stage[wave * STAGE_PER_WAVE + j][lane] = v[j];
                     __syncthreads();
@@ -478,8 +496,12 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     int long_x = (int)std::min<size_t>((size_t)N / LONG_SEG + 1, (size_t)std::max(1, cu / nchunk));
     size_t short_blocks = ceil_div((size_t)N * nchunk, 16);
     if (short_blocks > (size_t)cu * 4) short_blocks = (size_t)cu * 4;
-    hipLaunchKernelGGL(seg_sum_kernel, dim3((unsigned)(long_x * nchunk + short_blocks)), dim3(1024), 0, g_ctx.stream, dE,
-                       rows, seg_start, keys, meta, D, nchunk, long_x, (int)short_blocks);
+    if (g_ctx.scatter_tree)
+        hipLaunchKernelGGL(seg_sum_kernel<true>, dim3((unsigned)(long_x * nchunk + short_blocks)), dim3(1024), 0,
+                           g_ctx.stream, dE, rows, seg_start, keys, meta, D, nchunk, long_x, (int)short_blocks);
+    else
+        hipLaunchKernelGGL(seg_sum_kernel<false>, dim3((unsigned)(long_x * nchunk + short_blocks)), dim3(1024), 0,
+                           g_ctx.stream, dE, rows, seg_start, keys, meta, D, nchunk, long_x, (int)short_blocks);
     LAUNCH_OK("embed_scatter_add segment sums");
     return 0;
 }

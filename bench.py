@@ -392,6 +392,10 @@ def bench_embed(br, args):
         gather(); scatter()
     t_g = time_region(br, gather, args.steps) / nbuf
     t_s = time_region(br, scatter, args.steps) / nbuf
+    br.tune("scatter_tree", 1)          # the opt-in fixed-tree order for long segments (deterministic, not bit-identical)
+    scatter()
+    t_s_tree = time_region(br, scatter, args.steps) / nbuf
+    br.tune("scatter_tree", 0)
     b_g = 8 * D * N + 4 * N
     b_s = 4 * D * N + 8 * D * U + 4 * N
     out = {"metric": "embedding gather + ordered scatter-add (BASELINE config 2)", "value": N / ((t_g + t_s) / 1e3),
@@ -401,7 +405,9 @@ def bench_embed(br, args):
                       "hottest_id_count": int(np.bincount(ids.ravel()).max())},
            "ops": [dict(op="embed_gather", ms=t_g, alg_mb=b_g / 1e6, gbs=b_g / t_g / 1e6, frac=b_g / t_g / 1e6 / PEAK_HBM_GBS),
                    dict(op="embed_scatter_add", ms=t_s, alg_mb=b_s / 1e6, gbs=b_s / t_s / 1e6,
-                        frac=b_s / t_s / 1e6 / PEAK_HBM_GBS)]}
+                        frac=b_s / t_s / 1e6 / PEAK_HBM_GBS),
+                   dict(op="embed_scatter_add (scatter_tree=1)", ms=t_s_tree, alg_mb=b_s / 1e6, gbs=b_s / t_s_tree / 1e6,
+                        frac=b_s / t_s_tree / 1e6 / PEAK_HBM_GBS)]}
     if args.cpu_layers > 0:
         import oracle as O
         Eh = E.numpy(); g0 = gs[0].numpy()

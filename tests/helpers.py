@@ -224,3 +224,15 @@ def ckpt_weight_offsets_like_dashboard(cfg):
     out[(0, 9)] = off; off += 4 * cfg["dim"] + 4 * 2 * cfg["dim"]
     out[(0, 10)] = off
     return out
+
+
+def np_embed_backward(dE0, dx, ids):
+    """dE0 + per-token sums of dx columns in float64 (the exact value both summation orders approximate)."""
+    B, D, S = dx.shape
+    V = dE0.shape[0]
+    out = dE0.astype(np.float64).copy()
+    flat = ids.reshape(-1)
+    cols = dx.transpose(0, 2, 1).reshape(B * S, D).astype(np.float64)
+    ok = (flat >= 0) & (flat < V)
+    np.add.at(out, flat[ok], cols[ok])
+    return out
