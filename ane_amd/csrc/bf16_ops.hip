@@ -660,9 +660,11 @@ struct BfCfg {
 
 // 8-column lanes when the rows allow 128-bit accesses; rows in (packed) registers when one workgroup can hold
 // them, else two sweeps.  The rms_lpr / rms_threads knobs override the strip width and workgroup size.
-BfCfg pick_bf(int C, bool vec_ok) {
+BfCfg pick_bf(int C, bool vec_ok, int S, int batch) {
     if (!vec_ok) return BfCfg{1, 64, 256, 0};
-    int lpr = g_ctx.rms_lpr == 8 ? 8 : 4;
+    // 128-byte strips (8 lanes x 8 columns) once they still give every compute unit a workgroup
+    const long strips8 = (long)ceil_div((size_t)S, 64) * batch;
+    int lpr = g_ctx.rms_lpr == 8 || (!g_ctx.rms_lpr && strips8 >= (g_ctx.num_cu > 0 ? g_ctx.num_cu : 256)) ? 8 : 4;
     int threads = g_ctx.rms_threads == 256 || g_ctx.rms_threads == 512 || g_ctx.rms_threads == 1024
                       ? g_ctx.rms_threads
                       : (C >= 512 ? 1024 : 256);   // measured at C = 1024, 16 x 256 columns: 11.0 / 20.5 us forward / backward with
@@ -780,7 +782,7 @@ MI355_API int mi355_rmsnorm_fwd_bf16_dev(uint16_t *y, const uint16_t *x, const f
     if (!mi355_ready("rmsnorm_fwd_bf16")) return -1;
     if (!y || !x || !w) return mi355_fail("rmsnorm_fwd_bf16: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_fwd_bf16: bad shape C=%d S=%d batch=%d", C, S, batch);
-    const BfCfg cfg = pick_bf(C, S % 8 == 0 && aligned16(x) && aligned16(y));
+    const BfCfg cfg = pick_bf(C, S % 8 == 0 && aligned16(x) && aligned16(y), S, batch);
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
     BF_DISPATCH(rms_fwd_bf16_kernel, cfg, nblk, y, x, w, C, S, strips, nblk, eps, 1.0f / (float)C);
@@ -794,7 +796,7 @@ MI355_API int mi355_rmsnorm_bwd_bf16_dev(uint16_t *dx, float *dw, const uint16_t
     if (!dx || !dw || !dy || !x || !w) return mi355_fail("rmsnorm_bwd_bf16: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_bwd_bf16: bad shape C=%d S=%d batch=%d", C, S, batch);
     if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd_bf16: variant must be 0 or 1");
-    const BfCfg cfg = pick_bf(C, S % 8 == 0 && aligned16(x) && aligned16(dy) && aligned16(dx));
+    const BfCfg cfg = pick_bf(C, S % 8 == 0 && aligned16(x) && aligned16(dy) && aligned16(dx), S, batch);
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
     float *part = mi355_dw_partials((size_t)nblk * C, dw, nullptr);

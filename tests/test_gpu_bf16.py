@@ -65,7 +65,7 @@ def test_swiglu_and_residual_bf16(br, n):
 
 
 @pytest.mark.parametrize("B,C,S", [(16, 1024, 256), (1, 768, 256), (2, 100, 37), (3, 48, 24), (2, 5000, 64), (5, 128, 256),
-                                   (2, 300, 16), (1, 2048, 8), (1, 1, 8)])
+                                   (2, 300, 16), (1, 2048, 8), (1, 1, 8), (64, 1024, 256), (70, 640, 256)])
 def test_rmsnorm_bf16(br, B, C, S):
     print("[case] bf16 rmsnorm B=%d C=%d S=%d" % (B, C, S), flush=True)
     (xb, x), (dyb, dy) = bf(H.normal(220, (B, C, S))), bf(H.normal(221, (B, C, S)))

@@ -22,7 +22,8 @@ def _rms_shapes():
         S = int(rng.choice([rng.integers(1, 40), 4 * rng.integers(1, 80), 256]))
         B = int(rng.integers(1, 5))
         out.append((B, C, S))
-    return out + [(1, 2048, 256), (3, 2049, 12), (2, 4096, 64), (7, 16, 1024)]
+    # the last three have enough columns for the 128-byte strips (fp32 and bf16 pickers switch on strips x batch)
+    return out + [(1, 2048, 256), (3, 2049, 12), (2, 4096, 64), (7, 16, 1024), (32, 1024, 256), (40, 768, 256), (9, 600, 1024)]
 
 
 @pytest.mark.parametrize("B,C,S", _rms_shapes())
