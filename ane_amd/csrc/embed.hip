@@ -291,9 +291,6 @@ __global__ __launch_bounds__(1024) void seg_sum_kernel(float *__restrict__ dE, c
             for (int k = 0; k < nw; k++) {
                 const int seg = work[k];
                 const int lo = seg_start[seg], hi = seg_start[seg + 1];
-                const int tok = keys[lo];
-                float acc = 0.f;
-                if (wave == 0 && d_ok) acc = dE[(size_t)tok * D + d];
                 // Software pipeline: the rows of stage s+1 are already on their way into registers while wave 0
                 // adds the rows of stage s out of LDS.
                 float v[STAGE_PER_WAVE];
@@ -305,7 +302,10 @@ __global__ __launch_bounds__(1024) void seg_sum_kernel(float *__restrict__ dE, c
                         v[j] = (rl < nrow && d_ok) ? __builtin_nontemporal_load(rows + (size_t)(base + rl) * D + d) : 0.f;
                     }
                 };
-                fetch(lo);
+                fetch(lo);                               // first, so that the token id and the old dE row load beside it
+                const int tok = keys[lo];
+                float acc = 0.f;
+                if (wave == 0 && d_ok) acc = dE[(size_t)tok * D + d];
                 for (int base = lo; base < hi; base += STAGE_ROWS) {
                     const int nrow = min(STAGE_ROWS, hi - base);
                     if constexpr (TREE) {
