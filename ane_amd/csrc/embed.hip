@@ -115,10 +115,10 @@ struct ClampId {
 
 // meta[0] = number of segments, meta[2] = number of valid (in-range) entries.
 //
-// Segment starts are found in three small launches: (1) every workgroup flags the heads among its
+// Segment starts are found in two small launches: (1) every workgroup flags the heads among its
 // 1024 sorted entries (key differs from its predecessor), counts them and writes the inverse
-// permutation; (2) one workgroup scans the per-workgroup counts; (3) every workgroup writes the
-// positions of its heads at its offset.
+// permutation; (2) every workgroup adds up the counts before its own and writes the positions of its
+// heads at that offset.
 constexpr int PLAN_T = 1024;
 
 __device__ __forceinline__ int block_excl_scan_1024(int v, int *lds, int &total) {
@@ -165,28 +165,22 @@ __global__ __launch_bounds__(PLAN_T) void plan_flags_kernel(int *__restrict__ ra
     if (threadIdx.x == 0) blk_count[blockIdx.x] = total;
 }
 
-__global__ __launch_bounds__(PLAN_T) void plan_scan_kernel(int *__restrict__ blk_off, int *__restrict__ seg_start,
-                                                           int *__restrict__ meta, const int *__restrict__ blk_count,
-                                                           int nb) {
-    __shared__ int lds[PLAN_T / 64];
-    int carry = 0;
-    for (int b0 = 0; b0 < nb; b0 += PLAN_T) {
-        const int b = b0 + threadIdx.x;
-        const int v = b < nb ? blk_count[b] : 0;
-        int total;
-        const int ex = block_excl_scan_1024(v, lds, total);
-        if (b < nb) blk_off[b] = carry + ex;
-        carry += total;
-    }
-    if (threadIdx.x == 0) {
-        meta[0] = carry;
-        seg_start[carry] = meta[2];                 // end of the last segment = number of valid entries
-    }
-}
-
-__global__ __launch_bounds__(PLAN_T) void plan_write_kernel(int *__restrict__ seg_start, const int *__restrict__ blk_off,
+// Second (and last) launch: every workgroup sums the head counts of the workgroups before it (a few reads),
+// scans its own flags and writes its segment starts; the last one also writes the segment count and the end of
+// the last segment.
+__global__ __launch_bounds__(PLAN_T) void plan_write_kernel(int *__restrict__ seg_start, int *__restrict__ meta,
+                                                            const int *__restrict__ blk_count,
                                                             const int *__restrict__ keys, int N, int V) {
     __shared__ int lds[PLAN_T / 64];
+    __shared__ int before;
+    int part = 0;
+    for (int b = threadIdx.x; b < (int)blockIdx.x; b += PLAN_T) part += blk_count[b];
+    int dummy;
+    const int ex0 = block_excl_scan_1024(part, lds, dummy);     // dummy = total over the workgroup
+    (void)ex0;
+    if (threadIdx.x == 0) before = dummy;
+    __syncthreads();
+    const int off = before;
     const int i = blockIdx.x * PLAN_T + threadIdx.x;
     int head = 0;
     if (i < N) {
@@ -196,7 +190,11 @@ __global__ __launch_bounds__(PLAN_T) void plan_write_kernel(int *__restrict__ se
     }
     int total;
     const int ex = block_excl_scan_1024(head, lds, total);
-    if (head) seg_start[blk_off[blockIdx.x] + ex] = i;
+    if (head) seg_start[off + ex] = i;
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+        meta[0] = off + total;
+        seg_start[off + total] = meta[2];           // end of the last segment = number of valid entries
+    }
 }
 
 // dx [batch][D][S] -> rows[rank[n]][D] (token-major, in sorted order), through a 64x64 LDS tile
@@ -465,14 +463,13 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     const int nplan = (int)ceil_div((size_t)N, PLAN_T);
     const size_t off_keys = 0, off_vals = nb, off_rank = 2 * nb;
     const size_t off_seg = 3 * nb, off_cnt = off_seg + al((size_t)(N + 1) * sizeof(int));
-    const size_t off_boff = off_cnt + al((size_t)nplan * sizeof(int));
-    const size_t off_meta = off_boff + al((size_t)nplan * sizeof(int)), off_temp = off_meta + 256;
+    const size_t off_meta = off_cnt + al((size_t)nplan * sizeof(int)), off_temp = off_meta + 256;
     const size_t off_rows = off_temp + al(temp_bytes);
     const size_t total = off_rows + al((size_t)N * D * sizeof(float));
     char *ws = (char *)mi355_ws(total);
     if (!ws) return -1;
     int *keys = (int *)(ws + off_keys), *vals = (int *)(ws + off_vals), *rank = (int *)(ws + off_rank);
-    int *seg_start = (int *)(ws + off_seg), *blk_count = (int *)(ws + off_cnt), *blk_off = (int *)(ws + off_boff);
+    int *seg_start = (int *)(ws + off_seg), *blk_count = (int *)(ws + off_cnt);
     int *meta = (int *)(ws + off_meta);
     float *rows = (float *)(ws + off_rows);
 
@@ -481,9 +478,8 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     if (e != hipSuccess) return mi355_fail("embed_scatter_add: sort: %s", hipGetErrorString(e));
     hipLaunchKernelGGL(plan_flags_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, rank, blk_count, meta, keys, vals,
                        N, V);
-    hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(PLAN_T), 0, g_ctx.stream, blk_off, seg_start, meta, blk_count,
-                       nplan);
-    hipLaunchKernelGGL(plan_write_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, seg_start, blk_off, keys, N, V);
+    hipLaunchKernelGGL(plan_write_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, seg_start, meta, blk_count, keys, N,
+                       V);
     LAUNCH_OK("embed_scatter_add plan");
     const int t_tiles = (int)ceil_div((size_t)S, TT);
     const dim3 tgrid((unsigned)(batch * t_tiles), (unsigned)ceil_div((size_t)D, TD));
