@@ -9,14 +9,15 @@
 //
 // Scatter-add: the reference adds dx[:,t] into dE[tok_t] for t ascending, so each (row, d) sum has
 // a fixed order.  To reproduce it bit for bit:
-//   1. stable radix sort of (token, position) pairs by token (rocPRIM device primitive);
-//   2. dx is transposed through LDS into token-major rows written in SORTED order, so a
+//   1. the (token, position) pairs are put in token order, positions ascending within a token: for up to
+//      16 384 positions by counting smaller pairs (two small launches, no full sort), beyond that by the
+//      rocPRIM stable radix sort;
+//   2. dx is transposed through LDS into token-major rows written in that SORTED order, so a
 //      segment (all positions of one token) is a run of consecutive rows;
-//   3. each (segment, 64-float chunk) is summed sequentially starting from the value already
-//      in dE — short segments by one wave straight from memory, long segments by a whole
-//      workgroup that stages 240 rows at a time in LDS to keep enough loads in flight while one
-//      wave performs the ordered adds; both kinds share one launch so the long chains overlap
-//      the many short ones.
+//   3. each segment is summed sequentially starting from the value already in dE — short segments by one
+//      wave straight from memory, long segments by a whole workgroup whose other waves stage the rows in LDS
+//      while one wave performs the ordered adds; both kinds share one launch so the long chains overlap the
+//      many short ones.
 #include "common.h"
 
 #include <algorithm>
@@ -27,9 +28,11 @@ namespace {
 
 constexpr int TT = 64;   // tokens per tile
 constexpr int TD = 64;   // dims per tile
-constexpr int LONG_SEG = 64;    // segments longer than this take the workgroup path
-constexpr int STAGE_PER_WAVE = 15;
-constexpr int STAGE_ROWS = 16 * STAGE_PER_WAVE;   // 240 rows x 256 B = 60 KiB of LDS, plus a 4 KiB work list
+constexpr int LONG_SEG = 32;    // segments longer than this take the workgroup path
+constexpr int LCH = 32;             // floats per chunk of a long segment
+constexpr int MAX_ORDERED = 256;    // long segments that the segment-sum workgroups order by length
+constexpr int ROWS_PER_WAVE = 16;   // rows a staging wave brings in per stage
+constexpr int STAGE_ROWS = 15 * ROWS_PER_WAVE;    // two buffers of 240 rows x 128 B = 60 KiB of LDS
 
 // ---------------------------------------------------------------------------------------------
 // Gather
@@ -113,12 +116,16 @@ struct ClampId {
     __host__ __device__ int operator()(int32_t id) const { return (id < 0 || id >= V) ? V : id; }
 };
 
-// meta[0] = number of segments, meta[2] = number of valid (in-range) entries.
+// What the segment sums read: seg_list[i] = {first row, end row, token, 0} of segment i (rows = sorted
+// positions), long_list = the entries of the long segments, meta[0] / meta[1] = the lengths of the two lists,
+// qhead[c] = next entry of the long list that the workgroups of column chunk c have not taken yet (the first
+// long_x entries are taken without asking); rank[position] = its row.
 //
-// Segment starts are found in two small launches: (1) every workgroup flags the heads among its
-// 1024 sorted entries (key differs from its predecessor), counts them and writes the inverse
-// permutation; (2) every workgroup adds up the counts before its own and writes the positions of its
-// heads at that offset.
+// Large inputs (more than 16 384 positions, or a vocabulary of 2^18 and more): the library sort, then (1) every
+// workgroup flags the heads among its 1024 sorted entries (key differs from its predecessor), counts them and
+// writes the inverse permutation; (2) every workgroup adds up the counts before its own and writes the positions
+// of its heads at that offset (meta[2] = number of in-range entries = end of the last segment); (3) one thread per
+// segment writes the list entries.
 constexpr int PLAN_T = 1024;
 
 __device__ __forceinline__ int block_excl_scan_1024(int v, int *lds, int &total) {
@@ -145,10 +152,16 @@ __device__ __forceinline__ int block_excl_scan_1024(int v, int *lds, int &total)
 }
 
 __global__ __launch_bounds__(PLAN_T) void plan_flags_kernel(int *__restrict__ rank, int *__restrict__ blk_count,
-                                                            int *__restrict__ meta, const int *__restrict__ keys,
-                                                            const int *__restrict__ vals, int N, int V) {
+                                                            int *__restrict__ meta, int *__restrict__ qhead,
+                                                            const int *__restrict__ keys,
+                                                            const int *__restrict__ vals, int N, int V, int nq,
+                                                            int long_x) {
     __shared__ int lds[PLAN_T / 64];
     const int i = blockIdx.x * PLAN_T + threadIdx.x;
+    if (blockIdx.x == 0) {
+        if (threadIdx.x == 0) meta[1] = 0;
+        for (int c = threadIdx.x; c < nq; c += PLAN_T) qhead[c] = long_x;
+    }
     int head = 0;
     if (i < N) {
         const int k = keys[i];
@@ -195,6 +208,163 @@ __global__ __launch_bounds__(PLAN_T) void plan_write_kernel(int *__restrict__ se
         meta[0] = off + total;
         seg_start[off + total] = meta[2];           // end of the last segment = number of valid entries
     }
+}
+
+// The plan for N <= 16 384 positions and a vocabulary below 2^18, in two launches and without a sort of the whole
+// array.  A (token, position) pair is packed into one word, token above position; all words are distinct, and the
+// sorted index of a position is the number of words smaller than its own.
+//   1. chunk_sort_kernel: every 256 consecutive words are sorted by counting, within their workgroup.
+//   2. rank_list_kernel: every workgroup holds all sorted chunks in LDS (64 KiB); 16 lanes share one position
+//      and binary-search four chunks each for (a) the number of smaller words = the sorted index, (b) the largest
+//      smaller word = the predecessor, which tells whether the position is the first of its token, and (c) the
+//      number of words up to the last one of the same token = the end of the segment.  First positions append
+//      their segment {first row, end row, token} to the segment list, and to the long list if it is long.  The
+//      order of the lists depends on the order of the atomic appends; the sums do not, since a segment is summed
+//      by whoever takes it, from its own rows only.
+constexpr int SMALL_N = 16384, POS_BITS = 14, CHUNK = 256, CHUNK_PITCH = CHUNK + 1;
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ unsigned pack_word(const int32_t *__restrict__ ids, int i, int N, int V) {
+    unsigned key = (unsigned)V;                             // padding and out-of-range ids sort last
+    if (i < N) {
+        const int id = ids[i];
+        if (id >= 0 && id < V) key = (unsigned)id;
+    }
+    return (key << POS_BITS) | (unsigned)i;
+}
+
+__global__ __launch_bounds__(CHUNK) void chunk_sort_kernel(unsigned *__restrict__ sorted_chunks, int *__restrict__ meta,
+                                                           int *__restrict__ qhead, const int32_t *__restrict__ ids,
+                                                           int N, int V, int nq, int long_x) {
+    __shared__ __attribute__((aligned(16))) unsigned sw[CHUNK];
+    const int t = threadIdx.x;
+    if (blockIdx.x == 0) {
+        if (t < 2) meta[t] = 0;
+        for (int c = t; c < nq; c += CHUNK) qhead[c] = long_x;
+    }
+    const unsigned w = pack_word(ids, blockIdx.x * CHUNK + t, N, V);
+    sw[t] = w;
+    __syncthreads();
+    int r = 0;
+#pragma unroll 8
+    for (int j = 0; j < CHUNK; j += 4) {
+        const v4u q = *reinterpret_cast<const v4u *>(&sw[j]);
+        r += (q.x < w ? 1 : 0) + (q.y < w ? 1 : 0) + (q.z < w ? 1 : 0) + (q.w < w ? 1 : 0);
+    }
+    sorted_chunks[blockIdx.x * CHUNK + r] = w;
+}
+
+__global__ __launch_bounds__(1024) void rank_list_kernel(int *__restrict__ rank, v4i *__restrict__ seg_list,
+                                                         v4i *__restrict__ long_list, int *__restrict__ meta,
+                                                         const unsigned *__restrict__ sorted_chunks,
+                                                         const int32_t *__restrict__ ids, int N, int V, int nchunks) {
+    __shared__ unsigned sc[(SMALL_N / CHUNK) * CHUNK_PITCH];    // pitch 257: lanes on different chunks, different banks
+    __shared__ int nh, nl, base_h, base_l;
+    const int t = threadIdx.x;
+    {
+        v4u q[SMALL_N / 4096];                                  // all loads first, then the LDS writes
+#pragma unroll
+        for (int i = 0; i < SMALL_N / 4096; i++) {
+            const int j = i * 4096 + t * 4;
+            q[i] = j < nchunks * CHUNK ? *reinterpret_cast<const v4u *>(&sorted_chunks[j]) : v4u{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int i = 0; i < SMALL_N / 4096; i++) {
+            const int j = i * 4096 + t * 4;
+            unsigned *dst = sc + (j / CHUNK) * CHUNK_PITCH + (j % CHUNK);
+            dst[0] = q[i].x; dst[1] = q[i].y; dst[2] = q[i].z; dst[3] = q[i].w;
+        }
+    }
+    const int k = t & 15, e = blockIdx.x * 64 + (t >> 4);       // position e, helper lane k of 16
+    const unsigned w = pack_word(ids, e, N, V);
+    const unsigned key = w >> POS_BITS;
+    __syncthreads();
+    // the four searches of a lane are independent chains of LDS reads and run interleaved; a chunk index past the
+    // end is searched as chunk 0 and not counted
+    constexpr int PER_LANE = SMALL_N / CHUNK / 16;
+    const unsigned *chp[PER_LANE];
+    bool okc[PER_LANE];
+#pragma unroll
+    for (int m = 0; m < PER_LANE; m++) {
+        okc[m] = k + 16 * m < nchunks;
+        chp[m] = sc + (okc[m] ? k + 16 * m : 0) * CHUNK_PITCH;
+    }
+    auto count_below = [&](unsigned x, int (&p)[PER_LANE]) {      // per chunk: number of words < x
+#pragma unroll
+        for (int m = 0; m < PER_LANE; m++) p[m] = 0;
+#pragma unroll
+        for (int st = CHUNK / 2; st >= 1; st >>= 1) {
+#pragma unroll
+            for (int m = 0; m < PER_LANE; m++)
+                if (chp[m][p[m] + st - 1] < x) p[m] += st;
+        }
+#pragma unroll
+        for (int m = 0; m < PER_LANE; m++) p[m] += chp[m][p[m]] < x ? 1 : 0;
+    };
+    int p[PER_LANE];
+    count_below(w, p);
+    int below = 0;
+    unsigned pred1 = 0;                                         // largest smaller word + 1, or 0 if there is none
+#pragma unroll
+    for (int m = 0; m < PER_LANE; m++)
+        if (okc[m]) {
+            below += p[m];
+            if (p[m] > 0) pred1 = max(pred1, chp[m][p[m] - 1] + 1u);
+        }
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) {
+        below += __shfl_xor(below, m, 64);
+        pred1 = max(pred1, (unsigned)__shfl_xor((int)pred1, m, 64));
+    }
+    // the 16 lanes of a position agree on whether it is the first of its token; only then is the end searched
+    const bool first = e < N && key < (unsigned)V && (pred1 == 0 || ((pred1 - 1u) >> POS_BITS) != key);
+    int upto = 0;
+    if (first) {
+        // words up to the last one of this token = words below the first word of the next token (no overflow:
+        // a first position has key < V < 2^18)
+        count_below(((key + 1u) << POS_BITS), p);
+#pragma unroll
+        for (int m = 0; m < PER_LANE; m++) upto += okc[m] ? p[m] : 0;
+#pragma unroll
+        for (int m = 1; m < 16; m <<= 1) upto += __shfl_xor(upto, m, 64);
+    }
+    // one append per workgroup and list: the heads take their places within the workgroup through LDS
+    const bool mine = k == 0 && e < N;
+    const bool head = mine && first;
+    const bool is_long = head && upto - below > LONG_SEG;
+    if (t == 0) nh = nl = 0;
+    __syncthreads();
+    int ih = 0, il = 0;
+    if (head) ih = atomicAdd(&nh, 1);
+    if (is_long) il = atomicAdd(&nl, 1);
+    __syncthreads();
+    if (t == 0 && nh) {
+        // both list lengths move with one 64-bit atomic (meta[0] is its low word, meta[1] its high word): the
+        // appends of all workgroups queue up on this one address
+        const unsigned long long old = atomicAdd(reinterpret_cast<unsigned long long *>(meta),
+                                                 ((unsigned long long)(unsigned)nl << 32) | (unsigned)nh);
+        base_h = (int)(old & 0xffffffffu);
+        base_l = (int)(old >> 32);
+    }
+    __syncthreads();
+    if (mine) rank[e] = below;
+    if (head) {
+        const v4i entry = {below, upto, (int)key, 0};
+        seg_list[base_h + ih] = entry;
+        if (is_long) long_list[base_l + il] = entry;
+    }
+}
+
+// Large plan, last launch: one thread per segment writes its list entry; the long ones also go to the long list.
+__global__ __launch_bounds__(PLAN_T) void plan_list_kernel(v4i *__restrict__ seg_list, v4i *__restrict__ long_list,
+                                                           int *__restrict__ meta, const int *__restrict__ seg_start,
+                                                           const int *__restrict__ keys) {
+    const int seg = blockIdx.x * PLAN_T + threadIdx.x;
+    if (seg >= meta[0]) return;
+    const int lo = seg_start[seg], hi = seg_start[seg + 1];
+    const v4i entry = {lo, hi, keys[lo], 0};
+    seg_list[seg] = entry;
+    if (hi - lo > LONG_SEG) long_list[atomicAdd(&meta[1], 1)] = entry;
 }
 
 // dx [batch][D][S] -> rows[rank[n]][D] (token-major, in sorted order), through a 64x64 LDS tile
@@ -252,125 +422,205 @@ __global__ __launch_bounds__(256) void transpose_sorted_kernel(float *__restrict
 }
 
 // Segment sums.  One launch, two kinds of workgroup (1024 threads each):
-//  * the first `long_blocks` workgroups take the LONG segments (more than LONG_SEG rows): workgroup
-//    (x, chunk) walks segments x, x + gridDim.x/..., and for each long one sums its 64-float chunk: 16 waves
-//    stage 240 rows in LDS (15 loads in flight per lane), wave 0 adds them in order, 16 rows per batch of
-//    LDS reads so the adds are not exposed to the LDS latency;
-//  * the others take the short segments: one wave per (segment, 64-float chunk), rows read straight
+//  * the first `long_blocks` workgroups take the LONG segments (more than LONG_SEG rows).  Every one of them
+//    orders the long list by length (longest first, so that the longest chain of dependent adds starts at once
+//    and shares its workgroup with nothing else); workgroup (x, chunk) takes entry x of that order, then
+//    whatever entry the workgroups of its chunk have not taken yet, and sums the entry's 32-float chunk.  Waves 1-15
+//    stage the rows, 240 per stage: two rows per load instruction, eight loads per lane, three stages in
+//    flight in registers (720 rows, enough to cover the memory latency at the rate the adds consume them), and
+//    write them into one of two LDS buffers.  Wave 0 adds the rows of the other buffer in order, with the LDS
+//    reads of the next 16 rows issued ahead of the adds of the current 16, so the dependent adds run back to
+//    back.  One barrier per stage.
+//  * the others take the short segments: one wave per (segment, 256-float block), rows read straight
 //    from memory, eight loads in flight.
 // Either way every (row of dE, d) is written by exactly one lane, sequentially in position order,
-// starting from the value already in dE.
+// starting from the value already in dE.  Rows past the end of a segment are staged as -0.0f, which leaves
+// every float unchanged when added (+0.0f would turn a -0.0f sum into +0.0f).
 template <bool TREE>
-__global__ __launch_bounds__(1024) void seg_sum_kernel(float *__restrict__ dE, const float *__restrict__ rows,
-                                                       const int *__restrict__ seg_start, const int *__restrict__ keys,
-                                                       const int *__restrict__ meta, int D, int nchunk,
-                                                       int long_x, int short_blocks) {
-    __shared__ float stage[STAGE_ROWS][64];
-    __shared__ int work[1023];      // with nwork: 4 KiB, for 64 KiB of LDS in all
-    __shared__ int nwork;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+__global__ __launch_bounds__(1024, 8) void seg_sum_kernel(float *__restrict__ dE, const float *__restrict__ rows,
+                                                       const v4i *__restrict__ seg_list,
+                                                       const int *__restrict__ meta, const v4i *__restrict__ long_list,
+                                                       int *__restrict__ qhead, int D, int nchunk, int nchunk_long,
+                                                       int long_x, int short_blocks, bool vec) {
+    __shared__ float stage[2][STAGE_ROWS][LCH];
+    __shared__ v4i ent[MAX_ORDERED];
+    __shared__ short order[MAX_ORDERED];
+    __shared__ int next_item;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nseg = meta[0];
-    const int long_blocks = long_x * nchunk;
+    const int long_blocks = long_x * nchunk_long;
     if ((int)blockIdx.x < long_blocks) {
-        const int ch = blockIdx.x % nchunk, x0 = blockIdx.x / nchunk;
-        const int d = ch * 64 + lane;
+        const int ch = blockIdx.x % nchunk_long, x0 = blockIdx.x / nchunk_long;
+        const int col = lane & (LCH - 1), sub = lane / LCH;      // a load instruction covers rows r and r+1
+        const int d = ch * LCH + col;
         const bool d_ok = d < D;
-        // candidates of this workgroup column: segments x0, x0+long_x, ...; 1023 are screened at a time
-        for (int j0 = 0; x0 + (long)j0 * long_x < nseg; j0 += 1023) {
-            if (threadIdx.x == 0) nwork = 0;
-            __syncthreads();
+        // the long list in LDS, longest first (ties: smaller first row); beyond MAX_ORDERED entries, as listed.
+        // The entries are fetched before their number is known (the list has room for MAX_ORDERED and more), so
+        // that the two loads travel together.
+        v4i mine = {0, 0, 0, 0};
+        if (threadIdx.x < MAX_ORDERED) mine = long_list[threadIdx.x];
+        const int nlong = meta[1];
+        if (x0 >= nlong) return;
+        const int nord = min(nlong, MAX_ORDERED);
+        if ((int)threadIdx.x < nord) ent[threadIdx.x] = mine;
+        __syncthreads();
+        if ((int)threadIdx.x < nord && nlong <= MAX_ORDERED) {
+            const v4i ea = ent[threadIdx.x];
+            const int la = ea.y - ea.x;
+            int before = 0;
+            for (int b = 0; b < nord; b++) {
+                const v4i eb = ent[b];
+                const int lb = eb.y - eb.x;
+                before += (lb > la || (lb == la && eb.x < ea.x)) ? 1 : 0;
+            }
+            order[before] = (short)threadIdx.x;
+        }
+        __syncthreads();
+        for (int item = x0; item < nlong;) {
             {
-                const long seg = x0 + (long)(j0 + (int)threadIdx.x) * long_x;
-                if (threadIdx.x < 1023 && seg < nseg && seg_start[seg + 1] - seg_start[seg] > LONG_SEG)
-                    work[atomicAdd(&nwork, 1)] = (int)seg;
-            }
-            __syncthreads();
-            const int nw = nwork;
-            for (int k = 0; k < nw; k++) {
-                const int seg = work[k];
-                const int lo = seg_start[seg], hi = seg_start[seg + 1];
-                // Software pipeline: the rows of stage s+1 are already on their way into registers while wave 0
-                // adds the rows of stage s out of LDS.
-                float v[STAGE_PER_WAVE];
-                auto fetch = [&](int base) {
-                    const int nrow = min(STAGE_ROWS, hi - base);
-#pragma unroll
-                    for (int j = 0; j < STAGE_PER_WAVE; j++) {
-                        const int rl = wave * STAGE_PER_WAVE + j;
-                        v[j] = (rl < nrow && d_ok) ? __builtin_nontemporal_load(rows + (size_t)(base + rl) * D + d) : 0.f;
-                    }
-                };
-                fetch(lo);                               // first, so that the token id and the old dE row load beside it
-                const int tok = keys[lo];
-                float acc = 0.f;
-                if (wave == 0 && d_ok) acc = dE[(size_t)tok * D + d];
-                for (int base = lo; base < hi; base += STAGE_ROWS) {
-                    const int nrow = min(STAGE_ROWS, hi - base);
-                    if constexpr (TREE) {
-                        // fixed tree instead of the reference's chain (opt-in, "scatter_tree" knob): every wave sums
-                        // its 15 rows in order, wave 0 adds the 16 partial rows in wave order.  Deterministic, 8x
-                        // shorter chain, but rounded differently from the CPU loop.  Rows past the end are zeros.
-                        float p = v[0];
-#pragma unroll
-                        for (int j = 1; j < STAGE_PER_WAVE; j++) p += v[j];
-                        stage[wave][lane] = p;
+                const v4i e = nlong <= MAX_ORDERED ? ent[order[item]] : long_list[item];
+                const int lo = __builtin_amdgcn_readfirstlane(e.x), hi = __builtin_amdgcn_readfirstlane(e.y);
+                const int tok = __builtin_amdgcn_readfirstlane(e.z);
+                const int nstage = (hi - lo + STAGE_ROWS - 1) / STAGE_ROWS;
+                // The two roles run separate loops (so that neither carries the other's registers) and meet at
+                // one barrier per stage: barrier s tells wave 0 that buffer s&1 is complete, and tells the staging
+                // waves that wave 0 has finished with the other buffer.
+                if (wave == 0) {
+                    // this wave's chain of dependent adds sets the time of the launch: it goes first whenever it can issue
+                    __builtin_amdgcn_s_setprio(3);
+                    float acc = d_ok ? dE[(size_t)tok * D + d] : 0.f;
+                    for (int s = 0; s < nstage; s++) {
+                        float(*buf)[LCH] = stage[s & 1];
                         __syncthreads();
-                        if (base + STAGE_ROWS < hi) fetch(base + STAGE_ROWS);
-                        if (wave == 0) {
+                        if constexpr (TREE) {
+                            float t[30];
 #pragma unroll
-                            for (int q = 0; q < 16; q++) acc += stage[q][lane];
+                            for (int q = 0; q < 30; q++) t[q] = buf[q][col];
+#pragma unroll
+                            for (int q = 0; q < 30; q++) acc += t[q];
+                        } else {
+                            const int nrow = min(STAGE_ROWS, hi - (lo + s * STAGE_ROWS));
+                            if (nrow == STAGE_ROWS) {
+                                float t[2][16];
+#pragma unroll
+                                for (int j = 0; j < 16; j++) t[0][j] = buf[j][col];
+#pragma unroll
+                                for (int b = 0; b < STAGE_ROWS / 16; b++) {
+                                    if (b + 1 < STAGE_ROWS / 16) {
+#pragma unroll
+                                        for (int j = 0; j < 16; j++) t[(b + 1) & 1][j] = buf[(b + 1) * 16 + j][col];
+                                    }
+                                    // without the fences the compiler moves the reads down to 8 rows ahead of
+                                    // their adds, which exposes part of the LDS latency (1.42 us per stage; 1.13 with)
+                                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                                    for (int j = 0; j < 16; j++) acc += t[b & 1][j];
+                                    __builtin_amdgcn_sched_barrier(0);
+                                }
+                            } else {
+                                for (int rl = 0; rl < nrow; rl += 16) {      // rows past nrow hold -0.0f
+                                    float t[16];
+#pragma unroll
+                                    for (int j = 0; j < 16; j++) t[j] = buf[rl + j][col];
+#pragma unroll
+                                    for (int j = 0; j < 16; j++) acc += t[j];
+                                }
+                            }
                         }
+                    }
+                    if (sub == 0 && d_ok) dE[(size_t)tok * D + d] = acc;
+                    __builtin_amdgcn_s_setprio(0);
+                } else {
+                    float g0[8], g1[8], g2[8];
+                    auto fetch = [&](float (&g)[8], int s) {
+                        const int r0 = lo + s * STAGE_ROWS + (wave - 1) * ROWS_PER_WAVE + sub;
+#pragma unroll
+                        for (int j = 0; j < 8; j++) {
+                            const int r = r0 + 2 * j;
+                            g[j] = (r < hi && d_ok) ? __builtin_nontemporal_load(rows + (size_t)r * D + d) : -0.0f;
+                        }
+                    };
+                    auto put = [&](float (&g)[8], int s) {
+                        if (s >= nstage) return;
+                        float(*buf)[LCH] = stage[s & 1];
+                        if constexpr (TREE) {
+                            // fixed tree instead of the reference's chain (opt-in, "scatter_tree" knob): every lane
+                            // sums its 8 rows of the stage in order, wave 0 adds the 30 partial rows in order.
+                            // Deterministic, 8x shorter chain, but rounded differently from the CPU loop.
+                            float p = g[0];
+#pragma unroll
+                            for (int j = 1; j < 8; j++) p += g[j];
+                            buf[(wave - 1) * 2 + sub][col] = p;
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 8; j++) buf[(wave - 1) * ROWS_PER_WAVE + sub + 2 * j][col] = g[j];
+                        }
+                        fetch(g, s + 3);
                         __syncthreads();
-                        continue;
+                    };
+                    fetch(g0, 0);
+                    fetch(g1, 1);
+                    fetch(g2, 2);
+                    for (int s = 0; s < nstage; s += 3) {
+                        put(g0, s);
+                        put(g1, s + 1);
+                        put(g2, s + 2);
                     }
-#pragma unroll
-                    for (int j = 0; j < STAGE_PER_WAVE; j++) stage[wave * STAGE_PER_WAVE + j][lane] = v[j];
-                    __syncthreads();
-                    if (base + STAGE_ROWS < hi) fetch(base + STAGE_ROWS);
-                    if (wave == 0) {
-                        int rl = 0;
-                        for (; rl + 16 <= nrow; rl += 16) {
-                            float t[16];
-#pragma unroll
-                            for (int j = 0; j < 16; j++) t[j] = stage[rl + j][lane];
-#pragma unroll
-                            for (int j = 0; j < 16; j++) acc += t[j];
-                        }
-                        for (; rl < nrow; rl++) acc += stage[rl][lane];
-                    }
-                    __syncthreads();
                 }
-                if (wave == 0 && d_ok) dE[(size_t)tok * D + d] = acc;
             }
+            if (threadIdx.x == 0) next_item = atomicAdd(&qhead[ch], 1);
+            __syncthreads();             // also: the next segment's first stage reuses buffer 0
+            item = next_item;
             __syncthreads();
         }
         return;
     }
-    // short segments
-    const int gw = ((int)blockIdx.x - long_blocks) * 16 + wave;
+    // short segments: one wave per (segment, block of 256 columns), 128 bits per lane (64 columns and 32 bits
+    // per lane when D is not a multiple of 4)
+    const int gw = __builtin_amdgcn_readfirstlane(((int)blockIdx.x - long_blocks) * 16 + wave);
     const int nwaves = short_blocks * 16;
     const long units = (long)nseg * nchunk;
     for (long u = gw; u < units; u += nwaves) {
         const int seg = (int)(u / nchunk), ch = (int)(u - (long)seg * nchunk);
-        const int lo = seg_start[seg], hi = seg_start[seg + 1];
+        const v4i e = seg_list[seg];
+        const int lo = __builtin_amdgcn_readfirstlane(e.x), hi = __builtin_amdgcn_readfirstlane(e.y);
         if (hi - lo > LONG_SEG) continue;
-        const int d = ch * 64 + lane;
-        if (d >= D) continue;
-        const int tok = keys[lo];
-        float *dst = dE + (size_t)tok * D + d;
-        float acc = *dst;
-        const float *src = rows + (size_t)lo * D + d;
-        int r = lo;
-        for (; r + 8 <= hi; r += 8) {
-            float v[8];
+        const int tok = __builtin_amdgcn_readfirstlane(e.z);
+        if (vec) {
+            const int d = ch * 256 + lane * 4;
+            if (d >= D) continue;
+            float *dst = dE + (size_t)tok * D + d;
+            const float *src = rows + (size_t)lo * D + d;
+            v4f acc = ld4(dst);
+            int r = lo;
+            for (; r + 8 <= hi; r += 8) {
+                v4f v[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) v[j] = __builtin_nontemporal_load(src + (size_t)j * D);
+                for (int j = 0; j < 8; j++) v[j] = ld4_nt(src + (size_t)j * D);
 #pragma unroll
-            for (int j = 0; j < 8; j++) acc += v[j];
-            src += (size_t)8 * D;
+                for (int j = 0; j < 8; j++) acc += v[j];
+                src += (size_t)8 * D;
+            }
+            for (; r < hi; r++) { acc += ld4_nt(src); src += D; }
+            st4(dst, acc);
+        } else {
+            const int d = ch * 64 + lane;
+            if (d >= D) continue;
+            float *dst = dE + (size_t)tok * D + d;
+            const float *src = rows + (size_t)lo * D + d;
+            float acc = *dst;
+            int r = lo;
+            for (; r + 8 <= hi; r += 8) {
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = __builtin_nontemporal_load(src + (size_t)j * D);
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc += v[j];
+                src += (size_t)8 * D;
+            }
+            for (; r < hi; r++) { acc += __builtin_nontemporal_load(src); src += D; }
+            *dst = acc;
         }
-        for (; r < hi; r++) { acc += __builtin_nontemporal_load(src); src += D; }
-        *dst = acc;
     }
 }
 
@@ -443,7 +693,6 @@ MI355_API int mi355_embed_gather_dev(float *x, const float *E, const int32_t *id
 MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, int V, int D, int S,
                                           int batch) {
     if (!mi355_ready("embed_scatter_add")) return -1;
-    if (!mi355_outside_capture("embed_scatter_add (its library sort may record memset nodes)")) return -1;
     if (!dE || !dx || !ids) return mi355_fail("embed_scatter_add: NULL pointer");
     if (V <= 0 || D <= 0 || S <= 0 || batch <= 0)
         return mi355_fail("embed_scatter_add: bad shape V=%d D=%d S=%d batch=%d", V, D, S, batch);
@@ -451,53 +700,81 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     if (!aligned16(dx) || !aligned16(dE)) return mi355_fail("embed_scatter_add: pointers must be 16-byte aligned");
     const int N = batch * S;
     const int bits = key_bits(V);
+    const bool small = N <= SMALL_N && bits + POS_BITS <= 32;
+    if (!small &&
+        !mi355_outside_capture("embed_scatter_add beyond 16384 positions or a vocabulary of 2^18 (its library sort may "
+                               "record memset nodes)"))
+        return -1;
+    const bool vec = (D % 4 == 0);          // rows and dE are 16-byte aligned, so every row start is too
+    const int nchunk = (int)ceil_div((size_t)D, vec ? 256 : 64), nchunk_long = (int)ceil_div((size_t)D, LCH);
+    const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
+    // Every workgroup of the segment-sum launch reserves 64 KiB of LDS, so two fit on a compute unit and the grid is
+    // kept near one round of them: a larger grid is started only as fast as earlier workgroups retire.  At most
+    // N/(LONG_SEG+1) segments can be long.
+    const int max_long = std::max(N / (LONG_SEG + 1) + 1, MAX_ORDERED);
+    const int long_x = std::min(max_long, std::max(1, cu / nchunk_long));
 
     size_t temp_bytes = 0;
-    hipError_t e = rocprim::radix_sort_pairs(nullptr, temp_bytes, rocprim::make_transform_iterator(ids, ClampId{V}),
-                                             (int *)nullptr, rocprim::counting_iterator<int>(0), (int *)nullptr,
-                                             (size_t)N, 0, bits, g_ctx.stream);
-    if (e != hipSuccess) return mi355_fail("embed_scatter_add: sort sizing: %s", hipGetErrorString(e));
+    hipError_t e = hipSuccess;
+    if (!small) {
+        e = rocprim::radix_sort_pairs(nullptr, temp_bytes, rocprim::make_transform_iterator(ids, ClampId{V}),
+                                      (int *)nullptr, rocprim::counting_iterator<int>(0), (int *)nullptr, (size_t)N, 0,
+                                      bits, g_ctx.stream);
+        if (e != hipSuccess) return mi355_fail("embed_scatter_add: sort sizing: %s", hipGetErrorString(e));
+    }
 
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
     const size_t nb = al((size_t)N * sizeof(int));
     const int nplan = (int)ceil_div((size_t)N, PLAN_T);
+    const int nchunks = (int)ceil_div((size_t)N, CHUNK);
     const size_t off_keys = 0, off_vals = nb, off_rank = 2 * nb;
     const size_t off_seg = 3 * nb, off_cnt = off_seg + al((size_t)(N + 1) * sizeof(int));
-    const size_t off_meta = off_cnt + al((size_t)nplan * sizeof(int)), off_temp = off_meta + 256;
-    const size_t off_rows = off_temp + al(temp_bytes);
+    const size_t off_meta = off_cnt + al((size_t)nplan * sizeof(int));
+    const size_t off_long = off_meta + 256, off_list = off_long + al((size_t)max_long * sizeof(v4i));
+    const size_t off_q = off_list + al((size_t)N * sizeof(v4i));
+    const size_t off_temp = off_q + al((size_t)nchunk_long * sizeof(int));
+    const size_t off_chunks = off_temp + al(temp_bytes);
+    const size_t off_rows = off_chunks + al(small ? (size_t)nchunks * CHUNK * sizeof(unsigned) : 0);
     const size_t total = off_rows + al((size_t)N * D * sizeof(float));
     char *ws = (char *)mi355_ws(total);
     if (!ws) return -1;
     int *keys = (int *)(ws + off_keys), *vals = (int *)(ws + off_vals), *rank = (int *)(ws + off_rank);
     int *seg_start = (int *)(ws + off_seg), *blk_count = (int *)(ws + off_cnt);
-    int *meta = (int *)(ws + off_meta);
+    int *meta = (int *)(ws + off_meta), *qhead = (int *)(ws + off_q);
+    v4i *long_list = (v4i *)(ws + off_long), *seg_list = (v4i *)(ws + off_list);
     float *rows = (float *)(ws + off_rows);
 
-    e = rocprim::radix_sort_pairs(ws + off_temp, temp_bytes, rocprim::make_transform_iterator(ids, ClampId{V}), keys,
-                                  rocprim::counting_iterator<int>(0), vals, (size_t)N, 0, bits, g_ctx.stream);
-    if (e != hipSuccess) return mi355_fail("embed_scatter_add: sort: %s", hipGetErrorString(e));
-    hipLaunchKernelGGL(plan_flags_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, rank, blk_count, meta, keys, vals,
-                       N, V);
-    hipLaunchKernelGGL(plan_write_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, seg_start, meta, blk_count, keys, N,
-                       V);
+    if (small) {
+        unsigned *sorted_chunks = (unsigned *)(ws + off_chunks);
+        hipLaunchKernelGGL(chunk_sort_kernel, dim3(nchunks), dim3(CHUNK), 0, g_ctx.stream, sorted_chunks, meta, qhead, ids,
+                           N, V, nchunk_long, long_x);
+        hipLaunchKernelGGL(rank_list_kernel, dim3((unsigned)ceil_div((size_t)N, 64)), dim3(1024), 0, g_ctx.stream, rank,
+                           seg_list, long_list, meta, sorted_chunks, ids, N, V, nchunks);
+    } else {
+        e = rocprim::radix_sort_pairs(ws + off_temp, temp_bytes, rocprim::make_transform_iterator(ids, ClampId{V}), keys,
+                                      rocprim::counting_iterator<int>(0), vals, (size_t)N, 0, bits, g_ctx.stream);
+        if (e != hipSuccess) return mi355_fail("embed_scatter_add: sort: %s", hipGetErrorString(e));
+        hipLaunchKernelGGL(plan_flags_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, rank, blk_count, meta, qhead,
+                           keys, vals, N, V, nchunk_long, long_x);
+        hipLaunchKernelGGL(plan_write_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, seg_start, meta, blk_count,
+                           keys, N, V);
+        hipLaunchKernelGGL(plan_list_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, seg_list, long_list, meta,
+                           seg_start, keys);
+    }
     LAUNCH_OK("embed_scatter_add plan");
     const int t_tiles = (int)ceil_div((size_t)S, TT);
     const dim3 tgrid((unsigned)(batch * t_tiles), (unsigned)ceil_div((size_t)D, TD));
     if (tgrid.y > 65535) return mi355_fail("embed_scatter_add: D too large");
     hipLaunchKernelGGL(transpose_sorted_kernel, tgrid, dim3(256), 0, g_ctx.stream, rows, dx, rank, D, S, t_tiles);
     LAUNCH_OK("embed_scatter_add transpose");
-    const int nchunk = (int)ceil_div((size_t)D, 64);
-    const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
-    // at most N/LONG_SEG segments can be long; a few dozen workgroup columns cover them
-    int long_x = (int)std::min<size_t>((size_t)N / LONG_SEG + 1, (size_t)std::max(1, cu / nchunk));
-    size_t short_blocks = ceil_div((size_t)N * nchunk, 16);
-    if (short_blocks > (size_t)cu * 4) short_blocks = (size_t)cu * 4;
+    const size_t short_blocks = std::min<size_t>(ceil_div((size_t)N * nchunk, 16), (size_t)cu);
+    const dim3 sgrid((unsigned)((size_t)long_x * nchunk_long + short_blocks));
     if (g_ctx.scatter_tree)
-        hipLaunchKernelGGL(seg_sum_kernel<true>, dim3((unsigned)(long_x * nchunk + short_blocks)), dim3(1024), 0,
-                           g_ctx.stream, dE, rows, seg_start, keys, meta, D, nchunk, long_x, (int)short_blocks);
+        hipLaunchKernelGGL(seg_sum_kernel<true>, sgrid, dim3(1024), 0, g_ctx.stream, dE, rows, seg_list, meta,
+                           long_list, qhead, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec);
     else
-        hipLaunchKernelGGL(seg_sum_kernel<false>, dim3((unsigned)(long_x * nchunk + short_blocks)), dim3(1024), 0,
-                           g_ctx.stream, dE, rows, seg_start, keys, meta, D, nchunk, long_x, (int)short_blocks);
+        hipLaunchKernelGGL(seg_sum_kernel<false>, sgrid, dim3(1024), 0, g_ctx.stream, dE, rows, seg_list, meta,
+                           long_list, qhead, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec);
     LAUNCH_OK("embed_scatter_add segment sums");
     return 0;
 }

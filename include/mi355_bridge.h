@@ -108,8 +108,8 @@ int mi355_qknorm_rope_bwd_bf16_dev(uint16_t *dq, uint16_t *dk, float *dwq, float
 /* Graphs: record a launch-bound sequence of device-resident ops once, replay it as one submission.  No
  * counterpart in the reference (its ops are synchronous CPU calls).  Between begin and end the *_dev ops are
  * recorded instead of run; calls that allocate, wait or touch the host (buf_alloc/free/read/write, sync,
- * set_stream, workspace growth, a first-time RoPE table, embed_scatter_add, sgemm, ckpt_*) fail with -1 and end
- * in a failed capture, so run the sequence once eagerly first.  mi355_graph_launch enqueues the replay on the
+ * set_stream, workspace growth, a first-time RoPE table, embed_scatter_add beyond 16384 positions, sgemm,
+ * ckpt_*) fail with -1 and end in a failed capture, so run the sequence once eagerly first.  mi355_graph_launch enqueues the replay on the
  * bridge stream; it fails if a workspace was reallocated since the recording (record again).  Accumulating ops
  * (dw +=) accumulate on every replay. */
 typedef struct mi355_graph mi355_graph;

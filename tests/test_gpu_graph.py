@@ -8,6 +8,7 @@ import helpers as H
 pytestmark = pytest.mark.gpu
 
 C_, S, B, HID, HEADS, KVH, HD, V = 256, 64, 2, 512, 4, 2, 32, 1031
+VE = 5                     # embedding rows: few, so that the scatter-add has long segments too
 ALPHA = np.float32(24 ** 0.25)
 
 
@@ -25,7 +26,9 @@ def make(br):
              tgt=br.DevArray.from_numpy(np.random.default_rng(19).integers(0, V, S).astype(np.int32)),
              dl=z(V, S), loss=z(1), scale=z(1), q8=br.DevArray(B * C_ * S, np.int8), deq=z(B, C_, S),
              h16=br.DevArray((B, HEADS * HD, S), np.uint16), fq=z(B, HEADS * HD, S), fk=z(B, KVH * HD, S),
-             fv=z(B, KVH * HD, S), ssq=z(1), clip=z(1), m=z(C_), v=z(C_), scratch=f(20, 4096))
+             fv=z(B, KVH * HD, S), ssq=z(1), clip=z(1), m=z(C_), v=z(C_), scratch=f(20, 4096),
+             E=f(21, VE, C_), ids=br.DevArray.from_numpy(H.zipf_ids(22, B * S, VE).reshape(B, S)), emb=z(B, C_, S),
+             dE=f(23, VE, C_))
     return d
 
 
@@ -33,6 +36,8 @@ def run(br, d, cos, sin):
     """A layer's worth of ops: forward, backward with accumulating weight gradients, loss, INT8, staging, optimizer."""
     L, ck = br.lib, br.check
     n_c, n_h = B * C_ * S, B * HID * S
+    ck(L.mi355_embed_gather_dev(d["emb"].ptr, d["E"].ptr, d["ids"].ptr, VE, C_, S, B))
+    ck(L.mi355_embed_scatter_add_dev(d["dE"].ptr, d["dy"].ptr, d["ids"].ptr, VE, C_, S, B))    # accumulates per run
     ck(L.mi355_rmsnorm_fwd_dev(d["xn"].ptr, d["x"].ptr, d["w1"].ptr, C_, S, B, 1e-5))
     ck(L.mi355_qknorm_rope_fwd_dev(d["qr"].ptr, d["kr"].ptr, d["q"].ptr, d["k"].ptr, d["wq"].ptr, d["wk"].ptr, HEADS, KVH, HD,
                                    S, B, cos, sin, 1e-5))
@@ -104,12 +109,12 @@ def test_graph_capture_refuses_ops_that_allocate(br):
     L = br.lib
     dE = br.DevArray((50, 16)); dx = br.DevArray.from_numpy(H.normal(40, (1, 16, 8)))
     ids = br.DevArray.from_numpy(np.arange(8, dtype=np.int32))
-    br.check(L.mi355_embed_scatter_add_dev(dE.ptr, dx.ptr, ids.ptr, 50, 16, 8, 1))
+    br.check(L.mi355_embed_scatter_add_dev(dE.ptr, dx.ptr, ids.ptr, 1 << 18, 16, 8, 1))   # sizes the workspace
     br.sync()
     a = br.DevArray(64)
     br.check(L.mi355_graph_begin())
     assert L.mi355_graph_begin() == -1
-    assert L.mi355_embed_scatter_add_dev(dE.ptr, dx.ptr, ids.ptr, 50, 16, 8, 1) == -1
+    assert L.mi355_embed_scatter_add_dev(dE.ptr, dx.ptr, ids.ptr, 1 << 18, 16, 8, 1) == -1    # library-sort path
     assert L.mi355_sgemm_dev(0, 0, 4, 4, 4, 1.0, a.ptr, 4, a.ptr, 4, 0.0, a.ptr, 4) == -1
     assert "captured" in br.last_error()
     br.check(L.mi355_axpby_dev(a.ptr, a.ptr, None, 2.0, 64, 1))

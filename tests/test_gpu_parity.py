@@ -354,8 +354,15 @@ def test_embed_gather_bit_exact(br, V, D, B, S, oob):
     (64, 768, 8, 256, 0),         # tiny vocabulary: every segment is long
     (70, 4, 1, 1, 0),
     (40, 130, 2, 100, 1),
-    (3000, 24, 160, 256, 3),      # 40960 positions: beyond the single-launch segment planner
-    (900, 16, 128, 256, 0),       # 32768 positions: its upper limit
+    (3000, 24, 160, 256, 3),      # 40960 positions: the library-sort planner
+    (900, 16, 128, 256, 0),       # 32768 positions
+    (5000, 8, 64, 256, 2),        # 16384 positions: the most the in-LDS planner takes
+    (5000, 8, 1, 16385, 2),       # one more: library sort
+    (300000, 8, 4, 100, 1),       # vocabulary of 2^18 and more: library sort whatever the length
+    (262143, 8, 4, 100, 3),       # the largest vocabulary of the in-LDS planner (out-of-range ids share the top key)
+    (300, 4, 64, 256, 0),         # ~55 positions per token: 300 long segments, more than are ordered by length
+    (9, 36, 1, 255, 0),           # a partial last chunk of the planner
+    (50, 3, 1, 257, 5),
 ])
 def test_embed_scatter_add_bit_exact_and_deterministic(br, V, D, B, S, oob):
     say("scatter_add V=%d D=%d B=%d S=%d" % (V, D, B, S))
@@ -399,9 +406,20 @@ def test_embed_scatter_add_tree_order_is_deterministic_and_close(br):
     if exact is not None:
         assert np.max(np.abs(outs[0] - exact)) <= 1.5 * np.max(np.abs(ref - exact)) + 1e-7
     counts = np.bincount(ids.ravel(), minlength=V)
-    short = counts <= 64
+    short = counts <= 32           # segments of up to 32 rows are summed by one wave, in the reference order
     assert np.array_equal(outs[0][short], ref[short])                 # rows of short segments keep the reference order
     assert not np.array_equal(outs[0][~short], ref[~short])           # the long ones are rounded differently
+
+
+def test_embed_scatter_add_no_valid_id(br):
+    """Every id out of range: nothing is added (ids outside [0,V) are skipped, as the oracle's loop does)."""
+    V, D, B, S = 100, 20, 2, 50
+    ids = np.where(np.arange(B * S).reshape(B, S) % 2 == 0, -1, V).astype(np.int32)
+    dx = H.normal(66, (B, D, S))
+    dE0 = H.normal(67, (V, D))
+    idd, dxd, dEd = dev(br, ids), dev(br, dx), dev(br, dE0)
+    br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, idd.ptr, V, D, S, B))
+    assert dEd.numpy().tobytes() == dE0.tobytes()
 
 
 def test_embed_scatter_add_single_hot_token(br):
