@@ -176,6 +176,18 @@ class Workload:
         elif name == "qknorm_rope_fwd":
             ck(lib.mi355_qknorm_rope_fwd_dev(d["q_rot"].ptr, d["k_rot"].ptr, d["q"].ptr, d["k"].ptr, d["wq"].ptr,
                                              d["wk"].ptr, c["heads"], c["kv_heads"], hd, S, B, self.cos, self.sin, 1e-5))
+        elif name == "qk_unfused_fwd":     # the same op as three launches: per-head RMSNorm of Q, of K, then RoPE in place
+            ck(lib.mi355_rmsnorm_fwd_dev(d["q_rot"].ptr, d["q"].ptr, d["wq"].ptr, hd, S, B * c["heads"], 1e-5))
+            ck(lib.mi355_rmsnorm_fwd_dev(d["k_rot"].ptr, d["k"].ptr, d["wk"].ptr, hd, S, B * c["kv_heads"], 1e-5))
+            ck(lib.mi355_rope_dev(d["q_rot"].ptr, d["k_rot"].ptr, d["q_rot"].ptr, d["k_rot"].ptr, c["heads"],
+                                  c["kv_heads"], hd, S, B, self.cos, self.sin, +1))
+        elif name == "qk_unfused_bwd":     # inverse RoPE of the upstream gradients, then per-head RMSNorm backward
+            ck(lib.mi355_rope_dev(d["q_rot"].ptr, d["k_rot"].ptr, d["gq"].ptr, d["gk"].ptr, c["heads"], c["kv_heads"], hd,
+                                  S, B, self.cos, self.sin, -1))
+            ck(lib.mi355_rmsnorm_bwd_dev(d["dq"].ptr, d["dwq"].ptr, d["q_rot"].ptr, d["q"].ptr, d["wq"].ptr, hd, S,
+                                         B * c["heads"], 1e-5, 0))
+            ck(lib.mi355_rmsnorm_bwd_dev(d["dk"].ptr, d["dwk"].ptr, d["k_rot"].ptr, d["k"].ptr, d["wk"].ptr, hd, S,
+                                         B * c["kv_heads"], 1e-5, 0))
         elif name == "residual1":
             ck(lib.mi355_axpby_dev(d["x2"].ptr, d["x"].ptr, d["o"].ptr, self.alpha, n_c, 0))
         elif name == "res_rms1":       # x2 = x + alpha*o ; x2n = rmsnorm(x2)   (train.m:460-461)
@@ -265,6 +277,14 @@ def per_op_table(br, wl, reps):
     table = []
     if wl.bf16:
         del names["res_rms1"]          # the fused residual + RMSNorm exists for fp32 storage only
+    elif wl.cfg["qk_norm"]:
+        # the fused QK-norm + RoPE again as its unfused composition (three launches, priced at the fused op's bytes);
+        # run last: it overwrites q_rot/k_rot with intermediates
+        names["qk_unfused_fwd"] = "qknorm_rope_fwd (unfused: 3 launches)"
+        names["qk_unfused_bwd"] = "qknorm_rope_bwd (unfused: 3 launches)"
+        ab = dict(ab)
+        ab[names["qk_unfused_fwd"]] = ab["qknorm_rope_fwd"]
+        ab[names["qk_unfused_bwd"]] = ab["qknorm_rope_bwd"]
     for opname, key in names.items():
         def run():
             for d in wl.lay:
@@ -273,6 +293,9 @@ def per_op_table(br, wl, reps):
         run()
         ms = time_region(br, run, reps) / len(wl.lay)
         table.append(dict(op=key, ms=ms, alg_mb=ab[key] / 1e6, gbs=ab[key] / ms / 1e6, frac=ab[key] / ms / 1e6 / PEAK_HBM_GBS))
+    if "qk_unfused_fwd" in names:      # put the fused op's outputs back (the parity check reads them)
+        for d in wl.lay:
+            wl.op("qknorm_rope_fwd", d)
     for key, fn in (("softmax_ce", wl.ce), ("int8_scale", lambda: wl.int8(("scale",))),
                     ("int8_quant", lambda: wl.int8(("quant",))), ("int8_dequant", lambda: wl.int8(("dequant",)))):
         fn()
