@@ -391,7 +391,7 @@ __device__ __forceinline__ void ldtab(float (&r)[VEC], const float *p) {
 // one lane = one interleaved row pair of one head x VEC columns; Q pair rows first, then K
 template <int VEC>
 __global__ __launch_bounds__(BT) void rope_bf16_kernel(bf16_t *q_out, bf16_t *k_out, const bf16_t *q_in,
-                                                       const bf16_t *k_in, int heads, int kv_heads, int hd, int S,
+                                                       const bf16_t *k_in, int heads, int /*kv_heads*/, int hd, int S,
                                                        int batch, const float *__restrict__ cos_t,
                                                        const float *__restrict__ sin_t, float sgn, size_t total) {
     const size_t idx = (size_t)blockIdx.x * BT + threadIdx.x;

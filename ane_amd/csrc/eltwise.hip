@@ -146,7 +146,7 @@ __global__ void axpby_scalar(float *y, const float *a, const float *b, float alp
 // rows: all (batch, head, pair) triples of Q then of K; tables [hd/2][S].
 template <int VEC>
 __global__ __launch_bounds__(EW_THREADS) void rope_kernel(float *q_out, float *k_out, const float *q_in,
-                                                          const float *k_in, int heads, int kv_heads, int hd, int S,
+                                                          const float *k_in, int heads, int /*kv_heads*/, int hd, int S,
                                                           int batch, const float *__restrict__ cos_t,
                                                           const float *__restrict__ sin_t, float sgn, size_t total) {
     const int cols = (S + VEC - 1) / VEC;   // column groups per row

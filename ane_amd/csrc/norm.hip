@@ -247,7 +247,6 @@ __global__ __launch_bounds__(THREADS) void res_rms_fwd_kernel(float *y, float *_
         }
 #pragma unroll
         for (int k = 0; k < CAP; k++) {
-            const int c = row0 + k * RPS;
 #pragma unroll
             for (int j = 0; j < VEC; j++) acc[0][j] += yv[k][j] * yv[k][j];
         }
