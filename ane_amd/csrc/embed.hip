@@ -28,9 +28,10 @@ namespace {
 
 constexpr int TT = 64;   // tokens per tile
 constexpr int TD = 64;   // dims per tile
-constexpr int LONG_SEG = 32;    // segments longer than this take the workgroup path
+constexpr int LONG_SEG = 96;    // segments longer than this take the workgroup path (a wave sums 96 rows in ~14 us)
 constexpr int LCH = 32;             // floats per chunk of a long segment
 constexpr int MAX_ORDERED = 256;    // long segments that the segment-sum workgroups order by length
+constexpr int MAX_MINE = 32;        // long segments a workgroup streams through its stages without a pause
 constexpr int ROWS_PER_WAVE = 16;   // rows a staging wave brings in per stage
 constexpr int STAGE_ROWS = 15 * ROWS_PER_WAVE;    // two buffers of 240 rows x 128 B = 60 KiB of LDS
 
@@ -118,8 +119,7 @@ struct ClampId {
 
 // What the segment sums read: seg_list[i] = {first row, end row, token, 0} of segment i (rows = sorted
 // positions), long_list = the entries of the long segments, meta[0] / meta[1] = the lengths of the two lists,
-// qhead[c] = next entry of the long list that the workgroups of column chunk c have not taken yet (the first
-// long_x entries are taken without asking); rank[position] = its row.
+// rank[position] = its row.
 //
 // Large inputs (more than 16 384 positions, or a vocabulary of 2^18 and more): the library sort, then (1) every
 // workgroup flags the heads among its 1024 sorted entries (key differs from its predecessor), counts them and
@@ -152,16 +152,11 @@ __device__ __forceinline__ int block_excl_scan_1024(int v, int *lds, int &total)
 }
 
 __global__ __launch_bounds__(PLAN_T) void plan_flags_kernel(int *__restrict__ rank, int *__restrict__ blk_count,
-                                                            int *__restrict__ meta, int *__restrict__ qhead,
-                                                            const int *__restrict__ keys,
-                                                            const int *__restrict__ vals, int N, int V, int nq,
-                                                            int long_x) {
+                                                            int *__restrict__ meta, const int *__restrict__ keys,
+                                                            const int *__restrict__ vals, int N, int V) {
     __shared__ int lds[PLAN_T / 64];
     const int i = blockIdx.x * PLAN_T + threadIdx.x;
-    if (blockIdx.x == 0) {
-        if (threadIdx.x == 0) meta[1] = 0;
-        for (int c = threadIdx.x; c < nq; c += PLAN_T) qhead[c] = long_x;
-    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) meta[1] = 0;
     int head = 0;
     if (i < N) {
         const int k = keys[i];
@@ -234,14 +229,10 @@ __device__ __forceinline__ unsigned pack_word(const int32_t *__restrict__ ids, i
 }
 
 __global__ __launch_bounds__(CHUNK) void chunk_sort_kernel(unsigned *__restrict__ sorted_chunks, int *__restrict__ meta,
-                                                           int *__restrict__ qhead, const int32_t *__restrict__ ids,
-                                                           int N, int V, int nq, int long_x) {
+                                                           const int32_t *__restrict__ ids, int N, int V) {
     __shared__ __attribute__((aligned(16))) unsigned sw[CHUNK];
     const int t = threadIdx.x;
-    if (blockIdx.x == 0) {
-        if (t < 2) meta[t] = 0;
-        for (int c = t; c < nq; c += CHUNK) qhead[c] = long_x;
-    }
+    if (blockIdx.x == 0 && t < 2) meta[t] = 0;
     const unsigned w = pack_word(ids, blockIdx.x * CHUNK + t, N, V);
     sw[t] = w;
     __syncthreads();
@@ -423,10 +414,9 @@ __global__ __launch_bounds__(256) void transpose_sorted_kernel(float *__restrict
 
 // Segment sums.  One launch, two kinds of workgroup (1024 threads each):
 //  * the first `long_blocks` workgroups take the LONG segments (more than LONG_SEG rows).  Every one of them
-//    orders the long list by length (longest first, so that the longest chain of dependent adds starts at once
-//    and shares its workgroup with nothing else); workgroup (x, chunk) takes entry x of that order, then
-//    whatever entry the workgroups of its chunk have not taken yet, and sums the entry's 32-float chunk.  Waves 1-15
-//    stage the rows, 240 per stage: two rows per load instruction, eight loads per lane, three stages in
+//    orders the long list by length (longest first, so that the longest chain of dependent adds starts at once);
+//    workgroup (x, chunk) takes one entry per pass over the long_x columns and sums the 32-float chunk of each,
+//    all of them as one stream of stages.  Waves 1-15 stage the rows, 240 per stage: two rows per load instruction, eight loads per lane, three stages in
 //    flight in registers (720 rows, enough to cover the memory latency at the rate the adds consume them), and
 //    write them into one of two LDS buffers.  Wave 0 adds the rows of the other buffer in order, with the LDS
 //    reads of the next 16 rows issued ahead of the adds of the current 16, so the dependent adds run back to
@@ -440,12 +430,12 @@ template <bool TREE>
 __global__ __launch_bounds__(1024, 8) void seg_sum_kernel(float *__restrict__ dE, const float *__restrict__ rows,
                                                        const v4i *__restrict__ seg_list,
                                                        const int *__restrict__ meta, const v4i *__restrict__ long_list,
-                                                       int *__restrict__ qhead, int D, int nchunk, int nchunk_long,
+                                                       int D, int nchunk, int nchunk_long,
                                                        int long_x, int short_blocks, bool vec) {
     __shared__ float stage[2][STAGE_ROWS][LCH];
     __shared__ v4i ent[MAX_ORDERED];
     __shared__ short order[MAX_ORDERED];
-    __shared__ int next_item;
+    __shared__ int it_lo[MAX_MINE], it_hi[MAX_MINE], it_tok[MAX_MINE];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nseg = meta[0];
     const int long_blocks = long_x * nchunk_long;
@@ -476,21 +466,42 @@ __global__ __launch_bounds__(1024, 8) void seg_sum_kernel(float *__restrict__ dE
             order[before] = (short)threadIdx.x;
         }
         __syncthreads();
-        for (int item = x0; item < nlong;) {
-            {
-                const v4i e = nlong <= MAX_ORDERED ? ent[order[item]] : long_list[item];
-                const int lo = __builtin_amdgcn_readfirstlane(e.x), hi = __builtin_amdgcn_readfirstlane(e.y);
-                const int tok = __builtin_amdgcn_readfirstlane(e.z);
-                const int nstage = (hi - lo + STAGE_ROWS - 1) / STAGE_ROWS;
-                // The two roles run separate loops (so that neither carries the other's registers) and meet at
-                // one barrier per stage: barrier s tells wave 0 that buffer s&1 is complete, and tells the staging
-                // waves that wave 0 has finished with the other buffer.
-                if (wave == 0) {
-                    // this wave's chain of dependent adds sets the time of the launch: it goes first whenever it can issue
-                    __builtin_amdgcn_s_setprio(3);
-                    float acc = d_ok ? dE[(size_t)tok * D + d] : 0.f;
-                    for (int s = 0; s < nstage; s++) {
-                        float(*buf)[LCH] = stage[s & 1];
+        // This workgroup's entries of that order: one per pass over the columns, the passes running alternately
+        // up and down the columns so that the column with the longest entry gets the shortest of the next two
+        // passes.  MAX_MINE of them at a time go through the stages back to back, as one stream: the staging waves
+        // run ahead over the boundary between two segments, so a segment of one stage costs one stage.
+        const int full_passes = nlong / long_x, rest = nlong - full_passes * long_x;
+        const int my_off_last = (full_passes & 1) ? long_x - 1 - x0 : x0;
+        const int n_all = full_passes + (my_off_last < rest ? 1 : 0);
+        for (int first = 0; first < n_all; first += MAX_MINE) {
+            const int n_my = min(MAX_MINE, n_all - first);
+            if ((int)threadIdx.x < n_my) {
+                const int m = first + threadIdx.x;
+                const int idx = m * long_x + ((m & 1) ? long_x - 1 - x0 : x0);
+                const v4i e = nlong <= MAX_ORDERED ? ent[order[idx]] : long_list[idx];
+                it_lo[threadIdx.x] = e.x; it_hi[threadIdx.x] = e.y; it_tok[threadIdx.x] = e.z;
+            }
+            __syncthreads();
+            int nstages = 0;
+            for (int k = 0; k < n_my; k++) nstages += (it_hi[k] - it_lo[k] + STAGE_ROWS - 1) / STAGE_ROWS;
+            nstages = __builtin_amdgcn_readfirstlane(nstages);
+            // The two roles run separate loops (so that neither carries the other's registers) and meet at one
+            // barrier per stage: barrier g tells wave 0 that buffer g&1 is complete, and tells the staging waves
+            // that wave 0 has finished with the other buffer.
+            if (wave == 0) {
+                // this wave's chain of dependent adds sets the time of the launch: it goes first whenever it can issue
+                __builtin_amdgcn_s_setprio(3);
+                auto old_value = [&](int k) {           // what dE holds for entry k (0 beyond the last entry)
+                    return (k < n_my && d_ok) ? dE[(size_t)it_tok[k] * D + d] : 0.f;
+                };
+                // the old value of an entry is loaded while the entry before it is summed (a short entry is over before
+                // a load issued at its own start would be back)
+                float acc = old_value(0), acc1 = old_value(1);
+                int g = 0;                                  // stage count over all entries: selects the buffer
+                for (int k = 0; k < n_my; k++) {
+                    const int lo = __builtin_amdgcn_readfirstlane(it_lo[k]), hi = __builtin_amdgcn_readfirstlane(it_hi[k]);
+                    for (int base = lo; base < hi; base += STAGE_ROWS, g++) {
+                        float(*buf)[LCH] = stage[g & 1];
                         __syncthreads();
                         if constexpr (TREE) {
                             float t[30];
@@ -499,7 +510,7 @@ __global__ __launch_bounds__(1024, 8) void seg_sum_kernel(float *__restrict__ dE
 #pragma unroll
                             for (int q = 0; q < 30; q++) acc += t[q];
                         } else {
-                            const int nrow = min(STAGE_ROWS, hi - (lo + s * STAGE_ROWS));
+                            const int nrow = min(STAGE_ROWS, hi - base);
                             if (nrow == STAGE_ROWS) {
                                 float t[2][16];
 #pragma unroll
@@ -528,50 +539,55 @@ __global__ __launch_bounds__(1024, 8) void seg_sum_kernel(float *__restrict__ dE
                             }
                         }
                     }
-                    if (sub == 0 && d_ok) dE[(size_t)tok * D + d] = acc;
-                    __builtin_amdgcn_s_setprio(0);
-                } else {
-                    float g0[8], g1[8], g2[8];
-                    auto fetch = [&](float (&g)[8], int s) {
-                        const int r0 = lo + s * STAGE_ROWS + (wave - 1) * ROWS_PER_WAVE + sub;
+                    // the entry is done: store it, go on with the next one
+                    if (sub == 0 && d_ok) dE[(size_t)it_tok[k] * D + d] = acc;
+                    acc = acc1;
+                    acc1 = old_value(k + 2);
+                }
+                __builtin_amdgcn_s_setprio(0);
+            } else {
+                float g0[8], g1[8], g2[8];
+                int fk = 0, fs = 0;                         // entry and stage of the next fetch
+                auto fetch_next = [&](float (&g)[8]) {
+                    if (fk >= n_my) return;                 // past the last stage: the registers are not used again
+                    const int lo = __builtin_amdgcn_readfirstlane(it_lo[fk]), hi = __builtin_amdgcn_readfirstlane(it_hi[fk]);
+                    const int r0 = lo + fs * STAGE_ROWS + (wave - 1) * ROWS_PER_WAVE + sub;
 #pragma unroll
-                        for (int j = 0; j < 8; j++) {
-                            const int r = r0 + 2 * j;
-                            g[j] = (r < hi && d_ok) ? __builtin_nontemporal_load(rows + (size_t)r * D + d) : -0.0f;
-                        }
-                    };
-                    auto put = [&](float (&g)[8], int s) {
-                        if (s >= nstage) return;
-                        float(*buf)[LCH] = stage[s & 1];
-                        if constexpr (TREE) {
-                            // fixed tree instead of the reference's chain (opt-in, "scatter_tree" knob): every lane
-                            // sums its 8 rows of the stage in order, wave 0 adds the 30 partial rows in order.
-                            // Deterministic, 8x shorter chain, but rounded differently from the CPU loop.
-                            float p = g[0];
-#pragma unroll
-                            for (int j = 1; j < 8; j++) p += g[j];
-                            buf[(wave - 1) * 2 + sub][col] = p;
-                        } else {
-#pragma unroll
-                            for (int j = 0; j < 8; j++) buf[(wave - 1) * ROWS_PER_WAVE + sub + 2 * j][col] = g[j];
-                        }
-                        fetch(g, s + 3);
-                        __syncthreads();
-                    };
-                    fetch(g0, 0);
-                    fetch(g1, 1);
-                    fetch(g2, 2);
-                    for (int s = 0; s < nstage; s += 3) {
-                        put(g0, s);
-                        put(g1, s + 1);
-                        put(g2, s + 2);
+                    for (int j = 0; j < 8; j++) {
+                        const int r = r0 + 2 * j;
+                        g[j] = (r < hi && d_ok) ? __builtin_nontemporal_load(rows + (size_t)r * D + d) : -0.0f;
                     }
+                    fs++;
+                    if (lo + fs * STAGE_ROWS >= hi) { fk++; fs = 0; }
+                };
+                auto put = [&](float (&g)[8], int gi) {
+                    if (gi >= nstages) return;
+                    float(*buf)[LCH] = stage[gi & 1];
+                    if constexpr (TREE) {
+                        // fixed tree instead of the reference's chain (opt-in, "scatter_tree" knob): every lane
+                        // sums its 8 rows of the stage in order, wave 0 adds the 30 partial rows in order.
+                        // Deterministic, 8x shorter chain, but rounded differently from the CPU loop.
+                        float p = g[0];
+#pragma unroll
+                        for (int j = 1; j < 8; j++) p += g[j];
+                        buf[(wave - 1) * 2 + sub][col] = p;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 8; j++) buf[(wave - 1) * ROWS_PER_WAVE + sub + 2 * j][col] = g[j];
+                    }
+                    fetch_next(g);
+                    __syncthreads();
+                };
+                fetch_next(g0);
+                fetch_next(g1);
+                fetch_next(g2);
+                for (int gi = 0; gi < nstages; gi += 3) {
+                    put(g0, gi);
+                    put(g1, gi + 1);
+                    put(g2, gi + 2);
                 }
             }
-            if (threadIdx.x == 0) next_item = atomicAdd(&qhead[ch], 1);
-            __syncthreads();             // also: the next segment's first stage reuses buffer 0
-            item = next_item;
-            __syncthreads();
+            __syncthreads();             // the next round rewrites the table and reuses buffer 0
         }
         return;
     }
@@ -731,8 +747,7 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     const size_t off_seg = 3 * nb, off_cnt = off_seg + al((size_t)(N + 1) * sizeof(int));
     const size_t off_meta = off_cnt + al((size_t)nplan * sizeof(int));
     const size_t off_long = off_meta + 256, off_list = off_long + al((size_t)max_long * sizeof(v4i));
-    const size_t off_q = off_list + al((size_t)N * sizeof(v4i));
-    const size_t off_temp = off_q + al((size_t)nchunk_long * sizeof(int));
+    const size_t off_temp = off_list + al((size_t)N * sizeof(v4i));
     const size_t off_chunks = off_temp + al(temp_bytes);
     const size_t off_rows = off_chunks + al(small ? (size_t)nchunks * CHUNK * sizeof(unsigned) : 0);
     const size_t total = off_rows + al((size_t)N * D * sizeof(float));
@@ -740,22 +755,22 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     if (!ws) return -1;
     int *keys = (int *)(ws + off_keys), *vals = (int *)(ws + off_vals), *rank = (int *)(ws + off_rank);
     int *seg_start = (int *)(ws + off_seg), *blk_count = (int *)(ws + off_cnt);
-    int *meta = (int *)(ws + off_meta), *qhead = (int *)(ws + off_q);
+    int *meta = (int *)(ws + off_meta);
     v4i *long_list = (v4i *)(ws + off_long), *seg_list = (v4i *)(ws + off_list);
     float *rows = (float *)(ws + off_rows);
 
     if (small) {
         unsigned *sorted_chunks = (unsigned *)(ws + off_chunks);
-        hipLaunchKernelGGL(chunk_sort_kernel, dim3(nchunks), dim3(CHUNK), 0, g_ctx.stream, sorted_chunks, meta, qhead, ids,
-                           N, V, nchunk_long, long_x);
+        hipLaunchKernelGGL(chunk_sort_kernel, dim3(nchunks), dim3(CHUNK), 0, g_ctx.stream, sorted_chunks, meta, ids,
+                           N, V);
         hipLaunchKernelGGL(rank_list_kernel, dim3((unsigned)ceil_div((size_t)N, 64)), dim3(1024), 0, g_ctx.stream, rank,
                            seg_list, long_list, meta, sorted_chunks, ids, N, V, nchunks);
     } else {
         e = rocprim::radix_sort_pairs(ws + off_temp, temp_bytes, rocprim::make_transform_iterator(ids, ClampId{V}), keys,
                                       rocprim::counting_iterator<int>(0), vals, (size_t)N, 0, bits, g_ctx.stream);
         if (e != hipSuccess) return mi355_fail("embed_scatter_add: sort: %s", hipGetErrorString(e));
-        hipLaunchKernelGGL(plan_flags_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, rank, blk_count, meta, qhead,
-                           keys, vals, N, V, nchunk_long, long_x);
+        hipLaunchKernelGGL(plan_flags_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, rank, blk_count, meta,
+                           keys, vals, N, V);
         hipLaunchKernelGGL(plan_write_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, seg_start, meta, blk_count,
                            keys, N, V);
         hipLaunchKernelGGL(plan_list_kernel, dim3(nplan), dim3(PLAN_T), 0, g_ctx.stream, seg_list, long_list, meta,
@@ -771,10 +786,10 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     const dim3 sgrid((unsigned)((size_t)long_x * nchunk_long + short_blocks));
     if (g_ctx.scatter_tree)
         hipLaunchKernelGGL(seg_sum_kernel<true>, sgrid, dim3(1024), 0, g_ctx.stream, dE, rows, seg_list, meta,
-                           long_list, qhead, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec);
+                           long_list, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec);
     else
         hipLaunchKernelGGL(seg_sum_kernel<false>, sgrid, dim3(1024), 0, g_ctx.stream, dE, rows, seg_list, meta,
-                           long_list, qhead, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec);
+                           long_list, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec);
     LAUNCH_OK("embed_scatter_add segment sums");
     return 0;
 }

@@ -406,7 +406,7 @@ def test_embed_scatter_add_tree_order_is_deterministic_and_close(br):
     if exact is not None:
         assert np.max(np.abs(outs[0] - exact)) <= 1.5 * np.max(np.abs(ref - exact)) + 1e-7
     counts = np.bincount(ids.ravel(), minlength=V)
-    short = counts <= 32           # segments of up to 32 rows are summed by one wave, in the reference order
+    short = counts <= 96           # segments of up to 96 rows are summed by one wave, in the reference order
     assert np.array_equal(outs[0][short], ref[short])                 # rows of short segments keep the reference order
     assert not np.array_equal(outs[0][~short], ref[~short])           # the long ones are rounded differently
 
