@@ -62,6 +62,40 @@ def test_rmsnorm_fwd_bwd(br, B, Cc, S):
             assert H.rel_err(dwd.numpy(), dw0 + t64dw) <= TOL
 
 
+def test_rmsnorm_columns_of_zeros_tiny_and_huge_values(br):
+    """Columns the reference loop handles without a special case: all zeros (the scale is rsqrt(eps)), values whose
+    squares underflow, and values whose squares overflow fp32 (the mean is inf, the scale 0, the output 0)."""
+    B, Cc, S = 2, 256, 64
+    x = H.normal(4, (B, Cc, S)); w = H.normal(5, Cc, 1.0, 0.02); dy = H.normal(6, (B, Cc, S))
+    x[0, :, 0] = 0.0
+    x[0, :, 1] *= np.float32(1e-25)
+    x[1, :, 2] *= np.float32(1e19)
+    x[1, :, 3] = 0.0; x[1, 7, 3] = 3.0          # one non-zero channel
+    xd, wd, dyd = dev(br, x), dev(br, w), dev(br, dy)
+    yd = br.DevArray(x.shape); dxd = br.DevArray(x.shape); dwd = br.DevArray(Cc)
+    br.check(br.lib.mi355_rmsnorm_fwd_dev(yd.ptr, xd.ptr, wd.ptr, Cc, S, B, 1e-5))
+    y, ry = yd.numpy(), O.rmsnorm(x, w)
+    assert np.isfinite(ry).all() and np.isfinite(y).all()
+    assert np.array_equal(y[0, :, 0], np.zeros(Cc, np.float32)) and np.array_equal(y[1, :, 2], ry[1, :, 2])
+    # column by column: the columns differ by 40 orders of magnitude, so one tensor-wide scale would hide the small ones
+    for b in range(B):
+        for t in range(4):
+            assert H.rel_err(y[b, :, t], ry[b, :, t]) <= TOL, (b, t)
+    assert H.rel_err(y[:, :, 4:], ry[:, :, 4:]) <= TOL
+    br.check(br.lib.mi355_buf_zero(dwd.handle))
+    br.check(br.lib.mi355_rmsnorm_bwd_dev(dxd.ptr, dwd.ptr, dyd.ptr, xd.ptr, wd.ptr, Cc, S, B, 1e-5, 0))
+    rdx, rdw = O.rmsnorm_bwd(dy, x, w, variant=0)
+    dx = dxd.numpy()
+    fin = np.isfinite(rdx)
+    assert np.array_equal(np.isfinite(dx), fin)                 # the overflowing column is inf/nan in both, or in neither
+    for b in range(B):
+        for t in range(S):
+            if fin[b, :, t].all():
+                assert H.rel_err(dx[b, :, t], rdx[b, :, t]) <= TOL, (b, t)
+    if np.isfinite(rdw).all():
+        assert H.rel_err(dwd.numpy(), rdw) <= TOL
+
+
 def test_rmsnorm_golden_reference_recipe(br):
     x, dy, w = GOLD["rms_x"], GOLD["rms_dy"], GOLD["rms_w"]
     Cc, S = x.shape
