@@ -10,7 +10,7 @@
 // Scatter-add: the reference adds dx[:,t] into dE[tok_t] for t ascending, so each (row, d) sum has
 // a fixed order.  To reproduce it bit for bit:
 //   1. the (token, position) pairs are put in token order, positions ascending within a token: for up to
-//      16 384 positions by counting smaller pairs (two small launches, no full sort), beyond that by the
+//      16 384 positions by counting smaller pairs (no full sort; fused with step 2), beyond that by the
 //      rocPRIM stable radix sort;
 //   2. dx is transposed through LDS into token-major rows written in that SORTED order, so a
 //      segment (all positions of one token) is a run of consecutive rows;
@@ -209,13 +209,15 @@ __global__ __launch_bounds__(PLAN_T) void plan_write_kernel(int *__restrict__ se
 // array.  A (token, position) pair is packed into one word, token above position; all words are distinct, and the
 // sorted index of a position is the number of words smaller than its own.
 //   1. chunk_sort_kernel: every 256 consecutive words are sorted by counting, within their workgroup.
-//   2. rank_list_kernel: every workgroup holds all sorted chunks in LDS (64 KiB); 16 lanes share one position
-//      and binary-search four chunks each for (a) the number of smaller words = the sorted index, (b) the largest
+//   2. rank_transpose_kernel: every workgroup (64 positions of one sequence) holds all sorted chunks in LDS
+//      (64 KiB); 16 lanes share one position and binary-search four chunks each for (a) the number of smaller words = the sorted index, (b) the largest
 //      smaller word = the predecessor, which tells whether the position is the first of its token, and (c) the
 //      number of words up to the last one of the same token = the end of the segment.  First positions append
 //      their segment {first row, end row, token} to the segment list, and to the long list if it is long.  The
 //      order of the lists depends on the order of the atomic appends; the sums do not, since a segment is summed
-//      by whoever takes it, from its own rows only.
+//      by whoever takes it, from its own rows only.  The same workgroup then writes its slab of dx token-major at
+//      the rows just found (the transpose of the large path, fused in: the slab's loads are issued before the
+//      searches and land meanwhile).
 constexpr int SMALL_N = 16384, POS_BITS = 14, CHUNK = 256, CHUNK_PITCH = CHUNK + 1;
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
@@ -245,13 +247,39 @@ __global__ __launch_bounds__(CHUNK) void chunk_sort_kernel(unsigned *__restrict_
     sorted_chunks[blockIdx.x * CHUNK + r] = w;
 }
 
-__global__ __launch_bounds__(1024) void rank_list_kernel(int *__restrict__ rank, v4i *__restrict__ seg_list,
-                                                         v4i *__restrict__ long_list, int *__restrict__ meta,
-                                                         const unsigned *__restrict__ sorted_chunks,
-                                                         const int32_t *__restrict__ ids, int N, int V, int nchunks) {
-    __shared__ unsigned sc[(SMALL_N / CHUNK) * CHUNK_PITCH];    // pitch 257: lanes on different chunks, different banks
+__global__ __launch_bounds__(1024) void rank_transpose_kernel(float *__restrict__ rows, v4i *__restrict__ seg_list,
+                                                              v4i *__restrict__ long_list, int *__restrict__ meta,
+                                                              const unsigned *__restrict__ sorted_chunks,
+                                                              const float *__restrict__ dx,
+                                                              const int32_t *__restrict__ ids, int N, int V, int nchunks,
+                                                              int D, int S, int t_tiles) {
+    // the sorted chunks (pitch 257: lanes on different chunks, different banks) and, once the rows are known,
+    // four 64x64 transpose tiles share the same LDS
+    __shared__ union {
+        unsigned sc[(SMALL_N / CHUNK) * CHUNK_PITCH];
+        float tile[4][TD][TT + 1];
+    } sh;
+    __shared__ int dst_row[TT];
     __shared__ int nh, nl, base_h, base_l;
     const int t = threadIdx.x;
+    // this workgroup: 64 positions of one sequence; its slab of dx is independent of the ranks, so the loads of the
+    // first three groups of four tiles (768 columns of D) go out now and land while the ranks are computed
+    const int bt = blockIdx.x;
+    const int b = bt / t_tiles, t0 = (bt - b * t_tiles) * TT;
+    const int tq4 = t >> 8, ltq = t & 15, lr0 = (t & 255) >> 4;        // quarter; lane along t; row group
+    const int tt = t0 + 4 * ltq;
+    const bool vec_ld = (S & 3) == 0 && tt + 3 < S;
+    v4f pre0[4], pre1[4], pre2[4];
+    {
+        auto issue = [&](int g, v4f (&pre)[4]) {
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                const int d = (g * 4 + tq4) * TD + lr0 + 16 * kk;
+                pre[kk] = (vec_ld && d < D) ? ld4_nt(dx + ((size_t)b * D + d) * S + tt) : v4f{0.f, 0.f, 0.f, 0.f};
+            }
+        };
+        issue(0, pre0); issue(1, pre1); issue(2, pre2);
+    }
     {
         v4u q[SMALL_N / 4096];                                  // all loads first, then the LDS writes
 #pragma unroll
@@ -262,13 +290,17 @@ __global__ __launch_bounds__(1024) void rank_list_kernel(int *__restrict__ rank,
 #pragma unroll
         for (int i = 0; i < SMALL_N / 4096; i++) {
             const int j = i * 4096 + t * 4;
-            unsigned *dst = sc + (j / CHUNK) * CHUNK_PITCH + (j % CHUNK);
+            unsigned *dst = sh.sc + (j / CHUNK) * CHUNK_PITCH + (j % CHUNK);
             dst[0] = q[i].x; dst[1] = q[i].y; dst[2] = q[i].z; dst[3] = q[i].w;
         }
     }
-    const int k = t & 15, e = blockIdx.x * 64 + (t >> 4);       // position e, helper lane k of 16
+    // 16 lanes per position
+    const int k = t & 15, tl_mine = t >> 4;
+    const bool live = t0 + tl_mine < S;
+    const int e = live ? b * S + t0 + tl_mine : N;              // N: packs as padding, never written
     const unsigned w = pack_word(ids, e, N, V);
     const unsigned key = w >> POS_BITS;
+    if (t == 0) nh = nl = 0;
     __syncthreads();
     // the four searches of a lane are independent chains of LDS reads and run interleaved; a chunk index past the
     // end is searched as chunk 0 and not counted
@@ -278,7 +310,7 @@ __global__ __launch_bounds__(1024) void rank_list_kernel(int *__restrict__ rank,
 #pragma unroll
     for (int m = 0; m < PER_LANE; m++) {
         okc[m] = k + 16 * m < nchunks;
-        chp[m] = sc + (okc[m] ? k + 16 * m : 0) * CHUNK_PITCH;
+        chp[m] = sh.sc + (okc[m] ? k + 16 * m : 0) * CHUNK_PITCH;
     }
     auto count_below = [&](unsigned x, int (&p)[PER_LANE]) {      // per chunk: number of words < x
 #pragma unroll
@@ -319,26 +351,77 @@ __global__ __launch_bounds__(1024) void rank_list_kernel(int *__restrict__ rank,
 #pragma unroll
         for (int m = 1; m < 16; m <<= 1) upto += __shfl_xor(upto, m, 64);
     }
-    // one append per workgroup and list: the heads take their places within the workgroup through LDS
-    const bool mine = k == 0 && e < N;
+    // one append per workgroup and list: the heads take their places within the workgroup through LDS, and one
+    // 64-bit atomic moves both list lengths (meta[0] is its low word, meta[1] its high word).  The appends of all
+    // workgroups queue up on that address, so nobody waits for the answer before the transpose is done.
+    const bool mine = k == 0 && live;
     const bool head = mine && first;
     const bool is_long = head && upto - below > LONG_SEG;
-    if (t == 0) nh = nl = 0;
-    __syncthreads();
     int ih = 0, il = 0;
     if (head) ih = atomicAdd(&nh, 1);
     if (is_long) il = atomicAdd(&nl, 1);
-    __syncthreads();
-    if (t == 0 && nh) {
-        // both list lengths move with one 64-bit atomic (meta[0] is its low word, meta[1] its high word): the
-        // appends of all workgroups queue up on this one address
-        const unsigned long long old = atomicAdd(reinterpret_cast<unsigned long long *>(meta),
-                                                 ((unsigned long long)(unsigned)nl << 32) | (unsigned)nh);
-        base_h = (int)(old & 0xffffffffu);
-        base_l = (int)(old >> 32);
+    if (k == 0) dst_row[tl_mine] = live ? below : -1;
+    __syncthreads();                                            // also: the chunks in LDS are no longer needed
+    unsigned long long old_len = 0;
+    if (t == 0 && nh)
+        old_len = atomicAdd(reinterpret_cast<unsigned long long *>(meta),
+                            ((unsigned long long)(unsigned)nl << 32) | (unsigned)nh);
+
+    // dx [b][D][t0..t0+63] -> rows[dst_row][D]: each quarter of the workgroup moves one 64x64 tile at a time
+    {
+        const bool d_vec = (D & 3) == 0;
+        float(*tile)[TT + 1] = sh.tile[tq4];
+        auto move_group = [&](int d0, const v4f *pre) {          // pre: this lane's four loads, already issued
+            if (d0 < D) {   // lanes along t
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {
+                    const int dl = lr0 + 16 * kk, d = d0 + dl;
+                    if (d >= D) continue;
+                    const float *src = dx + ((size_t)b * D + d) * S + tt;
+                    if (vec_ld) {
+                        const v4f v = pre ? pre[kk] : ld4_nt(src);
+                        tile[dl][4 * ltq + 0] = v.x; tile[dl][4 * ltq + 1] = v.y;
+                        tile[dl][4 * ltq + 2] = v.z; tile[dl][4 * ltq + 3] = v.w;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+                            if (tt + j < S) tile[dl][4 * ltq + j] = src[j];
+                    }
+                }
+            }
+            __syncthreads();
+            if (d0 < D) {   // lanes along d
+                const int dq = ltq, r0 = lr0;
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) {
+                    const int tl = r0 + 16 * kk;
+                    const int row = dst_row[tl];
+                    if (row < 0) continue;
+                    const int d = d0 + 4 * dq;
+                    float *dst = rows + (size_t)row * D + d;
+                    if (d_vec && d + 3 < D) {
+                        v4f v = {tile[4 * dq][tl], tile[4 * dq + 1][tl], tile[4 * dq + 2][tl], tile[4 * dq + 3][tl]};
+                        st4(dst, v);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+                            if (d + j < D) dst[j] = tile[4 * dq + j][tl];
+                    }
+                }
+            }
+            __syncthreads();
+        };
+        // the groups whose loads went out before the ranks were computed, then the rest (uniform trip counts)
+        if (0 * 4 * TD < D) move_group((0 * 4 + tq4) * TD, pre0);
+        if (1 * 4 * TD < D) move_group((1 * 4 + tq4) * TD, pre1);
+        if (2 * 4 * TD < D) move_group((2 * 4 + tq4) * TD, pre2);
+        for (int g = 3; g * 4 * TD < D; g++) move_group((g * 4 + tq4) * TD, nullptr);
+    }
+    if (t == 0) {
+        base_h = (int)(old_len & 0xffffffffu);
+        base_l = (int)(old_len >> 32);
     }
     __syncthreads();
-    if (mine) rank[e] = below;
     if (head) {
         const v4i entry = {below, upto, (int)key, 0};
         seg_list[base_h + ih] = entry;
@@ -763,8 +846,9 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
         unsigned *sorted_chunks = (unsigned *)(ws + off_chunks);
         hipLaunchKernelGGL(chunk_sort_kernel, dim3(nchunks), dim3(CHUNK), 0, g_ctx.stream, sorted_chunks, meta, ids,
                            N, V);
-        hipLaunchKernelGGL(rank_list_kernel, dim3((unsigned)ceil_div((size_t)N, 64)), dim3(1024), 0, g_ctx.stream, rank,
-                           seg_list, long_list, meta, sorted_chunks, ids, N, V, nchunks);
+        const int t_tiles_s = (int)ceil_div((size_t)S, TT);
+        hipLaunchKernelGGL(rank_transpose_kernel, dim3((unsigned)(batch * t_tiles_s)), dim3(1024), 0, g_ctx.stream, rows,
+                           seg_list, long_list, meta, sorted_chunks, dx, ids, N, V, nchunks, D, S, t_tiles_s);
     } else {
         e = rocprim::radix_sort_pairs(ws + off_temp, temp_bytes, rocprim::make_transform_iterator(ids, ClampId{V}), keys,
                                       rocprim::counting_iterator<int>(0), vals, (size_t)N, 0, bits, g_ctx.stream);
@@ -777,10 +861,12 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
                            seg_start, keys);
     }
     LAUNCH_OK("embed_scatter_add plan");
-    const int t_tiles = (int)ceil_div((size_t)S, TT);
-    const dim3 tgrid((unsigned)(batch * t_tiles), (unsigned)ceil_div((size_t)D, TD));
-    if (tgrid.y > 65535) return mi355_fail("embed_scatter_add: D too large");
-    hipLaunchKernelGGL(transpose_sorted_kernel, tgrid, dim3(256), 0, g_ctx.stream, rows, dx, rank, D, S, t_tiles);
+    if (!small) {
+        const int t_tiles = (int)ceil_div((size_t)S, TT);
+        const dim3 tgrid((unsigned)(batch * t_tiles), (unsigned)ceil_div((size_t)D, TD));
+        if (tgrid.y > 65535) return mi355_fail("embed_scatter_add: D too large");
+        hipLaunchKernelGGL(transpose_sorted_kernel, tgrid, dim3(256), 0, g_ctx.stream, rows, dx, rank, D, S, t_tiles);
+    }
     LAUNCH_OK("embed_scatter_add transpose");
     const size_t short_blocks = std::min<size_t>(ceil_div((size_t)N * nchunk, 16), (size_t)cu);
     const dim3 sgrid((unsigned)((size_t)long_x * nchunk_long + short_blocks));
