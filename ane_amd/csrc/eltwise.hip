@@ -236,6 +236,59 @@ __global__ __launch_bounds__(1024) void scale_from_partials_kernel(float *scale,
     }
 }
 
+// min, max and max|x| over the tensor (the loop's range diagnostics, vDSP_minv / vDSP_maxv / vDSP_maxmgv at
+// training/training_dynamic/train.m:664-666,738-742): per-workgroup triples, then one workgroup folds them.
+// All three are exact whatever the order; NaNs are skipped (fminf/fmaxf).
+__global__ __launch_bounds__(EW_THREADS) void minmax_kernel(float *__restrict__ part, const float *__restrict__ x,
+                                                            size_t n, size_t n4, bool vec) {
+    __shared__ float red[3][EW_THREADS / 64];
+    float lo = INFINITY, hi = -INFINITY;
+    const size_t stride = (size_t)gridDim.x * EW_THREADS;
+    const size_t tid = (size_t)blockIdx.x * EW_THREADS + threadIdx.x;
+    if (vec) {
+        for (size_t i = tid; i < n4; i += stride) {
+            v4f v = ld4_nt(x + 4 * i);
+#pragma unroll
+            for (int j = 0; j < 4; j++) { lo = fminf(lo, v[j]); hi = fmaxf(hi, v[j]); }
+        }
+        if (blockIdx.x == 0)
+            for (size_t i = n4 * 4 + threadIdx.x; i < n; i += EW_THREADS) { lo = fminf(lo, x[i]); hi = fmaxf(hi, x[i]); }
+    } else {
+        for (size_t i = tid; i < n; i += stride) { lo = fminf(lo, x[i]); hi = fmaxf(hi, x[i]); }
+    }
+#pragma unroll
+    for (int k = 1; k < 64; k <<= 1) {
+        lo = fminf(lo, __shfl_xor(lo, k, 64));
+        hi = fmaxf(hi, __shfl_xor(hi, k, 64));
+    }
+    if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = lo; red[1][threadIdx.x >> 6] = hi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 1; k < EW_THREADS / 64; k++) { lo = fminf(lo, red[0][k]); hi = fmaxf(hi, red[1][k]); }
+        part[2 * blockIdx.x] = lo;
+        part[2 * blockIdx.x + 1] = hi;
+    }
+}
+
+__global__ __launch_bounds__(1024) void minmax_final_kernel(float *out, const float *__restrict__ part, int nblk) {
+    __shared__ float red[2][16];
+    float lo = INFINITY, hi = -INFINITY;
+    for (int i = threadIdx.x; i < nblk; i += 1024) { lo = fminf(lo, part[2 * i]); hi = fmaxf(hi, part[2 * i + 1]); }
+#pragma unroll
+    for (int k = 1; k < 64; k <<= 1) {
+        lo = fminf(lo, __shfl_xor(lo, k, 64));
+        hi = fmaxf(hi, __shfl_xor(hi, k, 64));
+    }
+    if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = lo; red[1][threadIdx.x >> 6] = hi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 1; k < 16; k++) { lo = fminf(lo, red[0][k]); hi = fmaxf(hi, red[1][k]); }
+        out[0] = lo;
+        out[1] = hi;
+        out[2] = fmaxf(fabsf(lo), fabsf(hi));       // max |x| is |min| or |max|
+    }
+}
+
 __device__ __forceinline__ int quant1(float x, float scale, int rounding) {
     float v = x / scale;              // IEEE division, as the reference (bridge/ane_bridge.m:361)
     v = fminf(v, 127.0f);
@@ -528,6 +581,23 @@ MI355_API int mi355_rope_dev(float *q_out, float *k_out, const float *q_in, cons
                            (float)dir, total);
     }
     LAUNCH_OK("rope");
+    return 0;
+}
+
+// ---- range diagnostics ----
+MI355_API int mi355_minmax_dev(float *out3_dev, const float *x, size_t n) {
+    if (!mi355_ready("minmax")) return -1;
+    if (!out3_dev || !x) return mi355_fail("minmax: NULL pointer");
+    if (n == 0) return mi355_fail("minmax: empty tensor");
+    const bool vec = aligned16(x);
+    const size_t n4 = vec ? n / 4 : 0;
+    size_t blocks = ceil_div(vec ? (n4 ? n4 : 1) : n, (size_t)EW_THREADS);
+    if (blocks > 4096) blocks = 4096;
+    float *part = (float *)mi355_ws(2 * blocks * sizeof(float));
+    if (!part) return -1;
+    hipLaunchKernelGGL(minmax_kernel, dim3((unsigned)blocks), dim3(EW_THREADS), 0, g_ctx.stream, part, x, n, n4, vec);
+    hipLaunchKernelGGL(minmax_final_kernel, dim3(1), dim3(1024), 0, g_ctx.stream, out3_dev, part, (int)blocks);
+    LAUNCH_OK("minmax");
     return 0;
 }
 

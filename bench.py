@@ -582,6 +582,8 @@ def bench_aux(br, args):
         kb + qb, nset)
     add("gqa_reduce", lambda: [br.check(br.lib.mi355_gqa_reduce_dev(k.ptr, q.ptr, kvh, ratio, hd, S, B)) for q, k in zip(qs, ks)],
         kb + qb, nset)
+    mm = A(3)      # range diagnostics of dq (training/training_dynamic/train.m:664): one read of the tensor
+    add("minmax", lambda: [br.check(br.lib.mi355_minmax_dev(mm.ptr, q.ptr, q.size)) for q in qs], qb, nset)
     rb = CV * D * 4
     add("vocab_compact_embed", lambda: [br.check(br.lib.mi355_vocab_compact_embed_dev(x.ptr, full.ptr, cmapd.ptr, CV, V, D)) for x in comp],
         2 * rb, len(comp))

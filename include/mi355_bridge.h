@@ -232,6 +232,11 @@ int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, 
 int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float *logits,
                          const int32_t *targets, int V, int S, float grad_scale);
 
+/* Range diagnostics of the loops: out3_dev = {min x, max x, max |x|}.  Replaces vDSP_minv / vDSP_maxv /
+ * vDSP_maxmgv — training/training_dynamic/train.m:664-666 (dq, dk, dv magnitudes) and :738-742 (range of x and
+ * dy).  Exact in any order; NaNs are skipped. */
+int mi355_minmax_dev(float *out3_dev, const float *x, size_t n);
+
 /* Per-tensor symmetric INT8.  Replaces the quantizer of ane_bridge_build_weight_blob_quantized —
  * bridge/ane_bridge.m:346-365 — and the MIL quantize/dequantize pair of ane_int8_bench.m:83-92.
  * scale = max|x|/127 (1.0 when the tensor is all zero); q = clamp(x/scale, -128, 127) rounded

@@ -51,6 +51,7 @@ def _load():
         "orc_embed_lookup": (C.c_int, [_f32p, _f32p, _i32p, C.c_int, C.c_int, C.c_int]),
         "orc_embed_backward": (None, [_f32p, _f32p, _i32p, C.c_int, C.c_int, C.c_int]),
         "orc_cross_entropy": (C.c_float, [_f32p, _f32p, _i32p, C.c_int, C.c_int, C.c_float]),
+        "orc_minmax": (None, [_f32p, _f32p, C.c_size_t]),
         "orc_int8_scale": (C.c_float, [_f32p, C.c_size_t]),
         "orc_int8_quant": (None, [_i8p, _f32p, C.c_size_t, C.c_float, C.c_int]),
         "orc_int8_dequant": (None, [_f32p, _i8p, C.c_size_t, C.c_float]),
@@ -208,6 +209,14 @@ def cross_entropy(logits, targets, grad_scale=1.0):
     dl = np.empty_like(logits)
     loss = lib.orc_cross_entropy(dl, logits, targets, V, S, grad_scale)
     return float(loss), dl
+
+
+def minmax(x):
+    """(min, max, max|x|) of a tensor — train.m:664-666,738-742."""
+    x = _f32(x)
+    out = np.empty(3, np.float32)
+    lib.orc_minmax(out, x.reshape(-1), x.size)
+    return out
 
 
 def int8_scale(x):

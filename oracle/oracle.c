@@ -349,6 +349,18 @@ ORC_API float orc_cross_entropy(float *dlogits, const float *logits, const int32
     return total / (float)S;
 }
 
+/* Range diagnostics — training/training_dynamic/train.m:664-666 (vDSP_maxmgv) and :738-742 (vDSP_maxv,
+ * vDSP_minv): out = {min, max, max |x|}.  NaNs are skipped. */
+ORC_API void orc_minmax(float *out3, const float *x, size_t n) {
+    float lo = INFINITY, hi = -INFINITY, mg = 0.f;
+    for (size_t i = 0; i < n; i++) {
+        lo = fminf(lo, x[i]);
+        hi = fmaxf(hi, x[i]);
+        mg = fmaxf(mg, fabsf(x[i]));
+    }
+    out3[0] = lo; out3[1] = hi; out3[2] = mg;
+}
+
 /* ---------------------------------------------------------------------------------------------
  * Per-tensor symmetric INT8 — bridge/ane_bridge.m:346-365: scale = max|x|/127 (0 -> 1),
  * v = x/scale clamped to [-128,127]; rounding 1 = half away from zero (the reference's

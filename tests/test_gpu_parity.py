@@ -466,6 +466,21 @@ def test_embed_scatter_add_single_hot_token(br):
     assert dEd.numpy().tobytes() == O.embed_backward(dE0, dx, ids).tobytes()
 
 
+@pytest.mark.parametrize("n", [1024 * 4096, 2048 * 256 * 16, 13, 1, 4099])
+def test_minmax_exact(br, n):
+    say("minmax n=%d" % n)
+    x = H.normal(71, n) * np.float32(2.0)
+    if n > 100:
+        x[n // 3] = np.float32(-77.0); x[n // 2] = np.float32(55.5); x[7] = np.nan
+    xd = dev(br, x); od = br.DevArray(3)
+    br.check(br.lib.mi355_minmax_dev(od.ptr, xd.ptr, n))
+    assert od.numpy().tobytes() == O.minmax(x).tobytes()
+    if n > 4:       # an address that is not 16-byte aligned takes the scalar path
+        off = dev(br, np.concatenate([np.array([1e9], np.float32), x]))
+        br.check(br.lib.mi355_minmax_dev(od.ptr, off.ptr + 4, n))
+        assert od.numpy().tobytes() == O.minmax(x).tobytes()
+
+
 # ---------------------------------------------------------------------------------------------
 # softmax + cross-entropy
 # ---------------------------------------------------------------------------------------------

@@ -421,3 +421,14 @@ def test_int8_golden_ties_and_bounds():
     assert np.array_equal(O.int8_quant(np.array([1e6, -1e6], np.float32), 1.0, 0), np.array([127, -128], np.int8))
     q = O.int8_quant(y, s, 0)
     assert np.array_equal(q, np.clip(np.rint(y / np.float32(s)), -128, 127).astype(np.int8))
+
+
+def test_minmax_matches_numpy_and_skips_nan():
+    """orc_minmax (the loop's vDSP_minv / vDSP_maxv / vDSP_maxmgv diagnostics) against numpy's reductions."""
+    x = H.normal(70, 10007) * np.float32(3.0)
+    lo, hi, mg = O.minmax(x)
+    assert lo == x.min() and hi == x.max() and mg == np.abs(x).max()
+    assert tuple(O.minmax(np.array([-2.5], np.float32))) == (-2.5, -2.5, 2.5)
+    y = x.copy(); y[5] = np.nan; y[100] = -50.0
+    lo, hi, mg = O.minmax(y)
+    assert lo == -50.0 and hi == np.nanmax(y) and mg == 50.0
