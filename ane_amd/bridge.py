@@ -89,6 +89,8 @@ SIGNATURES = {
     "mi355_adam_update_dev": (_i, [_p, _p, _p, _p, _z, _i, _f, _f, _f, _f, _f, _f, _p, _i]),
     "mi355_sumsq_accum_multi_dev": (_i, [_p, _p, _p, _i, _f]),
     "mi355_adam_update_multi_dev": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _f, _f, _f, _f, _f, _p, _i]),
+    "mi355_vocab_map_build_dev": (_i, [_p, _p, _p, _p, _z, _i]),
+    "mi355_vocab_remap_dev": (_i, [_p, _p, _p, _z, _i]),
     "mi355_vocab_compact_embed_dev": (_i, [_p, _p, _p, _i, _i, _i]),
     "mi355_vocab_update_full_dev": (_i, [_p, _p, _p, _i, _i, _i]),
     "mi355_vocab_scatter_grads_dev": (_i, [_p, _p, _p, _i, _i, _i]),

@@ -752,6 +752,45 @@ __global__ __launch_bounds__(256) void rows_by_index_kernel(float *__restrict__ 
     }
 }
 
+// Vocabulary map (training/training_dynamic/cpu_ops.h:102-126): mark the tokens that occur in the data, number
+// the marked ones in ascending token order.
+__global__ __launch_bounds__(256) void vocab_fill_kernel(int *__restrict__ f2c, int V) {
+    const int v = blockIdx.x * 256 + threadIdx.x;
+    if (v < V) f2c[v] = -1;
+}
+__global__ __launch_bounds__(256) void vocab_mark_kernel(int *__restrict__ f2c, const uint16_t *__restrict__ data,
+                                                         size_t n, int V) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+        const int tok = data[i];
+        if (tok < V) f2c[tok] = 0;                 // every writer stores the same value
+    }
+}
+// one workgroup walks the vocabulary 1024 tokens at a time (a one-time step of the loops' start-up)
+__global__ __launch_bounds__(PLAN_T) void vocab_number_kernel(int *__restrict__ f2c, int *__restrict__ c2f,
+                                                              int *__restrict__ cv_out, int V) {
+    __shared__ int lds[PLAN_T / 64];
+    int base = 0;
+    for (int v0 = 0; v0 < V; v0 += PLAN_T) {
+        const int v = v0 + threadIdx.x;
+        const int used = (v < V && f2c[v] == 0) ? 1 : 0;
+        int total;
+        const int ex = block_excl_scan_1024(used, lds, total);
+        if (v < V) f2c[v] = used ? base + ex : -1;
+        if (used) c2f[base + ex] = v;
+        base += total;
+    }
+    if (threadIdx.x == 0) *cv_out = base;
+}
+// ids of the full vocabulary -> ids of the compact one (train.m:403); an id outside [0,V) or unused becomes -1
+__global__ __launch_bounds__(256) void vocab_remap_kernel(int32_t *__restrict__ out, const int32_t *__restrict__ ids,
+                                                          const int *__restrict__ f2c, size_t n, int V) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int id = ids[i];
+    out[i] = (id >= 0 && id < V) ? f2c[id] : -1;
+}
+
 template <int MODE>
 int rows_by_index(const char *who, float *dst, const float *src, const int32_t *idx, int n, int D, int rows_dst,
                   int rows_src) {
@@ -877,6 +916,35 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
         hipLaunchKernelGGL(seg_sum_kernel<false>, sgrid, dim3(1024), 0, g_ctx.stream, dE, rows, seg_list, meta,
                            long_list, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec);
     LAUNCH_OK("embed_scatter_add segment sums");
+    return 0;
+}
+
+MI355_API int mi355_vocab_map_build_dev(int32_t *full_to_compact, int32_t *compact_to_full, int32_t *compact_vocab_dev,
+                                        const uint16_t *data, size_t n_tokens, int V) {
+    if (!mi355_ready("vocab_map_build")) return -1;
+    if (!full_to_compact || !compact_to_full || !compact_vocab_dev || (!data && n_tokens))
+        return mi355_fail("vocab_map_build: NULL pointer");
+    if (V <= 0) return mi355_fail("vocab_map_build: bad vocabulary size %d", V);
+    hipLaunchKernelGGL(vocab_fill_kernel, dim3((unsigned)ceil_div((size_t)V, 256)), dim3(256), 0, g_ctx.stream,
+                       full_to_compact, V);
+    if (n_tokens) {
+        const size_t blocks = std::min<size_t>(ceil_div(n_tokens, 256), 4096);
+        hipLaunchKernelGGL(vocab_mark_kernel, dim3((unsigned)blocks), dim3(256), 0, g_ctx.stream, full_to_compact, data,
+                           n_tokens, V);
+    }
+    hipLaunchKernelGGL(vocab_number_kernel, dim3(1), dim3(PLAN_T), 0, g_ctx.stream, full_to_compact, compact_to_full,
+                       compact_vocab_dev, V);
+    LAUNCH_OK("vocab_map_build");
+    return 0;
+}
+
+MI355_API int mi355_vocab_remap_dev(int32_t *out, const int32_t *ids, const int32_t *full_to_compact, size_t n, int V) {
+    if (!mi355_ready("vocab_remap")) return -1;
+    if (!out || !ids || !full_to_compact) return mi355_fail("vocab_remap: NULL pointer");
+    if (n == 0 || V <= 0) return mi355_fail("vocab_remap: bad size");
+    hipLaunchKernelGGL(vocab_remap_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, g_ctx.stream, out, ids,
+                       full_to_compact, n, V);
+    LAUNCH_OK("vocab_remap");
     return 0;
 }
 

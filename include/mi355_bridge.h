@@ -335,8 +335,18 @@ int mi355_ckpt_create(const char *path, const mi355_ckpt_hdr *hdr);
 int mi355_ckpt_load_dev(const char *path, uint64_t byte_offset, float *dst_dev, uint64_t count);
 int mi355_ckpt_store_dev(const char *path, uint64_t byte_offset, const float *src_dev, uint64_t count);
 
+/* Vocabulary map.  Replaces vocab_map_build — training/training_dynamic/cpu_ops.h:102-126: full_to_compact[V]
+ * gets the compact id of every token that occurs in data[0..n_tokens) (numbered in ascending token order) and
+ * -1 for the others; compact_to_full (room for V entries) gets the inverse; *compact_vocab_dev their number.
+ * Tokens >= V in the data are ignored.  mi355_vocab_remap_dev maps ids of the full vocabulary to compact ids
+ * (the loop at training/training_dynamic/train.m:403); an id outside [0,V) or without a compact id gives -1. */
+int mi355_vocab_map_build_dev(int32_t *full_to_compact, int32_t *compact_to_full, int32_t *compact_vocab_dev,
+                              const uint16_t *data, size_t n_tokens, int V);
+int mi355_vocab_remap_dev(int32_t *out, const int32_t *ids, const int32_t *full_to_compact, size_t n, int V);
+
 /* Vocabulary compaction — training/training_dynamic/cpu_ops.h:127-148.  compact_to_full[CV] is the map that
- * vocab_map_build (cpu_ops.h:103-125, host code, unchanged) produces: distinct row numbers of the full table.
+ * vocab_map_build (cpu_ops.h:103-125; above, or the host code unchanged) produces: distinct row numbers of the
+ * full table.
  *   compact_embed: compact[c] = full[map[c]]           (vocab_compact_embed, cpu_ops.h:127-132)
  *   update_full:   full[map[c]] = compact[c]           (vocab_update_full,   cpu_ops.h:145-148)
  *   scatter_grads: full_grad[map[c]] += compact_grad[c] (vocab_scatter_grads, cpu_ops.h:135-142)

@@ -674,6 +674,25 @@ def test_vocab_compaction_bit_exact(br, V, D, ntok):
     assert Ed.numpy().tobytes() == O.vocab_update_full(E, new, c2f).tobytes()
 
 
+@pytest.mark.parametrize("V,ntok", [(32000, 200000), (300, 500), (1000, 64), (5, 1000), (151936, 16384), (1031, 1)])
+def test_vocab_map_build_and_remap_exact(br, V, ntok):
+    """The map of training/training_dynamic/cpu_ops.h:102-126 built on the device, and the id remap of train.m:403."""
+    data = H.zipf_ids(49, ntok, min(V, 65536)).astype(np.uint16)
+    f2c, c2f = O.vocab_map_build(data, V)
+    dd = br.DevArray.from_numpy(data)
+    f2cd = br.DevArray(V, np.int32); c2fd = br.DevArray(V, np.int32); cvd = br.DevArray(1, np.int32)
+    br.check(br.lib.mi355_vocab_map_build_dev(f2cd.ptr, c2fd.ptr, cvd.ptr, dd.ptr, ntok, V))
+    cv = int(cvd.numpy()[0])
+    assert cv == c2f.size
+    assert np.array_equal(f2cd.numpy(), f2c) and np.array_equal(c2fd.numpy()[:cv], c2f)
+    ids = np.concatenate([data.astype(np.int32), np.array([-1, V, V + 7, 0, V - 1], np.int32)])
+    want = np.where((ids >= 0) & (ids < V), f2c[np.clip(ids, 0, V - 1)], -1).astype(np.int32)
+    idd = br.DevArray.from_numpy(ids); od = br.DevArray(ids.size, np.int32)
+    br.check(br.lib.mi355_vocab_remap_dev(od.ptr, idd.ptr, f2cd.ptr, ids.size, V))
+    assert np.array_equal(od.numpy(), want)
+    assert (od.numpy()[:ntok] >= 0).all()                      # every token of the data has a compact id
+
+
 @pytest.mark.parametrize("B,kvh,ratio,hd,S", [(16, 8, 2, 128, 256), (2, 3, 4, 6, 5), (1, 1, 1, 4, 4)])
 def test_gqa_tile_reduce(br, B, kvh, ratio, hd, S):
     k = H.normal(54, (B, kvh * hd, S)); g = H.normal(55, (B, kvh * ratio * hd, S))
