@@ -209,7 +209,7 @@ __global__ __launch_bounds__(PLAN_T) void plan_write_kernel(int *__restrict__ se
 // array.  A (token, position) pair is packed into one word, token above position; all words are distinct, and the
 // sorted index of a position is the number of words smaller than its own.
 //   1. chunk_sort_kernel: every 256 consecutive words are sorted by counting, within their workgroup.
-//   2. rank_transpose_kernel: every workgroup (64 positions of one sequence) holds all sorted chunks in LDS
+//   2. rank_transpose_kernel: every workgroup (64 consecutive positions) holds all sorted chunks in LDS
 //      (64 KiB); 16 lanes share one position and binary-search four chunks each for (a) the number of smaller words = the sorted index, (b) the largest
 //      smaller word = the predecessor, which tells whether the position is the first of its token, and (c) the
 //      number of words up to the last one of the same token = the end of the segment.  First positions append
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(1024) void rank_transpose_kernel(float *__restrict_
                                                               const unsigned *__restrict__ sorted_chunks,
                                                               const float *__restrict__ dx,
                                                               const int32_t *__restrict__ ids, int N, int V, int nchunks,
-                                                              int D, int S, int t_tiles) {
+                                                              int D, int S) {
     // the sorted chunks (pitch 257: lanes on different chunks, different banks) and, once the rows are known,
     // four 64x64 transpose tiles share the same LDS
     __shared__ union {
@@ -262,20 +262,22 @@ __global__ __launch_bounds__(1024) void rank_transpose_kernel(float *__restrict_
     __shared__ int dst_row[TT];
     __shared__ int nh, nl, base_h, base_l;
     const int t = threadIdx.x;
-    // this workgroup: 64 positions of one sequence; its slab of dx is independent of the ranks, so the loads of the
-    // first three groups of four tiles (768 columns of D) go out now and land while the ranks are computed
-    const int bt = blockIdx.x;
-    const int b = bt / t_tiles, t0 = (bt - b * t_tiles) * TT;
-    const int tq4 = t >> 8, ltq = t & 15, lr0 = (t & 255) >> 4;        // quarter; lane along t; row group
-    const int tt = t0 + 4 * ltq;
-    const bool vec_ld = (S & 3) == 0 && tt + 3 < S;
+    // this workgroup: 64 consecutive positions (of one or several sequences); their columns of dx are independent of
+    // the ranks, so the loads of the first three groups of four tiles (768 columns of D) go out now and land while
+    // the ranks are computed.  A lane moves four consecutive positions; with S a multiple of 4 they lie in one
+    // sequence and are one 128-bit load.
+    const int n0 = blockIdx.x * TT;
+    const int tq4 = t >> 8, ltq = t & 15, lr0 = (t & 255) >> 4;        // quarter; lane along positions; row group
+    const int n4 = n0 + 4 * ltq;
+    const bool vec_ld = (S & 3) == 0 && n4 + 3 < N;
+    const int b4 = n4 / S, t4 = n4 - b4 * S;
     v4f pre0[4], pre1[4], pre2[4];
     {
         auto issue = [&](int g, v4f (&pre)[4]) {
 #pragma unroll
             for (int kk = 0; kk < 4; kk++) {
                 const int d = (g * 4 + tq4) * TD + lr0 + 16 * kk;
-                pre[kk] = (vec_ld && d < D) ? ld4_nt(dx + ((size_t)b * D + d) * S + tt) : v4f{0.f, 0.f, 0.f, 0.f};
+                pre[kk] = (vec_ld && d < D) ? ld4_nt(dx + ((size_t)b4 * D + d) * S + t4) : v4f{0.f, 0.f, 0.f, 0.f};
             }
         };
         issue(0, pre0); issue(1, pre1); issue(2, pre2);
@@ -296,8 +298,8 @@ __global__ __launch_bounds__(1024) void rank_transpose_kernel(float *__restrict_
     }
     // 16 lanes per position
     const int k = t & 15, tl_mine = t >> 4;
-    const bool live = t0 + tl_mine < S;
-    const int e = live ? b * S + t0 + tl_mine : N;              // N: packs as padding, never written
+    const int e = min(n0 + tl_mine, N);                         // N: packs as padding, never written
+    const bool live = e < N;
     const unsigned w = pack_word(ids, e, N, V);
     const unsigned key = w >> POS_BITS;
     if (t == 0) nh = nl = 0;
@@ -372,20 +374,24 @@ __global__ __launch_bounds__(1024) void rank_transpose_kernel(float *__restrict_
         const bool d_vec = (D & 3) == 0;
         float(*tile)[TT + 1] = sh.tile[tq4];
         auto move_group = [&](int d0, const v4f *pre) {          // pre: this lane's four loads, already issued
-            if (d0 < D) {   // lanes along t
+            if (d0 < D) {   // lanes along positions
 #pragma unroll
                 for (int kk = 0; kk < 4; kk++) {
                     const int dl = lr0 + 16 * kk, d = d0 + dl;
                     if (d >= D) continue;
-                    const float *src = dx + ((size_t)b * D + d) * S + tt;
                     if (vec_ld) {
-                        const v4f v = pre ? pre[kk] : ld4_nt(src);
+                        const v4f v = pre ? pre[kk] : ld4_nt(dx + ((size_t)b4 * D + d) * S + t4);
                         tile[dl][4 * ltq + 0] = v.x; tile[dl][4 * ltq + 1] = v.y;
                         tile[dl][4 * ltq + 2] = v.z; tile[dl][4 * ltq + 3] = v.w;
                     } else {
 #pragma unroll
-                        for (int j = 0; j < 4; j++)
-                            if (tt + j < S) tile[dl][4 * ltq + j] = src[j];
+                        for (int j = 0; j < 4; j++) {
+                            const int n = n4 + j;
+                            if (n < N) {
+                                const int bb = n / S;
+                                tile[dl][4 * ltq + j] = dx[((size_t)bb * D + d) * S + (n - bb * S)];
+                            }
+                        }
                     }
                 }
             }
@@ -885,9 +891,8 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
         unsigned *sorted_chunks = (unsigned *)(ws + off_chunks);
         hipLaunchKernelGGL(chunk_sort_kernel, dim3(nchunks), dim3(CHUNK), 0, g_ctx.stream, sorted_chunks, meta, ids,
                            N, V);
-        const int t_tiles_s = (int)ceil_div((size_t)S, TT);
-        hipLaunchKernelGGL(rank_transpose_kernel, dim3((unsigned)(batch * t_tiles_s)), dim3(1024), 0, g_ctx.stream, rows,
-                           seg_list, long_list, meta, sorted_chunks, dx, ids, N, V, nchunks, D, S, t_tiles_s);
+        hipLaunchKernelGGL(rank_transpose_kernel, dim3((unsigned)ceil_div((size_t)N, TT)), dim3(1024), 0, g_ctx.stream, rows,
+                           seg_list, long_list, meta, sorted_chunks, dx, ids, N, V, nchunks, D, S);
     } else {
         e = rocprim::radix_sort_pairs(ws + off_temp, temp_bytes, rocprim::make_transform_iterator(ids, ClampId{V}), keys,
                                       rocprim::counting_iterator<int>(0), vals, (size_t)N, 0, bits, g_ctx.stream);

@@ -396,6 +396,8 @@ def test_embed_gather_bit_exact(br, V, D, B, S, oob):
     (262143, 8, 4, 100, 3),       # the largest vocabulary of the in-LDS planner (out-of-range ids share the top key)
     (300, 4, 64, 256, 0),         # ~55 positions per token: 300 long segments, more than are ordered by length
     (9, 36, 1, 255, 0),           # a partial last chunk of the planner
+    (1000, 32, 2048, 8, 3),       # many short sequences: a block of 64 positions spans eight of them
+    (1000, 20, 700, 6, 2),        # ... with S not a multiple of 4
     (50, 3, 1, 257, 5),
 ])
 def test_embed_scatter_add_bit_exact_and_deterministic(br, V, D, B, S, oob):
