@@ -867,18 +867,22 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
         if (e != hipSuccess) return mi355_fail("embed_scatter_add: sort sizing: %s", hipGetErrorString(e));
     }
 
-    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
-    const size_t nb = al((size_t)N * sizeof(int));
+    // one workspace, carved in 256-byte steps; the sort's arrays only where the library sort runs
     const int nplan = (int)ceil_div((size_t)N, PLAN_T);
     const int nchunks = (int)ceil_div((size_t)N, CHUNK);
-    const size_t off_keys = 0, off_vals = nb, off_rank = 2 * nb;
-    const size_t off_seg = 3 * nb, off_cnt = off_seg + al((size_t)(N + 1) * sizeof(int));
-    const size_t off_meta = off_cnt + al((size_t)nplan * sizeof(int));
-    const size_t off_long = off_meta + 256, off_list = off_long + al((size_t)max_long * sizeof(v4i));
-    const size_t off_temp = off_list + al((size_t)N * sizeof(v4i));
-    const size_t off_chunks = off_temp + al(temp_bytes);
-    const size_t off_rows = off_chunks + al(small ? (size_t)nchunks * CHUNK * sizeof(unsigned) : 0);
-    const size_t total = off_rows + al((size_t)N * D * sizeof(float));
+    size_t total = 0;
+    auto take = [&total](size_t bytes) {
+        const size_t off = total;
+        total += (bytes + 255) & ~(size_t)255;
+        return off;
+    };
+    const size_t big = small ? 0 : 1;
+    const size_t off_keys = take(big * N * sizeof(int)), off_vals = take(big * N * sizeof(int));
+    const size_t off_rank = take(big * N * sizeof(int)), off_seg = take(big * ((size_t)N + 1) * sizeof(int));
+    const size_t off_cnt = take(big * nplan * sizeof(int)), off_temp = take(temp_bytes);
+    const size_t off_chunks = take(small ? (size_t)nchunks * CHUNK * sizeof(unsigned) : 0);
+    const size_t off_meta = take(256), off_long = take((size_t)max_long * sizeof(v4i));
+    const size_t off_list = take((size_t)N * sizeof(v4i)), off_rows = take((size_t)N * D * sizeof(float));
     char *ws = (char *)mi355_ws(total);
     if (!ws) return -1;
     int *keys = (int *)(ws + off_keys), *vals = (int *)(ws + off_vals), *rank = (int *)(ws + off_rank);
