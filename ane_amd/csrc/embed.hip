@@ -40,19 +40,17 @@ constexpr int STAGE_ROWS = 15 * ROWS_PER_WAVE;    // two buffers of 240 rows x 1
 // ---------------------------------------------------------------------------------------------
 template <bool VEC_D>
 __global__ __launch_bounds__(256) void gather_kernel(float *__restrict__ x, const float *__restrict__ E,
-                                                     const int32_t *__restrict__ ids, int V, int D, int S,
-                                                     int t_tiles) {
+                                                     const int32_t *__restrict__ ids, int V, int D, int S, int N) {
     __shared__ float tile[TT][TD + 1];
     __shared__ int tok[TT];
-    const int bt = blockIdx.x;                 // (b, t-tile)
-    const int b = bt / t_tiles, t0 = (bt - b * t_tiles) * TT;
+    const int n0 = blockIdx.x * TT;            // 64 consecutive positions, of one or several sequences
     const int d0 = blockIdx.y * TD;
     const int tid = threadIdx.x;
     if (tid < TT) {
-        const int t = t0 + tid;
+        const int n = n0 + tid;
         int id = -1;
-        if (t < S) {
-            id = ids[(size_t)b * S + t];
+        if (n < N) {
+            id = ids[n];
             if (id < 0 || id >= V) id = -1;
         }
         tok[tid] = id;
@@ -81,27 +79,29 @@ __global__ __launch_bounds__(256) void gather_kernel(float *__restrict__ x, cons
         }
     }
     __syncthreads();
-    // phase 2: LDS -> channel-first output, lanes along t
+    // phase 2: LDS -> channel-first output, lanes along positions; four consecutive positions lie in one sequence
+    // when S is a multiple of 4
     {
         const int tq = tid & 15, r0 = tid >> 4;
-        const bool s_vec = (S & 3) == 0;
-        const int t = t0 + 4 * tq;
+        const int n4 = n0 + 4 * tq;
         const int i0 = tok[4 * tq], i1 = tok[4 * tq + 1], i2 = tok[4 * tq + 2], i3 = tok[4 * tq + 3];
-        const bool all = (i0 >= 0) & (i1 >= 0) & (i2 >= 0) & (i3 >= 0) & s_vec;
+        const bool all = (i0 >= 0) & (i1 >= 0) & (i2 >= 0) & (i3 >= 0) & ((S & 3) == 0) & (((uintptr_t)x & 15u) == 0);
+        const int b4 = n4 / S, t4 = n4 - b4 * S;
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const int dl = r0 + 16 * k;
             const int d = d0 + dl;
             if (d >= D) continue;
-            float *dst = x + ((size_t)b * D + d) * S + t;
             if (all) {
                 v4f v = {tile[4 * tq][dl], tile[4 * tq + 1][dl], tile[4 * tq + 2][dl], tile[4 * tq + 3][dl]};
-                st4(dst, v);
+                st4(x + ((size_t)b4 * D + d) * S + t4, v);
             } else {
-                if (i0 >= 0) dst[0] = tile[4 * tq][dl];
-                if (i1 >= 0) dst[1] = tile[4 * tq + 1][dl];
-                if (i2 >= 0) dst[2] = tile[4 * tq + 2][dl];
-                if (i3 >= 0) dst[3] = tile[4 * tq + 3][dl];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if (tok[4 * tq + j] < 0) continue;          // also: positions past the end
+                    const int n = n4 + j, bb = n / S;
+                    x[((size_t)bb * D + d) * S + (n - bb * S)] = tile[4 * tq + j][dl];
+                }
             }
         }
     }
@@ -824,12 +824,13 @@ MI355_API int mi355_embed_gather_dev(float *x, const float *E, const int32_t *id
     if (!mi355_ready("embed_gather")) return -1;
     if (!x || !E || !ids) return mi355_fail("embed_gather: NULL pointer");
     if (V <= 0 || D <= 0 || S <= 0 || batch <= 0) return mi355_fail("embed_gather: bad shape V=%d D=%d S=%d batch=%d", V, D, S, batch);
-    const int t_tiles = (int)ceil_div((size_t)S, TT);
-    const dim3 grid((unsigned)(batch * t_tiles), (unsigned)ceil_div((size_t)D, TD));
+    if ((size_t)batch * S > (size_t)1 << 30) return mi355_fail("embed_gather: more than 2^30 positions");
+    const int N = batch * S;
+    const dim3 grid((unsigned)ceil_div((size_t)N, TT), (unsigned)ceil_div((size_t)D, TD));
     if (grid.y > 65535) return mi355_fail("embed_gather: D too large");
     const bool vec_d = (D % 4 == 0) && aligned16(E) && aligned16(x);
-    if (vec_d) hipLaunchKernelGGL((gather_kernel<true>), grid, dim3(256), 0, g_ctx.stream, x, E, ids, V, D, S, t_tiles);
-    else hipLaunchKernelGGL((gather_kernel<false>), grid, dim3(256), 0, g_ctx.stream, x, E, ids, V, D, S, t_tiles);
+    if (vec_d) hipLaunchKernelGGL((gather_kernel<true>), grid, dim3(256), 0, g_ctx.stream, x, E, ids, V, D, S, N);
+    else hipLaunchKernelGGL((gather_kernel<false>), grid, dim3(256), 0, g_ctx.stream, x, E, ids, V, D, S, N);
     LAUNCH_OK("embed_gather");
     return 0;
 }

@@ -369,6 +369,9 @@ def _embed_case(seed, V, D, B, S, oob=0):
     (500, 50, 3, 37, 4),          # ragged D and S, out-of-range ids
     (70, 4, 1, 1, 0),
     (1000, 1024, 2, 256, 2),
+    (1000, 32, 2048, 8, 3),       # many short sequences: a block of 64 positions spans eight of them
+    (1000, 20, 700, 6, 2),        # ... with S not a multiple of 4
+    (50, 3, 1, 257, 5),
 ])
 def test_embed_gather_bit_exact(br, V, D, B, S, oob):
     say("gather V=%d D=%d B=%d S=%d" % (V, D, B, S))
