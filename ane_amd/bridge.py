@@ -68,6 +68,7 @@ SIGNATURES = {
     "mi355_rmsnorm_bwd_dev": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _f, _i]),
     "mi355_dw_defer": (_i, [_i]),
     "mi355_dw_flush": (_i, []),
+    "mi355_rmsnorm_bwd_residual_dev": (_i, [_p, _p, _p, _p, _p, _p, _p, _f, _i, _i, _i, _f, _i]),
     "mi355_residual_rmsnorm_fwd_dev": (_i, [_p, _p, _p, _p, _f, _p, _i, _i, _i, _f]),
     "mi355_swiglu_fwd_dev": (_i, [_p, _p, _p, _z]),
     "mi355_swiglu_bwd_dev": (_i, [_p, _p, _p, _p, _p, _z]),

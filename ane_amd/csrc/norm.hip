@@ -98,11 +98,14 @@ __global__ __launch_bounds__(THREADS) void rms_fwd_kernel(float *__restrict__ y,
     }
 }
 
-template <int VEC, int LPR, int THREADS, int CAP>
-__global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__restrict__ dw_part,
-                                                          const float *dy, const float *__restrict__ x,
-                                                          const float *__restrict__ w, int C, int S, int strips,
-                                                          int nblk, float eps, float invC, int variant) {
+// RES: the residual of the backward pass rides along (training/training_dynamic/train.m:586-595, :714-721):
+// dx = rmsnorm_bwd(...) + res, and optionally dx2 = alpha2 * dx.  Its rows are loaded with x and dy, so the fused
+// op has no extra latency phase; the adds are the ones the separate passes would do, in the same order.
+template <int VEC, int LPR, int THREADS, int CAP, bool RES>
+__device__ __forceinline__ void rms_bwd_body(float *dx, float *__restrict__ dw_part, const float *dy,
+                                             const float *__restrict__ x, const float *__restrict__ w, int C, int S,
+                                             int strips, int nblk, float eps, float invC, int variant,
+                                             const float *res, float *dx2, float alpha2) {
     constexpr int RPS = THREADS / LPR;
     constexpr int W = LPR * VEC;
     constexpr int NW = THREADS / 64;
@@ -115,6 +118,8 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
     const size_t base = (size_t)slab * C * S + col;
     const float *xs = x + base, *dys = dy + base;
     float *dxs = dx + base;
+    const float *ress = RES ? res + base : nullptr;
+    float *dx2s = (RES && dx2) ? dx2 + base : nullptr;
     float *part = dw_part + (size_t)blk * C;
 
     float acc[2][VEC];   // [0] = sum x^2, [1] = sum (dy*x)*w
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
         }
     };
     auto row_out = [&](int c, const float (&xr)[VEC], const float (&dyr)[VEC], float wc, const float (&rr)[VEC],
-                       const float (&dotn)[VEC]) {
+                       const float (&dotn)[VEC], const float (&rs)[VEC]) {
         float o[VEC];
         float p = 0.f;
 #pragma unroll
@@ -137,24 +142,38 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
             if (variant == 0) o[j] = ((dyr[j] - xr[j] * dotn[j]) * rr[j]) * wc;
             else o[j] = (dyr[j] * wc) * rr[j] - (xr[j] * dotn[j]) * rr[j];
             p += (dyr[j] * xr[j]) * rr[j];
+            if constexpr (RES) o[j] = o[j] + rs[j];
         }
         if (col_ok) stv_nt<VEC>(dxs + (size_t)c * S, o);
+        if constexpr (RES) {
+            if (dx2s && col_ok) {
+                float o2[VEC];
+#pragma unroll
+                for (int j = 0; j < VEC; j++) o2[j] = o[j] * alpha2;
+                stv_nt<VEC>(dx2s + (size_t)c * S, o2);
+            }
+        }
         p = group_sum<(LPR < 64 ? LPR : 64)>(p);
         if (lc == 0) part[c] = p;
     };
 
     if constexpr (CAP > 0) {
-        float xv[CAP][VEC], dv[CAP][VEC], wv[CAP];
+        float xv[CAP][VEC], dv[CAP][VEC], wv[CAP], rv[RES ? CAP : 1][VEC];
 #pragma unroll
         for (int k = 0; k < CAP; k++) {
             const int c = row0 + k * RPS;
             if (c < C && col_ok) {
                 ldv_nt<VEC>(xv[k], xs + (size_t)c * S);
                 ldv_nt<VEC>(dv[k], dys + (size_t)c * S);
+                if constexpr (RES) ldv_nt<VEC>(rv[k], ress + (size_t)c * S);
                 wv[k] = w[c];
             } else {
 #pragma unroll
                 for (int j = 0; j < VEC; j++) xv[k][j] = dv[k][j] = 0.f;
+                if constexpr (RES) {
+#pragma unroll
+                    for (int j = 0; j < VEC; j++) rv[k][j] = 0.f;
+                }
                 wv[k] = 0.f;
             }
         }
@@ -171,7 +190,7 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
 #pragma unroll
         for (int k = 0; k < CAP; k++) {
             const int c = row0 + k * RPS;
-            if (c < C) row_out(c, xv[k], dv[k], wv[k], rr, dotn);   // uniform per LPR lane group
+            if (c < C) row_out(c, xv[k], dv[k], wv[k], rr, dotn, rv[RES ? k : 0]);   // uniform per LPR lane group
         }
     } else {
         if (col_ok)
@@ -192,17 +211,39 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__re
         finish(rr, dotn);
 #pragma unroll 4
         for (int c = row0; c < C; c += RPS) {
-            float a[VEC], b[VEC];
+            float a[VEC], b[VEC], r[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; j++) r[j] = 0.f;
             if (col_ok) {
                 ldv_nt<VEC>(a, xs + (size_t)c * S);
                 ldv_nt<VEC>(b, dys + (size_t)c * S);
+                if constexpr (RES) ldv_nt<VEC>(r, ress + (size_t)c * S);
             } else {
 #pragma unroll
                 for (int j = 0; j < VEC; j++) a[j] = b[j] = 0.f;
             }
-            row_out(c, a, b, w[c], rr, dotn);
+            row_out(c, a, b, w[c], rr, dotn, r);
         }
     }
+}
+
+template <int VEC, int LPR, int THREADS, int CAP>
+__global__ __launch_bounds__(THREADS) void rms_bwd_kernel(float *dx, float *__restrict__ dw_part,
+                                                          const float *dy, const float *__restrict__ x,
+                                                          const float *__restrict__ w, int C, int S, int strips,
+                                                          int nblk, float eps, float invC, int variant) {
+    rms_bwd_body<VEC, LPR, THREADS, CAP, false>(dx, dw_part, dy, x, w, C, S, strips, nblk, eps, invC, variant, nullptr,
+                                                nullptr, 0.f);
+}
+
+template <int VEC, int LPR, int THREADS, int CAP>
+__global__ __launch_bounds__(THREADS) void rms_bwd_res_kernel(float *dx, float *__restrict__ dw_part,
+                                                              const float *dy, const float *__restrict__ x,
+                                                              const float *__restrict__ w, int C, int S, int strips,
+                                                              int nblk, float eps, float invC, int variant,
+                                                              const float *res, float *dx2, float alpha2) {
+    rms_bwd_body<VEC, LPR, THREADS, CAP, true>(dx, dw_part, dy, x, w, C, S, strips, nblk, eps, invC, variant, res, dx2,
+                                               alpha2);
 }
 
 
@@ -364,6 +405,15 @@ void launch_bwd(float *dx, float *part, const float *dy, const float *x, const f
                        dy, x, w, C, S, strips, nblk, eps, 1.0f / (float)C, variant);
 }
 
+template <int VEC, int LPR, int THREADS, int CAP>
+void launch_bwd_res(float *dx, float *part, const float *dy, const float *x, const float *w, int C, int S, int batch,
+                    float eps, int variant, const float *res, float *dx2, float alpha2) {
+    const int strips = (int)ceil_div((size_t)S, (size_t)LPR * VEC);
+    const int nblk = strips * batch;
+    hipLaunchKernelGGL((rms_bwd_res_kernel<VEC, LPR, THREADS, CAP>), dim3(nblk), dim3(THREADS), 0, g_ctx.stream, dx, part,
+                       dy, x, w, C, S, strips, nblk, eps, 1.0f / (float)C, variant, res, dx2, alpha2);
+}
+
 #define NORM_DISPATCH(FN, cfg, ...)                                                                   \
     do {                                                                                              \
         const int key = (cfg).vec * 1000000 + (cfg).lpr * 10000 + ((cfg).threads / 256) * 100 + (cfg).cap; \
@@ -421,6 +471,31 @@ MI355_API int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const
     if (!part) return -1;
     NORM_DISPATCH(launch_bwd, cfg, dx, part, dy, x, w, C, S, batch, eps, variant);
     LAUNCH_OK("rmsnorm_bwd");
+    if (mi355_dw_submit(dw, part, nblk, C)) return -1;
+    return mi355_dw_op_end();
+}
+
+MI355_API int mi355_rmsnorm_bwd_residual_dev(float *dx, float *dx_scaled, float *dw, const float *dy, const float *x,
+                                             const float *w, const float *res, float alpha, int C, int S, int batch,
+                                             float eps, int variant) {
+    if (!mi355_ready("rmsnorm_bwd_residual")) return -1;
+    if (!dx || !dw || !dy || !x || !w || !res) return mi355_fail("rmsnorm_bwd_residual: NULL pointer");
+    if (C <= 0 || S <= 0 || batch <= 0)
+        return mi355_fail("rmsnorm_bwd_residual: bad shape C=%d S=%d batch=%d", C, S, batch);
+    if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd_residual: variant must be 0 or 1");
+    if (dx_scaled && (dx_scaled == dx || dx_scaled == dy || dx_scaled == x || dx_scaled == res))
+        return mi355_fail("rmsnorm_bwd_residual: dx_scaled must not alias another operand");
+    const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(res) &&
+                        (!dx_scaled || aligned16(dx_scaled));
+    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 8, 0, g_ctx.rms_lpr, g_ctx.rms_threads, true);
+    // three operands of 16 rows per lane do not fit the registers: the 8-row tile, or the two-sweep variant
+    if (cfg.cap > 8) cfg = C <= 1024 ? NormCfg{4, 4, 512, 8} : NormCfg{cfg.vec, cfg.lpr, cfg.threads, 0};
+    const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
+    const int nblk = strips * batch;
+    float *part = mi355_dw_partials((size_t)nblk * C, dw, nullptr);
+    if (!part) return -1;
+    NORM_DISPATCH(launch_bwd_res, cfg, dx, part, dy, x, w, C, S, batch, eps, variant, res, dx_scaled, alpha);
+    LAUNCH_OK("rmsnorm_bwd_residual");
     if (mi355_dw_submit(dw, part, nblk, C)) return -1;
     return mi355_dw_op_end();
 }

@@ -60,6 +60,9 @@ def alg_bytes(cfg, a=4):
         "scale_copy": 2 * a * H * St,        # y = alpha*a over an [H,St] tensor: a plain copy-shaped stream (train.m:523,595)
         # residual + the RMSNorm after it in one launch; as two ops the same work is 12CSt + 8CSt + 4C
         "residual_rmsnorm_fwd": 4 * a * C * St + 4 * C,
+        # RMSNorm backward + the backward residual + the scaled copy in one launch (train.m:586-595); as three ops
+        # the same work is 12CSt + 12CSt + 8CSt
+        "rmsnorm_bwd_residual": 5 * a * C * St + 12 * C,
         "softmax_ce": 2 * a * V * S,
         "int8_scale": 4 * n8,
         "int8_quant": 5 * n8,
@@ -145,6 +148,7 @@ class Workload:
         self.y8 = A(n8)
         self.scale8 = A(1)
         self.scratch_h = A((B, H, S))          # output of the copy-shaped calibration op only
+        self.scratch_c = A((B, C, S))          # the scaled copy of the fused backward's timing run
         self.cos, self.sin = br.rope_tables_dev(S, cfg["hd"], cfg["theta"])
         # training/training_dynamic/train.m:188; BASELINE config 1 asks for (2*12)^0.25 at the Stories110M shape
         self.alpha = float(np.float32((2.0 * 12) ** 0.25 if not cfg["qk_norm"] else 1.0 / np.sqrt(2.0 * cfg["layers"])))
@@ -188,6 +192,10 @@ class Workload:
                                          B * c["heads"], 1e-5, 0))
             ck(lib.mi355_rmsnorm_bwd_dev(d["dk"].ptr, d["dwk"].ptr, d["k_rot"].ptr, d["k"].ptr, d["wk"].ptr, hd, S,
                                          B * c["kv_heads"], 1e-5, 0))
+        elif name == "rms_bwd_res":    # dx2 = rmsnorm_bwd(dx_ffn; x2, w_ffn) + dy ; scaled copy for the next stage (train.m:586-595)
+            # outputs go to buffers that no op of the sweep writes
+            ck(lib.mi355_rmsnorm_bwd_residual_dev(d["dy_out"].ptr, self.scratch_c.ptr, d["dw_ffn"].ptr, d["dx_ffn"].ptr,
+                                                  d["x2"].ptr, d["w_ffn"].ptr, d["dy"].ptr, self.alpha, C, S, B, 1e-5, 0))
         elif name == "residual1":
             ck(lib.mi355_axpby_dev(d["x2"].ptr, d["x"].ptr, d["o"].ptr, self.alpha, n_c, 0))
         elif name == "res_rms1":       # x2 = x + alpha*o ; x2n = rmsnorm(x2)   (train.m:460-461)
@@ -273,10 +281,12 @@ def per_op_table(br, wl, reps):
     ab = alg_bytes(wl.cfg, 2 if wl.bf16 else 4)
     names = {"rmsnorm_fwd": "rmsnorm_fwd", "rmsnorm_bwd": "rmsnorm_bwd", "qknorm_rope_fwd": "qknorm_rope_fwd",
              "qknorm_rope_bwd": "qknorm_rope_bwd", "swiglu_fwd": "swiglu_fwd", "swiglu_bwd": "swiglu_bwd",
-             "residual1": "residual", "res_rms1": "residual_rmsnorm_fwd", "scale_copy": "scale_copy"}
+             "residual1": "residual", "res_rms1": "residual_rmsnorm_fwd", "rms_bwd_res": "rmsnorm_bwd_residual",
+             "scale_copy": "scale_copy"}
     table = []
     if wl.bf16:
-        del names["res_rms1"]          # the fused residual + RMSNorm exists for fp32 storage only
+        del names["res_rms1"]          # the fused residual + RMSNorm ops exist for fp32 storage only
+        del names["rms_bwd_res"]
     elif wl.cfg["qk_norm"]:
         # the fused QK-norm + RoPE again as its unfused composition (three launches, priced at the fused op's bytes);
         # run last: it overwrites q_rot/k_rot with intermediates

@@ -158,6 +158,17 @@ int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const float *x,
 int mi355_dw_defer(int on);
 int mi355_dw_flush(void);
 
+/* RMSNorm backward with the residual of the backward pass riding along, one launch:
+ *   dx = rmsnorm_bwd(dy, x, w) + res;  dx_scaled = alpha * dx  (dx_scaled may be NULL);  dw += as rmsnorm_bwd.
+ * Replaces memset + rmsnorm_bwd + the add loop + vDSP_vsmul — training/training_dynamic/train.m:586-595 — and
+ * rmsnorm_bwd + the add loop of train.m:714-721.  The adds and the scale are the separate passes' own, in their
+ * order: the result equals mi355_rmsnorm_bwd_dev followed by mi355_axpby_dev (modes 2 and 1) bit for bit when
+ * both run on the same tile shape (they do below 32 x 256 columns), and to the rounding of the column sums
+ * otherwise.  dx may alias res or dy. */
+int mi355_rmsnorm_bwd_residual_dev(float *dx, float *dx_scaled, float *dw, const float *dy, const float *x,
+                                   const float *w, const float *res, float alpha, int C, int S, int batch, float eps,
+                                   int variant);
+
 /* Residual add fused with the RMSNorm that follows it in the loops: vDSP_vsma + rmsnorm at
  * training/training_dynamic/train.m:460-461 (and a layer's x_next feeding the next rmsnorm at :417).
  * y = a + alpha*b (as mode 0 of mi355_axpby_dev); yn = rmsnorm(y, w).  One launch instead of two; the

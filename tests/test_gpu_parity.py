@@ -96,6 +96,58 @@ def test_rmsnorm_columns_of_zeros_tiny_and_huge_values(br):
         assert H.rel_err(dwd.numpy(), rdw) <= TOL
 
 
+@pytest.mark.parametrize("B,Cc,S", [(16, 1024, 256), (32, 1024, 256), (1, 768, 256), (2, 100, 37), (2, 2500, 64), (3, 48, 20)])
+def test_rmsnorm_bwd_with_residual_equals_the_separate_passes(br, B, Cc, S):
+    """dx = rmsnorm_bwd + res and dx_scaled = alpha*dx in one launch (training/training_dynamic/train.m:586-595):
+    bit for bit what rmsnorm_bwd, the add and the scale give as three launches, and the oracle's composition."""
+    x = H.normal(10, (B, Cc, S)); w = H.normal(11, Cc, 1.0, 0.02); dy = H.normal(12, (B, Cc, S))
+    res = H.normal(13, (B, Cc, S)); dw0 = H.normal(14, Cc)
+    alpha = np.float32(1 / np.sqrt(2 * 28))
+    xd, wd, dyd, rd = dev(br, x), dev(br, w), dev(br, dy), dev(br, res)
+    n = x.size
+    # the same tile for both (at 32 x 256 columns and up the plain op would take a 16-row tile that the fused one,
+    # with three operands in registers, cannot: then the column sums are rounded differently)
+    br.tune("rms_lpr", 4); br.tune("rms_threads", 512)
+    try:
+        _bwd_residual_cases(br, B, Cc, S, x, w, dy, res, dw0, alpha, xd, wd, dyd, rd, n)
+    finally:
+        br.tune("rms_lpr", 0); br.tune("rms_threads", 0)
+    # default tiles: within tolerance of the oracle whatever the tile
+    b_dx = br.DevArray(x.shape); b_dw = dev(br, dw0)
+    br.check(br.lib.mi355_rmsnorm_bwd_residual_dev(b_dx.ptr, None, b_dw.ptr, dyd.ptr, xd.ptr, wd.ptr, rd.ptr, 0.0, Cc, S, B,
+                                                   1e-5, 0))
+    rdx, rdw = O.rmsnorm_bwd(dy, x, w, variant=0, dw=dw0)
+    assert H.rel_err(b_dx.numpy(), O.axpby(rdx, res, 0.0, 2)) <= TOL and H.rel_err(b_dw.numpy(), rdw) <= TOL
+
+
+def _bwd_residual_cases(br, B, Cc, S, x, w, dy, res, dw0, alpha, xd, wd, dyd, rd, n):
+    for variant in (0, 1):
+        # three launches
+        a_dx = br.DevArray(x.shape); a_sc = br.DevArray(x.shape); a_dw = dev(br, dw0)
+        br.check(br.lib.mi355_rmsnorm_bwd_dev(a_dx.ptr, a_dw.ptr, dyd.ptr, xd.ptr, wd.ptr, Cc, S, B, 1e-5, variant))
+        br.check(br.lib.mi355_axpby_dev(a_dx.ptr, a_dx.ptr, rd.ptr, 0.0, n, 2))
+        br.check(br.lib.mi355_axpby_dev(a_sc.ptr, a_dx.ptr, None, alpha, n, 1))
+        # one launch
+        b_dx = br.DevArray(x.shape); b_sc = br.DevArray(x.shape); b_dw = dev(br, dw0)
+        br.check(br.lib.mi355_rmsnorm_bwd_residual_dev(b_dx.ptr, b_sc.ptr, b_dw.ptr, dyd.ptr, xd.ptr, wd.ptr, rd.ptr, alpha,
+                                                       Cc, S, B, 1e-5, variant))
+        assert b_dx.numpy().tobytes() == a_dx.numpy().tobytes()
+        assert b_sc.numpy().tobytes() == a_sc.numpy().tobytes()
+        assert b_dw.numpy().tobytes() == a_dw.numpy().tobytes()
+        rdx, rdw = O.rmsnorm_bwd(dy, x, w, variant=variant, dw=dw0)
+        want = O.axpby(rdx, res, 0.0, 2)
+        assert H.rel_err(b_dx.numpy(), want) <= TOL
+        assert H.rel_err(b_sc.numpy(), O.axpby(want, None, alpha, 1)) <= TOL
+        assert H.rel_err(b_dw.numpy(), rdw) <= TOL
+        # in place over the residual, without the scaled copy (train.m:714-721)
+        c_dx = dev(br, res); c_dw = dev(br, dw0)
+        br.check(br.lib.mi355_rmsnorm_bwd_residual_dev(c_dx.ptr, None, c_dw.ptr, dyd.ptr, xd.ptr, wd.ptr, c_dx.ptr, 0.0,
+                                                       Cc, S, B, 1e-5, variant))
+        assert c_dx.numpy().tobytes() == a_dx.numpy().tobytes()
+    assert br.lib.mi355_rmsnorm_bwd_residual_dev(b_dx.ptr, b_dx.ptr, b_dw.ptr, dyd.ptr, xd.ptr, wd.ptr, rd.ptr, alpha, Cc, S, B,
+                                                 1e-5, 0) == -1
+
+
 def test_rmsnorm_golden_reference_recipe(br):
     x, dy, w = GOLD["rms_x"], GOLD["rms_dy"], GOLD["rms_w"]
     Cc, S = x.shape
