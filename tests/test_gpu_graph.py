@@ -46,6 +46,8 @@ def run(br, d, cos, sin):
     ck(L.mi355_swiglu_fwd_dev(d["act"].ptr, d["h1"].ptr, d["h3"].ptr, n_h))
     ck(L.mi355_swiglu_bwd_dev(d["dh1"].ptr, d["dh3"].ptr, d["ds"].ptr, d["h1"].ptr, d["h3"].ptr, n_h))
     ck(L.mi355_rmsnorm_bwd_dev(d["dx"].ptr, d["dw2"].ptr, d["dy"].ptr, d["x2"].ptr, d["w2"].ptr, C_, S, B, 1e-5, 0))
+    ck(L.mi355_rmsnorm_bwd_residual_dev(d["xn"].ptr, d["deq"].ptr, d["dw2"].ptr, d["dy"].ptr, d["x2"].ptr, d["w2"].ptr,
+                                        d["o"].ptr, ALPHA, C_, S, B, 1e-5, 0))
     ck(L.mi355_qknorm_rope_bwd_dev(d["dq"].ptr, d["dk"].ptr, d["dwq"].ptr, d["dwk"].ptr, d["gq"].ptr, d["gk"].ptr, d["q"].ptr,
                                    d["k"].ptr, d["wq"].ptr, d["wk"].ptr, HEADS, KVH, HD, S, B, cos, sin, 1e-5, 0))
     ck(L.mi355_softmax_ce_dev(d["dl"].ptr, d["loss"].ptr, d["logits"].ptr, d["tgt"].ptr, V, S, 256.0))
