@@ -429,6 +429,12 @@ def bench_embed(br, args):
     scatter()
     t_s_tree = time_region(br, scatter, args.steps) / nbuf
     br.tune("scatter_tree", 0)
+
+    def copy():                         # y = 1.0*a over one activation slab: the streaming rate next to the two ops, and
+        for x, g in zip(xs, gs):        # the known-size dispatch that scales the traffic counters of the profile
+            br.check(br.lib.mi355_axpby_dev(x.ptr, g.ptr, None, 1.0, g.size, 1))
+    copy()
+    t_c = time_region(br, copy, args.steps) / nbuf
     b_g = 8 * D * N + 4 * N
     b_s = 4 * D * N + 8 * D * U + 4 * N
     out = {"metric": "embedding gather + ordered scatter-add (BASELINE config 2)", "value": N / ((t_g + t_s) / 1e3),
@@ -440,7 +446,14 @@ def bench_embed(br, args):
                    dict(op="embed_scatter_add", ms=t_s, alg_mb=b_s / 1e6, gbs=b_s / t_s / 1e6,
                         frac=b_s / t_s / 1e6 / PEAK_HBM_GBS),
                    dict(op="embed_scatter_add (scatter_tree=1)", ms=t_s_tree, alg_mb=b_s / 1e6, gbs=b_s / t_s_tree / 1e6,
-                        frac=b_s / t_s_tree / 1e6 / PEAK_HBM_GBS)]}
+                        frac=b_s / t_s_tree / 1e6 / PEAK_HBM_GBS),
+                   dict(op="copy of one activation slab", ms=t_c, alg_mb=8 * D * N / 1e6, gbs=8 * D * N / t_c / 1e6,
+                        frac=8 * D * N / t_c / 1e6 / PEAK_HBM_GBS)],
+           "roofline": dict(bound="hbm", kernel="embed_scatter_add (3 launches)", achieved=b_s / t_s / 1e6, peak=PEAK_HBM_GBS,
+                            unit="GB/s", frac=b_s / t_s / 1e6 / PEAK_HBM_GBS,
+                            # chunk_sort 0.16 + rank_transpose 101.67 + seg_sum 74.31 MB (FETCH_SIZE + WRITE_SIZE, scaled)
+                            traffic=176.14e6, traffic_source="profiles/embed_config2_pmc_fetch_write.md",
+                            alg_bytes_per_launch=b_s, avg_launch_ms=t_s)}
     if args.cpu_layers > 0:
         import oracle as O
         Eh = E.numpy(); g0 = gs[0].numpy()
