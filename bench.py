@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X published HBM3E peak
 # HBM-side bytes per dispatch of the dominant kernel at the default workload, from the two rocprofv3 --pmc
 # runs summarised in profiles/qwen3_sweep_pmc_fetch_write.md (FETCH_SIZE x 1.9992 + WRITE_SIZE x 0.9992, the
 # factors the same counters need to read 50.33 MB for a plain 50.33 MB copy).  Not measured live.
-MEASURED_TRAFFIC_BYTES = {"swiglu_bwd": 251.54e6}
+MEASURED_TRAFFIC_BYTES = {"swiglu_bwd": 251.56e6}
 
 # Qwen3-0.6B (training/training_dynamic/models/qwen3_06b.h:6-16), batch 16
 Q3 = dict(C=1024, H=3072, heads=16, kv_heads=8, hd=128, S=256, batch=16, layers=28, V=151936, theta=1e6,
