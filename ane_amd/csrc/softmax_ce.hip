@@ -289,11 +289,23 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
     if (!mi355_ready(who)) return -1;
     if (!dlogits || !loss_dev || !logits || !targets) return mi355_fail("%s: NULL pointer", who);
     if (V <= 0 || S <= 0) return mi355_fail("%s: bad shape V=%d S=%d", who, V, S);
-    // rows per workgroup: about 600 workgroups per column strip (2+ per compute unit), between one and
-    // four 64-row register tiles; 256 rows measured best at V = 151936
-    int rpb = g_ctx.ce_rows > 0 ? g_ctx.ce_rows : (int)ceil_div((size_t)V, 600);
-    rpb = (int)ceil_div((size_t)rpb, CE_TILE_ROWS) * CE_TILE_ROWS;
-    if (g_ctx.ce_rows <= 0 && rpb > 4 * CE_TILE_ROWS) rpb = 4 * CE_TILE_ROWS;
+    // Rows per workgroup: one to six 64-row register tiles, chosen so that the workgroups of a column strip fill the
+    // compute units evenly (at least 1.75 per unit, and the last round of them as full as possible); ties go to
+    // the larger block, which leaves fewer partials to merge.  At V = 151936 on 256 units: 320 rows, 475
+    // workgroups (87 us for the op; 256 rows and 594 workgroups: 91 us; 384 rows and 396: 97 us).
+    int rpb = g_ctx.ce_rows;
+    if (rpb <= 0) {
+        const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
+        double best = -1.0;
+        rpb = CE_TILE_ROWS;
+        for (int t = 1; t <= 6; t++) {
+            const long nb = (long)ceil_div((size_t)V, (size_t)t * CE_TILE_ROWS);
+            if (t > 1 && nb * 4 < (long)cu * 7) break;
+            const long rounds = (nb + cu - 1) / cu;
+            const double score = (double)nb / (double)(rounds * cu) + 0.002 * t;
+            if (score > best) { best = score; rpb = t * CE_TILE_ROWS; }
+        }
+    }
     const int nblk = (int)ceil_div((size_t)V, (size_t)rpb);
     // four columns per lane: 16 bytes of fp32, 8 bytes of bf16
     const uintptr_t mask = 4 * sizeof(T) - 1;
