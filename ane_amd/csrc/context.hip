@@ -140,7 +140,7 @@ MI355_API int mi355_tune_set(const char *key, int value) {
     struct { const char *k; int *v; } tab[] = {
         {"rms_lpr", &g_ctx.rms_lpr}, {"rms_threads", &g_ctx.rms_threads},
         {"ew_unroll", &g_ctx.ew_unroll},
-        {"ce_rows", &g_ctx.ce_rows}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
+        {"ce_rows", &g_ctx.ce_rows}, {"ce_rows2", &g_ctx.ce_rows2}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
         {"gemm_splitk", &g_ctx.gemm_splitk}, {"scatter_tree", &g_ctx.scatter_tree},
     };
     for (auto &t : tab)

@@ -283,6 +283,19 @@ __global__ __launch_bounds__(CE_THREADS) void ce_grad_kernel(T *dlogits, const T
     }
 }
 
+// resident workgroups of the second pass per compute unit (asked of the runtime once per storage type)
+template <typename T>
+int grad_blocks_per_cu() {
+    static int cached = 0;
+    if (cached == 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, ce_grad_kernel<4, T>, CE_THREADS, 0) != hipSuccess || n <= 0)
+            n = 4;
+        cached = n;
+    }
+    return cached;
+}
+
 template <typename T>
 int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const int32_t *targets, int V, int S,
            float grad_scale) {
@@ -307,6 +320,23 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
         }
     }
     const int nblk = (int)ceil_div((size_t)V, (size_t)rpb);
+    // The second pass has no partials to merge and its own blocks: a multiple of 16 rows between 64 and 384 that
+    // fills the resident workgroup slots of the chip in as few rounds as it can (four workgroups fit a compute
+    // unit: at V = 151936, 160 rows = 950 workgroups for 1024 slots, 83 us for the op; 144 rows = 1056 workgroups,
+    // a second round for 32 of them, 98 us; 320 rows, less than half the slots, 88 us).
+    int rpb2 = g_ctx.ce_rows2;
+    if (rpb2 <= 0) {
+        const long slots = (long)(g_ctx.num_cu > 0 ? g_ctx.num_cu : 256) * grad_blocks_per_cu<T>();
+        double best = -1.0;
+        rpb2 = CE_TILE_ROWS;
+        for (int m = CE_TILE_ROWS / 16; m <= 6 * CE_TILE_ROWS / 16; m++) {
+            const long nb = (long)ceil_div((size_t)V, (size_t)m * 16);
+            const long rounds = (nb + slots - 1) / slots;
+            const double score = (double)nb / (double)(rounds * slots) - 0.05 * (double)(rounds - 1) + 1e-4 * m;
+            if (score > best) { best = score; rpb2 = m * 16; }
+        }
+    }
+    const int nblk2 = (int)ceil_div((size_t)V, (size_t)rpb2);
     // four columns per lane: 16 bytes of fp32, 8 bytes of bf16
     const uintptr_t mask = 4 * sizeof(T) - 1;
     const bool vec_ok = (S % 4 == 0) && (((uintptr_t)logits | (uintptr_t)dlogits) & mask) == 0;
@@ -329,12 +359,13 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
     hipLaunchKernelGGL(ce_combine_kernel<T>, dim3((unsigned)ceil_div((size_t)S, CB_COLS)), dim3(1024), 0, g_ctx.stream, colM,
                        colInv, colLoss, pm, pl, logits, targets, V, S, nblk);
     LAUNCH_OK("softmax_ce combine");
+    const dim3 grid2((unsigned)nblk2, (unsigned)strips);
     if (vec_ok)
-        hipLaunchKernelGGL((ce_grad_kernel<4, T>), grid, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
-                           targets, V, S, rpb, 1.0f / (float)S, grad_scale, loss_dev, colLoss);
+        hipLaunchKernelGGL((ce_grad_kernel<4, T>), grid2, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
+                           targets, V, S, rpb2, 1.0f / (float)S, grad_scale, loss_dev, colLoss);
     else
-        hipLaunchKernelGGL((ce_grad_kernel<1, T>), grid, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
-                           targets, V, S, rpb, 1.0f / (float)S, grad_scale, loss_dev, colLoss);
+        hipLaunchKernelGGL((ce_grad_kernel<1, T>), grid2, dim3(CE_THREADS), 0, g_ctx.stream, dlogits, logits, colM, colInv,
+                           targets, V, S, rpb2, 1.0f / (float)S, grad_scale, loss_dev, colLoss);
     LAUNCH_OK("softmax_ce grad");
     return 0;
 }

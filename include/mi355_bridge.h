@@ -55,7 +55,7 @@ size_t mi355_workspace_size(void);
 /* Tuning knobs for experiments; 0 = choose per shape (the default), unknown names return -1:
  * "rms_lpr" (lanes per strip row, 4/8/16) and "rms_threads" (256/512/1024) of the RMSNorm tiles, "qk_lpr" and
  * "qk_threads" (256/512) of the QK-norm + RoPE tiles, "ew_unroll" (accesses per lane of the streaming ops, 1/2/4),
- * "ce_rows" (rows of logits per workgroup), "gemm_splitk" (K slices of mi355_sgemm_dev; 1 = never split),
+ * "ce_rows" / "ce_rows2" (rows of logits per workgroup in the first / second pass of softmax-CE), "gemm_splitk" (K slices of mi355_sgemm_dev; 1 = never split),
  * "scatter_tree" (1: mi355_embed_scatter_add_dev sums long segments by a fixed tree instead of the reference's
  * sequential order: still deterministic and within 1e-5 of each row's scale, faster, no longer bit-identical to
  * the CPU loop). */
