@@ -55,7 +55,8 @@ size_t mi355_workspace_size(void);
 /* Tuning knobs for experiments; 0 = choose per shape (the default), unknown names return -1:
  * "rms_lpr" (lanes per strip row, 4/8/16) and "rms_threads" (256/512/1024) of the RMSNorm tiles, "qk_lpr" and
  * "qk_threads" (256/512) of the QK-norm + RoPE tiles, "ew_unroll" (accesses per lane of the streaming ops, 1/2/4),
- * "ce_rows" / "ce_rows2" (rows of logits per workgroup in the first / second pass of softmax-CE), "gemm_splitk" (K slices of mi355_sgemm_dev; 1 = never split),
+ * "ce_rows" / "ce_rows2" (rows of logits per workgroup in the first / second pass of softmax-CE),
+ * "gemm_splitk" (K slices of mi355_sgemm_dev; 1 = never split),
  * "scatter_tree" (1: mi355_embed_scatter_add_dev sums long segments by a fixed tree instead of the reference's
  * sequential order: still deterministic and within 1e-5 of each row's scale, faster, no longer bit-identical to
  * the CPU loop). */
@@ -109,9 +110,9 @@ int mi355_qknorm_rope_bwd_bf16_dev(uint16_t *dq, uint16_t *dk, float *dwq, float
  * counterpart in the reference (its ops are synchronous CPU calls).  Between begin and end the *_dev ops are
  * recorded instead of run; calls that allocate, wait or touch the host (buf_alloc/free/read/write, sync,
  * set_stream, workspace growth, a first-time RoPE table, embed_scatter_add beyond 16384 positions, sgemm,
- * ckpt_*) fail with -1 and end in a failed capture, so run the sequence once eagerly first.  mi355_graph_launch enqueues the replay on the
- * bridge stream; it fails if a workspace was reallocated since the recording (record again).  Accumulating ops
- * (dw +=) accumulate on every replay. */
+ * ckpt_*) fail with -1 and end in a failed capture, so run the sequence once eagerly first.  mi355_graph_launch
+ * enqueues the replay on the bridge stream; it fails if a workspace was reallocated since the recording (record
+ * again).  Accumulating ops (dw +=) accumulate on every replay. */
 typedef struct mi355_graph mi355_graph;
 int mi355_graph_begin(void);
 mi355_graph *mi355_graph_end(void);          /* NULL on failure */
