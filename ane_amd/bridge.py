@@ -83,6 +83,7 @@ SIGNATURES = {
     "mi355_softmax_ce_dev": (_i, [_p, _p, _p, _p, _i, _i, _f]),
     "mi355_minmax_dev": (_i, [_p, _p, _z]),
     "mi355_int8_scale_dev": (_i, [_p, _p, _z]),
+    "mi355_int8_quantize_dynamic_dev": (_i, [_p, _p, _p, _z, _i]),
     "mi355_int8_quant_dev": (_i, [_p, _p, _p, _z, _i]),
     "mi355_int8_dequant_dev": (_i, [_p, _p, _p, _z]),
     "mi355_sumsq_accum_dev": (_i, [_p, _p, _z, _f]),

@@ -326,6 +326,44 @@ __global__ void quant_scalar(int8_t *q, const float *x, const float *scale_p, si
     if (i < n) q[i] = (int8_t)quant1(x[i], *scale_p, rounding);
 }
 
+// Quantize with the scale taken from the per-workgroup maxima of absmax_kernel: every workgroup folds the maxima
+// itself, which saves the launch that would do it once; workgroup 0 also writes the scale out.
+template <int UNROLL>
+__global__ __launch_bounds__(EW_THREADS) void quant_dyn_kernel(int *__restrict__ q4, const float *__restrict__ x,
+                                                               const float *__restrict__ part, int nblk,
+                                                               float *__restrict__ scale_out, size_t n4, int rounding) {
+    const size_t base = (size_t)blockIdx.x * (EW_THREADS * UNROLL) + threadIdx.x;
+    v4f a[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) a[u] = ld4(x + 4 * i);
+    }
+    // the maxima (at most 256: a few cache lines, read by one wave per workgroup so that the thousand workgroups
+    // do not queue on them) are folded while the loads above are in flight
+    __shared__ float red;
+    if (threadIdx.x < 64) {
+        float m = 0.f;
+        for (int i = threadIdx.x; i < nblk; i += 64) m = fmaxf(m, part[i]);
+#pragma unroll
+        for (int k = 1; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
+        if (threadIdx.x == 0) red = m;
+    }
+    __syncthreads();
+    float scale = red / 127.0f;
+    if (scale == 0.0f) scale = 1.0f;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = scale;
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const size_t i = base + (size_t)u * EW_THREADS;
+        if (i < n4) {
+            unsigned int pk = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) pk |= ((unsigned int)(quant1(a[u][j], scale, rounding) & 0xFF)) << (8 * j);
+            q4[i] = (int)pk;
+        }
+    }
+}
 template <int UNROLL>
 __global__ __launch_bounds__(EW_THREADS) void dequant_kernel(float *__restrict__ x, const int *__restrict__ q4,
                                                              const float *__restrict__ scale_p, size_t n4) {
@@ -634,6 +672,33 @@ MI355_API int mi355_int8_quant_dev(int8_t *q, const float *x, const float *scale
         hipLaunchKernelGGL(quant_scalar, dim3((unsigned)ceil_div(n - lo, 256)), dim3(256), 0, g_ctx.stream, q, x,
                            scale_dev, lo, n, rounding);
         LAUNCH_OK("int8_quant tail");
+    }
+    return 0;
+}
+
+MI355_API int mi355_int8_quantize_dynamic_dev(int8_t *q, float *scale_dev, const float *x, size_t n, int rounding) {
+    if (!mi355_ready("int8_quantize_dynamic")) return -1;
+    if (!q || !x || !scale_dev) return mi355_fail("int8_quantize_dynamic: NULL pointer");
+    if (n == 0) return mi355_fail("int8_quantize_dynamic: empty tensor");
+    if (rounding != 0 && rounding != 1) return mi355_fail("int8_quantize_dynamic: rounding must be 0 or 1");
+    size_t n4, lo;
+    split_vec(n, aligned16(x) && ((uintptr_t)q & 3u) == 0, n4, lo);
+    if (n4 == 0) {      // no vector body: the two separate steps
+        if (mi355_int8_scale_dev(scale_dev, x, n)) return -1;
+        return mi355_int8_quant_dev(q, x, scale_dev, n, rounding);
+    }
+    size_t blocks = ceil_div(n4, (size_t)EW_THREADS);
+    if (blocks > 256) blocks = 256;         // one workgroup per compute unit; few maxima for the quantizer to fold
+    float *part = (float *)mi355_ws(blocks * sizeof(float));
+    if (!part) return -1;
+    hipLaunchKernelGGL(absmax_kernel, dim3((unsigned)blocks), dim3(EW_THREADS), 0, g_ctx.stream, part, x, n, n / 4, true);
+    const int u = pick_unroll(n4, 1);
+    EW_LAUNCH(quant_dyn_kernel, u, n4, (int *)q, x, part, (int)blocks, scale_dev, n4, rounding);
+    LAUNCH_OK("int8_quantize_dynamic");
+    if (lo < n) {
+        hipLaunchKernelGGL(quant_scalar, dim3((unsigned)ceil_div(n - lo, 256)), dim3(256), 0, g_ctx.stream, q, x,
+                           scale_dev, lo, n, rounding);
+        LAUNCH_OK("int8_quantize_dynamic tail");
     }
     return 0;
 }

@@ -67,6 +67,7 @@ def alg_bytes(cfg, a=4):
         "int8_scale": 4 * n8,
         "int8_quant": 5 * n8,
         "int8_dequant": 5 * n8,
+        "int8_quantize_dynamic": 9 * n8,     # the scale's read and the quantizer's read + write in two launches
     }
 
 
@@ -249,6 +250,8 @@ class Workload:
             self.br.check(lib.mi355_int8_quant_dev(self.q8.ptr, self.x8.ptr, self.scale8.ptr, n, 0))
         if "dequant" in which:
             self.br.check(lib.mi355_int8_dequant_dev(self.y8.ptr, self.q8.ptr, self.scale8.ptr, n))
+        if "dynamic" in which:       # scale + quantize as one call; same outputs as the two steps above
+            self.br.check(lib.mi355_int8_quantize_dynamic_dev(self.q8.ptr, self.scale8.ptr, self.x8.ptr, n, 0))
 
     def step(self):
         if self.fuse:
@@ -307,7 +310,8 @@ def per_op_table(br, wl, reps):
         for d in wl.lay:
             wl.op("qknorm_rope_fwd", d)
     for key, fn in (("softmax_ce", wl.ce), ("int8_scale", lambda: wl.int8(("scale",))),
-                    ("int8_quant", lambda: wl.int8(("quant",))), ("int8_dequant", lambda: wl.int8(("dequant",)))):
+                    ("int8_quant", lambda: wl.int8(("quant",))), ("int8_dequant", lambda: wl.int8(("dequant",))),
+                    ("int8_quantize_dynamic", lambda: wl.int8(("dynamic",)))):
         fn()
         ms = time_region(br, fn, max(reps, 3))
         table.append(dict(op=key, ms=ms, alg_mb=ab[key] / 1e6, gbs=ab[key] / ms / 1e6, frac=ab[key] / ms / 1e6 / PEAK_HBM_GBS))
@@ -736,7 +740,7 @@ def main():
 
     table = per_op_table(br, wl, args.op_reps)
     dom = max((r for r in table), key=lambda r: r["alg_mb"] * (args.layers if r["op"] not in
-                                                               ("softmax_ce", "int8_scale", "int8_quant", "int8_dequant") else 1))
+                                                               ("softmax_ce", "int8_scale", "int8_quant", "int8_dequant", "int8_quantize_dynamic") else 1))
     roofline = dict(bound="hbm", kernel=dom["op"], achieved=dom["gbs"], peak=PEAK_HBM_GBS, unit="GB/s",
                     frac=dom["gbs"] / PEAK_HBM_GBS,
                     traffic=MEASURED_TRAFFIC_BYTES.get(dom["op"]) if (cfg["name"], cfg["batch"], bf16) == ("qwen3-0.6b", 16, False) else None,

@@ -255,6 +255,9 @@ int mi355_minmax_dev(float *out3_dev, const float *x, size_t n);
  * half-to-even (rounding 0) or half away from zero (rounding 1, the reference's); x^ = q*scale. */
 int mi355_int8_scale_dev(float *scale_dev, const float *x, size_t n);
 int mi355_int8_quant_dev(int8_t *q, const float *x, const float *scale_dev, size_t n, int rounding);
+/* The activation path of W8A8 in one call: scale = max|x|/127 (written to scale_dev) and q = quantize(x, scale),
+ * two launches instead of the three of mi355_int8_scale_dev + mi355_int8_quant_dev; same bytes out. */
+int mi355_int8_quantize_dynamic_dev(int8_t *q, float *scale_dev, const float *x, size_t n, int rounding);
 int mi355_int8_dequant_dev(float *x, const int8_t *q, const float *scale_dev, size_t n);
 
 /* Optimizer tail — training/training_dynamic/train.m:748-877 in two sweeps instead of five.

@@ -523,6 +523,25 @@ def test_embed_scatter_add_single_hot_token(br):
     assert dEd.numpy().tobytes() == O.embed_backward(dE0, dx, ids).tobytes()
 
 
+@pytest.mark.parametrize("n", [1024 * 4096, 13, 4099, 3, 1024 * 1024 * 5 + 2])
+@pytest.mark.parametrize("rounding", [0, 1])
+def test_int8_quantize_dynamic_equals_scale_then_quant(br, n, rounding):
+    x = H.normal(72, n) * np.float32(3.0)
+    if n > 8: x[5] = np.float32(-11.0)
+    xd = dev(br, x)
+    s1 = br.DevArray(1); q1 = br.DevArray(n, np.int8)
+    br.check(br.lib.mi355_int8_scale_dev(s1.ptr, xd.ptr, n))
+    br.check(br.lib.mi355_int8_quant_dev(q1.ptr, xd.ptr, s1.ptr, n, rounding))
+    s2 = br.DevArray(1); q2 = br.DevArray(n, np.int8)
+    br.check(br.lib.mi355_int8_quantize_dynamic_dev(q2.ptr, s2.ptr, xd.ptr, n, rounding))
+    assert s2.numpy().tobytes() == s1.numpy().tobytes() and q2.numpy().tobytes() == q1.numpy().tobytes()
+    sc = O.int8_scale(x)
+    assert np.float32(sc) == s2.numpy()[0] and np.array_equal(q2.numpy(), O.int8_quant(x, sc, rounding))
+    z = dev(br, np.zeros(64, np.float32))               # all zeros: scale 1
+    br.check(br.lib.mi355_int8_quantize_dynamic_dev(q2.ptr, s2.ptr, z.ptr, min(n, 64), rounding))
+    assert s2.numpy()[0] == 1.0 and not q2.numpy()[:min(n, 64)].any()
+
+
 @pytest.mark.parametrize("n", [1024 * 4096, 2048 * 256 * 16, 13, 1, 4099])
 def test_minmax_exact(br, n):
     say("minmax n=%d" % n)
