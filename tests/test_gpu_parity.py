@@ -454,6 +454,8 @@ def test_embed_gather_bit_exact(br, V, D, B, S, oob):
     (1000, 32, 2048, 8, 3),       # many short sequences: a block of 64 positions spans eight of them
     (1000, 20, 700, 6, 2),        # ... with S not a multiple of 4
     (50, 3, 1, 257, 5),
+    (20, 12001, 1, 130, 2),       # wide rows: more column chunks than compute units
+    (7, 8192, 1, 600, 0),
 ])
 def test_embed_scatter_add_bit_exact_and_deterministic(br, V, D, B, S, oob):
     say("scatter_add V=%d D=%d B=%d S=%d" % (V, D, B, S))
