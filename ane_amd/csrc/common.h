@@ -27,7 +27,7 @@ struct Mi355Ctx {
     void *ws;          // grow-only workspace
     size_t ws_bytes;
     // tuning knobs (0 = pick per shape)
-    int rms_lpr, rms_threads, ew_unroll, ce_rows, ce_rows2, qk_lpr, qk_threads, gemm_splitk, scatter_tree;
+    int rms_lpr, rms_threads, ew_unroll, ce_rows, ce_rows2, qk_lpr, qk_threads, gemm_splitk, scatter_tree, buf_phase;
 };
 extern Mi355Ctx g_ctx;
 

@@ -140,7 +140,7 @@ MI355_API int mi355_tune_set(const char *key, int value) {
     struct { const char *k; int *v; } tab[] = {
         {"rms_lpr", &g_ctx.rms_lpr}, {"rms_threads", &g_ctx.rms_threads},
         {"ew_unroll", &g_ctx.ew_unroll},
-        {"ce_rows", &g_ctx.ce_rows}, {"ce_rows2", &g_ctx.ce_rows2}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
+        {"ce_rows", &g_ctx.ce_rows}, {"ce_rows2", &g_ctx.ce_rows2}, {"buf_phase", &g_ctx.buf_phase}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
         {"gemm_splitk", &g_ctx.gemm_splitk}, {"scatter_tree", &g_ctx.scatter_tree},
     };
     for (auto &t : tab)
@@ -152,7 +152,8 @@ MI355_API int mi355_tune_set(const char *key, int value) {
 // Buffers
 // ---------------------------------------------------------------------------------------------
 struct mi355_buf {
-    void *dev;
+    void *base;     // what hipMalloc returned
+    void *dev;      // what the caller sees
     size_t bytes;
 };
 
@@ -160,14 +161,26 @@ MI355_API mi355_buf *mi355_buf_alloc(size_t bytes) {
     if (!mi355_ready("buf_alloc")) return nullptr;
     if (bytes == 0) { mi355_fail("buf_alloc: zero bytes"); return nullptr; }
     if (!mi355_outside_capture("buf_alloc")) return nullptr;
+    // Large buffers start at a rotating multiple of 128 bytes within a 1 KiB group.  With S = 256 a row of an
+    // activation is 1 KiB, so a workgroup of a column-reduction kernel, which reads the same 64 bytes of every row,
+    // talks to one eighth of the memory channels, and one of those eighths is markedly slower under that pattern.
+    // Operands that all start on a 2 MiB boundary put their slow strips into the same workgroups; rotated starts
+    // spread them (RMSNorm backward at the Qwen3 shape: 16.1 -> 14.2 us).
+    static unsigned counter = 0;
+    size_t phase = 0;
+    if (bytes >= ((size_t)1 << 20)) {
+        if (g_ctx.buf_phase == 0) phase = (size_t)(counter++ % 8) * 128;
+        else phase = (size_t)((g_ctx.buf_phase - 1) % 8) * 128;
+    }
     void *p = nullptr;
-    hipError_t e = hipMalloc(&p, bytes);
+    hipError_t e = hipMalloc(&p, bytes + phase);
     if (e != hipSuccess) { mi355_fail("buf_alloc(%zu): %s", bytes, hipGetErrorString(e)); return nullptr; }
-    e = hipMemsetAsync(p, 0, bytes, g_ctx.stream);
+    e = hipMemsetAsync(p, 0, bytes + phase, g_ctx.stream);
     if (e != hipSuccess) { (void)hipFree(p); mi355_fail("buf_alloc memset: %s", hipGetErrorString(e)); return nullptr; }
     mi355_buf *b = (mi355_buf *)malloc(sizeof(mi355_buf));
     if (!b) { (void)hipFree(p); return nullptr; }
-    b->dev = p;
+    b->base = p;
+    b->dev = (char *)p + phase;
     b->bytes = bytes;
     return b;
 }
@@ -177,7 +190,7 @@ MI355_API void mi355_buf_free(mi355_buf *b) {
     if (!mi355_outside_capture("buf_free")) return;
     if (g_ctx.ready && b->dev) {
         (void)hipStreamSynchronize(g_ctx.stream);
-        (void)hipFree(b->dev);
+        (void)hipFree(b->base);
     }
     free(b);
 }

@@ -672,6 +672,10 @@ def main():
     ap.add_argument("--fuse", action="store_true",
                     help="run each residual and the RMSNorm after it as one launch (mi355_residual_rmsnorm_fwd_dev)")
     ap.add_argument("--op-reps", type=int, default=3)
+    ap.add_argument("--buf-phase", type=int, default=0,
+                    help="start of large buffers within a 1 KiB group: 0 = the library's default (a multiple of 128 bytes "
+                         "that rotates from one allocation to the next), 1..8 = always (value-1)*128 bytes (1: every "
+                         "buffer on a 2 MiB boundary, as plain hipMalloc gives)")
     ap.add_argument("--storage", default="f32", choices=["f32", "bf16"],
                     help="activation storage: f32 (the reference's, default) or the optional bf16 variants "
                          "(arithmetic stays f32; parity bound 5e-3 instead of 1e-5)")
@@ -690,6 +694,7 @@ def main():
 
     import ane_amd.bridge as br
     br.init()
+    br.tune("buf_phase", args.buf_phase)
     dev_name, drv_peak, cus = br.device_info()
     if args.workload == "embed":
         return bench_embed(br, args)
@@ -763,6 +768,8 @@ def main():
                    "residual_fused_into_next_rmsnorm": wl.fuse, "replayed_as_graph": bool(args.graph),
                    "activation_storage": args.storage,
                    "operands": "warm: one buffer set shared by all layers" if args.share_buffers else "cold: one buffer set per layer",
+                   "buffer_start_within_1KiB": ("rotating multiple of 128 B (mi355_buf_alloc default)" if args.buf_phase == 0
+                                                else "%d B" % (((args.buf_phase - 1) % 8) * 128)),
                    "weight_gradients": "reduced per op" if args.immediate_dw else "queued, reduced once per step"},
         "aggregate_gbs": total_bytes / ms / 1e6, "aggregate_frac_of_peak": total_bytes / ms / 1e6 / PEAK_HBM_GBS,
         "host_wall_ms_per_step": wall_ms,

@@ -59,7 +59,8 @@ size_t mi355_workspace_size(void);
  * "gemm_splitk" (K slices of mi355_sgemm_dev; 1 = never split),
  * "scatter_tree" (1: mi355_embed_scatter_add_dev sums long segments by a fixed tree instead of the reference's
  * sequential order: still deterministic and within 1e-5 of each row's scale, faster, no longer bit-identical to
- * the CPU loop). */
+ * the CPU loop), "buf_phase" (where mi355_buf_alloc starts buffers of 1 MiB and more within a 1 KiB group:
+ * 0 = a multiple of 128 bytes that rotates from one allocation to the next, 1..8 = always (value-1)*128). */
 int mi355_tune_set(const char *key, int value);
 
 /* ------------------------------------------------------------------------------------------
@@ -69,6 +70,8 @@ int mi355_tune_set(const char *key, int value);
  * ---------------------------------------------------------------------------------------- */
 typedef struct mi355_buf mi355_buf;
 
+/* The device address is 128-byte aligned (see "buf_phase" above: buffers that one op reads together should not
+ * all start at the same offset within 1 KiB, and by default they do not). */
 mi355_buf *mi355_buf_alloc(size_t bytes);                 /* NULL on failure; contents zeroed */
 void mi355_buf_free(mi355_buf *b);                        /* NULL-safe */
 void *mi355_buf_devptr(mi355_buf *b);                     /* raw device address (NULL if b NULL) */
