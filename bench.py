@@ -672,6 +672,8 @@ def main():
     ap.add_argument("--fuse", action="store_true",
                     help="run each residual and the RMSNorm after it as one launch (mi355_residual_rmsnorm_fwd_dev)")
     ap.add_argument("--op-reps", type=int, default=3)
+    ap.add_argument("--tune", action="append", default=[], metavar="KNOB=VALUE",
+                    help="set a tuning knob of the library (mi355_tune_set) before the run; repeatable")
     ap.add_argument("--buf-phase", type=int, default=0,
                     help="start of large buffers within a 1 KiB group: 0 = the library's default (a multiple of 128 bytes "
                          "that rotates from one allocation to the next), 1..8 = always (value-1)*128 bytes (1: every "
@@ -695,6 +697,9 @@ def main():
     import ane_amd.bridge as br
     br.init()
     br.tune("buf_phase", args.buf_phase)
+    for kv in args.tune:
+        k, _, v = kv.partition("=")
+        br.tune(k, int(v))
     dev_name, drv_peak, cus = br.device_info()
     if args.workload == "embed":
         return bench_embed(br, args)
