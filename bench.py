@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-One "step" = one pass of the Qwen3-0.6B full-step fused-op sweep (BASELINE config 4) over one
+One "step" = one pass of the Qwen3-0.6B full-step fused-op sweep (BASELINE.json config 4) over one
 synthetic batch of 16 x 256 tokens, fp32, channel-first:
     forward, layers 0..27 : rmsnorm(att) -> qknorm+rope -> residual -> rmsnorm(ffn) -> swiglu -> residual
                             (--fuse runs each residual and the RMSNorm that consumes its result as ONE launch,
@@ -36,7 +36,7 @@ MEASURED_TRAFFIC_BYTES = {"swiglu_bwd": 251.56e6}
 Q3 = dict(C=1024, H=3072, heads=16, kv_heads=8, hd=128, S=256, batch=16, layers=28, V=151936, theta=1e6,
           int8_shape=(1024, 4096), qk_norm=True, name="qwen3-0.6b")
 # Stories110M (training/training_dynamic/models/stories110m.h:6-16): one sequence per step as the reference
-# runs it, RoPE theta 10000, no QK-norm (BASELINE configs 0 and 1)
+# runs it, RoPE theta 10000, no QK-norm (BASELINE.json configs 0 and 1)
 S110 = dict(C=768, H=2048, heads=12, kv_heads=12, hd=64, S=256, batch=1, layers=12, V=32000, theta=1e4,
             int8_shape=(1024, 4096), qk_norm=False, name="stories110m")
 
@@ -151,7 +151,7 @@ class Workload:
         self.scratch_h = A((B, H, S))          # output of the copy-shaped calibration op only
         self.scratch_c = A((B, C, S))          # the scaled copy of the fused backward's timing run
         self.cos, self.sin = br.rope_tables_dev(S, cfg["hd"], cfg["theta"])
-        # training/training_dynamic/train.m:188; BASELINE config 1 asks for (2*12)^0.25 at the Stories110M shape
+        # training/training_dynamic/train.m:188; BASELINE.json config 1 asks for (2*12)^0.25 at the Stories110M shape
         self.alpha = float(np.float32((2.0 * 12) ** 0.25 if not cfg["qk_norm"] else 1.0 / np.sqrt(2.0 * cfg["layers"])))
         br.sync()
 
@@ -402,7 +402,7 @@ def zipf_ids(seed, n, vocab, s=1.1):
 
 
 def bench_embed(br, args):
-    """BASELINE config 2: vocab 32000 x dim 768 table, 64 sequences x 256 Zipf(1.1) ids; gather + ordered scatter-add."""
+    """BASELINE.json config 2: vocab 32000 x dim 768 table, 64 sequences x 256 Zipf(1.1) ids; gather + ordered scatter-add."""
     V, D, B, S = 32000, 768, 64, 256
     N = B * S
     ids = zipf_ids(0, N, V).reshape(B, S)
@@ -441,7 +441,7 @@ def bench_embed(br, args):
     t_c = time_region(br, copy, args.steps) / nbuf
     b_g = 8 * D * N + 4 * N
     b_s = 4 * D * N + 8 * D * U + 4 * N
-    out = {"metric": "embedding gather + ordered scatter-add (BASELINE config 2)", "value": N / ((t_g + t_s) / 1e3),
+    out = {"metric": "embedding gather + ordered scatter-add (BASELINE.json config 2)", "value": N / ((t_g + t_s) / 1e3),
            "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": t_g + t_s,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32+i32", "data": "synthetic",
            "config": {"workload": "embedding table [32000,768] fp32, 64x256 Zipf(1.1) ids, seed 0", "unique_ids": U,
@@ -687,8 +687,8 @@ def main():
                     help="record one step as a graph and time its replays (pays off where the step is launch-bound)")
     ap.add_argument("--workload", default="qwen3", choices=["qwen3", "stories110m", "embed", "optimizer", "aux", "host"],
                     help="qwen3 = the headline sweep (default); stories110m = the same sweep at the Stories110M shape "
-                         "(BASELINE configs 0/1: one [C,256] sequence per op, 12 layers, RoPE without QK-norm); "
-                         "embed = BASELINE config 2; optimizer = the Adam tail (each prints its own JSON line)")
+                         "(BASELINE.json configs 0/1: one [C,256] sequence per op, 12 layers, RoPE without QK-norm); "
+                         "embed = BASELINE.json config 2; optimizer = the Adam tail (each prints its own JSON line)")
     ap.add_argument("--batch", type=int, default=0, help="sequences per op (default: 16 for qwen3, 1 for stories110m)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -765,8 +765,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "%s full-step fused-op sweep%s: %d layers x 10 ops (batch %d x S %d, C %d, H %d, %d/%d "
                                "heads x %d, %s) + softmax-CE [%d,%d] + INT8 [1024,4096]" % (
-                                   cfg["name"], " (BASELINE config 4)" if cfg["name"] == "qwen3-0.6b" else
-                                   " (BASELINE configs 0/1 shapes)", args.layers, cfg["batch"], cfg["S"], cfg["C"],
+                                   cfg["name"], " (BASELINE.json config 4)" if cfg["name"] == "qwen3-0.6b" else
+                                   " (BASELINE.json configs 0/1 shapes)", args.layers, cfg["batch"], cfg["S"], cfg["C"],
                                    cfg["H"], cfg["heads"], cfg["kv_heads"], cfg["hd"],
                                    "QK-norm + RoPE" if cfg["qk_norm"] else "RoPE", cfg["V"], cfg["S"]),
                    "layers": args.layers, "tokens_per_step": tokens, "alg_gb_per_step": total_bytes / 1e9,

@@ -29,7 +29,7 @@ def say(msg):
 # RMSNorm
 # ---------------------------------------------------------------------------------------------
 RMS_SHAPES = [
-    (1, 768, 256),      # BASELINE config 0
+    (1, 768, 256),      # BASELINE.json config 0
     (16, 1024, 256),    # Qwen3-0.6B layer shape
     (3, 48, 20),        # golden-sized, S % 4 == 0 but narrow
     (2, 100, 37),       # S % 4 != 0 -> scalar columns
@@ -275,7 +275,7 @@ def test_axpby_bit_exact(br, n):
 # RoPE
 # ---------------------------------------------------------------------------------------------
 ROPE_CASES = [
-    (1, 12, 12, 64, 256, 10000.0),    # Stories110M, BASELINE config 1
+    (1, 12, 12, 64, 256, 10000.0),    # Stories110M, BASELINE.json config 1
     (16, 16, 8, 128, 256, 1e6),       # Qwen3-0.6B, GQA 16/8
     (2, 3, 1, 8, 10, 10000.0),        # S % 4 != 0
     (1, 4, 0, 16, 8, 1e6),            # Q only
@@ -417,7 +417,7 @@ def _embed_case(seed, V, D, B, S, oob=0):
 
 
 @pytest.mark.parametrize("V,D,B,S,oob", [
-    (32000, 768, 64, 256, 0),     # BASELINE config 2
+    (32000, 768, 64, 256, 0),     # BASELINE.json config 2
     (500, 50, 3, 37, 4),          # ragged D and S, out-of-range ids
     (70, 4, 1, 1, 0),
     (1000, 1024, 2, 256, 2),
@@ -438,7 +438,7 @@ def test_embed_gather_bit_exact(br, V, D, B, S, oob):
 
 
 @pytest.mark.parametrize("V,D,B,S,oob", [
-    (32000, 768, 64, 256, 0),     # BASELINE config 2: Zipf(1.1), heavy duplicates
+    (32000, 768, 64, 256, 0),     # BASELINE.json config 2: Zipf(1.1), heavy duplicates
     (500, 50, 3, 37, 4),
     (64, 768, 8, 256, 0),         # tiny vocabulary: every segment is long
     (70, 4, 1, 1, 0),
