@@ -91,6 +91,9 @@ SIGNATURES = {
     "mi355_adam_update_dev": (_i, [_p, _p, _p, _p, _z, _i, _f, _f, _f, _f, _f, _f, _p, _i]),
     "mi355_sumsq_accum_multi_dev": (_i, [_p, _p, _p, _i, _f]),
     "mi355_adam_update_multi_dev": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _f, _f, _f, _f, _f, _p, _i]),
+    "mi355_rmsnorm_tile": (_i, [_i, _i, _i, _i, _i, _p]),
+    "mi355_softmax_cols_dev": (_i, [_p, _p, _i, _i]),
+    "mi355_nll_from_probs_dev": (_i, [_p, _p, _p, _p, _i, _i]),
     "mi355_vocab_map_build_dev": (_i, [_p, _p, _p, _p, _z, _i]),
     "mi355_vocab_remap_dev": (_i, [_p, _p, _p, _z, _i]),
     "mi355_vocab_compact_embed_dev": (_i, [_p, _p, _p, _i, _i, _i]),
@@ -125,6 +128,10 @@ SIGNATURES = {
     "mi355_cvt_f16_f32_dev": (_i, [_p, _z, _p, _z, _z, _z]),
     "mi355_attn_grads_finish_dev": (_i, [_p, _p, _p, _p, _p, _p, _i, _z, _z, _z, _i, _i, _i, _i, _i, _p, _p]),
     "mi355_adam_update": (None, [_p, _p, _p, _p, _z, _i, _f, _f, _f, _f, _f]),
+    "mi355_vocab_map_build": (_i, [_p, _p, _p, _z, _i]),
+    "mi355_vocab_compact_embed": (None, [_p, _p, _p, _i, _i, _i]),
+    "mi355_vocab_scatter_grads": (None, [_p, _p, _p, _i, _i, _i]),
+    "mi355_vocab_update_full": (None, [_p, _p, _p, _i, _i, _i]),
     "mi355_rmsnorm": (None, [_p, _p, _p, _i, _i]),
     "mi355_rmsnorm_bwd": (None, [_p, _p, _p, _p, _p, _i, _i]),
     "mi355_cross_entropy_loss": (_f, [_p, _p, _p, _i, _i]),

@@ -146,7 +146,7 @@ MI355_API int mi355_ckpt_create(const char *path, const mi355_ckpt_hdr *hdr) {
 }
 
 MI355_API int mi355_ckpt_load_dev(const char *path, uint64_t byte_offset, float *dst_dev, uint64_t count) {
-    if (!mi355_ready("ckpt_load")) return -1;
+    if (!mi355_ready("ckpt_load") || !mi355_outside_capture("ckpt_load")) return -1;
     if (!path || !dst_dev) return mi355_fail("ckpt_load: NULL argument");
     char *buf = (char *)stage();
     if (!buf) return -1;
@@ -178,7 +178,7 @@ MI355_API int mi355_ckpt_load_dev(const char *path, uint64_t byte_offset, float 
 }
 
 MI355_API int mi355_ckpt_store_dev(const char *path, uint64_t byte_offset, const float *src_dev, uint64_t count) {
-    if (!mi355_ready("ckpt_store")) return -1;
+    if (!mi355_ready("ckpt_store") || !mi355_outside_capture("ckpt_store")) return -1;
     if (!path || !src_dev) return mi355_fail("ckpt_store: NULL argument");
     char *buf = (char *)stage();
     if (!buf) return -1;

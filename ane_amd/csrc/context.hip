@@ -116,6 +116,9 @@ MI355_API int mi355_set_stream(void *hip_stream) {
     if (!mi355_ready("set_stream")) return -1;
     if (!mi355_outside_capture("set_stream")) return -1;
     if (mi355_dw_flush()) return -1;        // queued reductions belong to the old stream
+    // Workspaces are shared by the ops of every stream and are freed behind a wait on the CURRENT stream only:
+    // nothing may still be running on the stream that is left behind.
+    HIP_OK(hipStreamSynchronize(g_ctx.stream));
     g_ctx.stream = (hipStream_t)hip_stream;
     return 0;
 }

@@ -342,6 +342,17 @@ struct NormCfg {
     int vec, lpr, threads, cap;
 };
 
+// The tiles that are instantiated (NORM_DISPATCH below has one case per entry): vec*1000000 + lpr*10000 + (threads/256)*100 + cap.
+constexpr int NORM_KEYS[] = {1640100, 4160100, 4160108, 4160116, 4160200, 4160208, 4160216, 4160400, 4160408,
+                             4080100, 4080108, 4080116, 4080200, 4080208, 4080216, 4080400, 4080408,
+                             4040100, 4040108, 4040116, 4040200, 4040208, 4040216, 4040400, 4040408};
+int norm_key(const NormCfg &c) { return c.vec * 1000000 + c.lpr * 10000 + (c.threads / 256) * 100 + c.cap; }
+bool norm_tile_exists(const NormCfg &c) {
+    for (int k : NORM_KEYS)
+        if (k == norm_key(c)) return true;
+    return false;
+}
+
 // Picks the tile: registers when the rows fit, and the narrowest strip needed to give every
 // compute unit at least two workgroups.
 NormCfg pick_cfg(int C, int S, int batch, bool vec_ok, int max_cap, int max_cap_1024, int lpr_knob, int thr_knob,
@@ -374,6 +385,7 @@ NormCfg pick_cfg(int C, int S, int batch, bool vec_ok, int max_cap, int max_cap_
             for (int cp : caps)
                 if (cp <= max_cap && (long)cp * rps >= C) { cap = cp; break; }
             if (thr == 1024 && cap > max_cap_1024) cap = 0;   // 16 waves per CU leave 128 VGPRs per lane
+            if (!norm_tile_exists(NormCfg{4, lpr, thr, cap})) continue;
             const long strips = ceil_div((size_t)S, (size_t)lpr * 4);
             const long nblk = strips * batch;
             long score = (cap > 0 ? 1000000 : 0);
@@ -414,14 +426,27 @@ void launch_bwd_res(float *dx, float *part, const float *dy, const float *x, con
                        dy, x, w, C, S, strips, nblk, eps, 1.0f / (float)C, variant, res, dx2, alpha2);
 }
 
+// The tile each entry point uses: op 0 = forward, 1 = backward, 2 = backward with the residual.
+NormCfg plan_tile(int op, int C, int S, int batch, bool vec_ok) {
+    if (op == 0) return pick_cfg(C, S, batch, vec_ok, 16, 8, g_ctx.rms_lpr, g_ctx.rms_threads, false);
+    if (op == 1) return pick_cfg(C, S, batch, vec_ok, 16, 0, g_ctx.rms_lpr, g_ctx.rms_threads, true);
+    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 8, 0, g_ctx.rms_lpr, g_ctx.rms_threads, true);
+    // three operands of 16 rows per lane do not fit the registers: the 8-row tile, or the two-sweep variant
+    if (cfg.cap > 8) cfg = C <= 1024 ? NormCfg{4, 4, 512, 8} : NormCfg{cfg.vec, cfg.lpr, cfg.threads, 0};
+    return cfg;
+}
+
 #define NORM_DISPATCH(FN, cfg, ...)                                                                   \
     do {                                                                                              \
-        const int key = (cfg).vec * 1000000 + (cfg).lpr * 10000 + ((cfg).threads / 256) * 100 + (cfg).cap; \
+        const int key = norm_key(cfg);                                                                \
         switch (key) {                                                                                \
             case 1640100: FN<1, 64, 256, 0>(__VA_ARGS__); break;                                      \
             case 4160100: FN<4, 16, 256, 0>(__VA_ARGS__); break;                                      \
             case 4160108: FN<4, 16, 256, 8>(__VA_ARGS__); break;                                      \
             case 4160116: FN<4, 16, 256, 16>(__VA_ARGS__); break;                                     \
+            case 4160200: FN<4, 16, 512, 0>(__VA_ARGS__); break;                                      \
+            case 4160208: FN<4, 16, 512, 8>(__VA_ARGS__); break;                                      \
+            case 4160216: FN<4, 16, 512, 16>(__VA_ARGS__); break;                                     \
             case 4160400: FN<4, 16, 1024, 0>(__VA_ARGS__); break;                                     \
             case 4160408: FN<4, 16, 1024, 8>(__VA_ARGS__); break;                                     \
             case 4040208: FN<4, 4, 512, 8>(__VA_ARGS__); break;                                       \
@@ -446,12 +471,21 @@ void launch_bwd_res(float *dx, float *part, const float *dy, const float *x, con
 
 }   // namespace
 
+// Host-only: which tile an entry point would run for a shape, and whether that tile exists.
+MI355_API int mi355_rmsnorm_tile(int op, int C, int S, int batch, int aligned, int *tile4) {
+    if (op < 0 || op > 2 || C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_tile: bad arguments");
+    const NormCfg cfg = plan_tile(op, C, S, batch, aligned && S % 4 == 0);
+    if (tile4) { tile4[0] = cfg.vec; tile4[1] = cfg.lpr; tile4[2] = cfg.threads; tile4[3] = cfg.cap; }
+    if (!norm_tile_exists(cfg)) return mi355_fail("rmsnorm: no kernel for tile key %d", norm_key(cfg));
+    return 0;
+}
+
 MI355_API int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, int C, int S, int batch, float eps) {
     if (!mi355_ready("rmsnorm_fwd")) return -1;
     if (!y || !x || !w) return mi355_fail("rmsnorm_fwd: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_fwd: bad shape C=%d S=%d batch=%d", C, S, batch);
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(y);
-    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 16, 8, g_ctx.rms_lpr, g_ctx.rms_threads, false);
+    NormCfg cfg = plan_tile(0, C, S, batch, vec_ok);
     NORM_DISPATCH(launch_fwd, cfg, y, x, w, C, S, batch, eps);
     LAUNCH_OK("rmsnorm_fwd");
     return 0;
@@ -464,7 +498,7 @@ MI355_API int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_bwd: bad shape C=%d S=%d batch=%d", C, S, batch);
     if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd: variant must be 0 or 1");
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(dy) && aligned16(dx);
-    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 16, 0, g_ctx.rms_lpr, g_ctx.rms_threads, true);
+    NormCfg cfg = plan_tile(1, C, S, batch, vec_ok);
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
     float *part = mi355_dw_partials((size_t)nblk * C, dw, nullptr);
@@ -487,9 +521,7 @@ MI355_API int mi355_rmsnorm_bwd_residual_dev(float *dx, float *dx_scaled, float 
         return mi355_fail("rmsnorm_bwd_residual: dx_scaled must not alias another operand");
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(res) &&
                         (!dx_scaled || aligned16(dx_scaled));
-    NormCfg cfg = pick_cfg(C, S, batch, vec_ok, 8, 0, g_ctx.rms_lpr, g_ctx.rms_threads, true);
-    // three operands of 16 rows per lane do not fit the registers: the 8-row tile, or the two-sweep variant
-    if (cfg.cap > 8) cfg = C <= 1024 ? NormCfg{4, 4, 512, 8} : NormCfg{cfg.vec, cfg.lpr, cfg.threads, 0};
+    NormCfg cfg = plan_tile(2, C, S, batch, vec_ok);
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
     float *part = mi355_dw_partials((size_t)nblk * C, dw, nullptr);

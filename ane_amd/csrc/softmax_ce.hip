@@ -161,7 +161,8 @@ __global__ __launch_bounds__(CE_THREADS) void ce_partial_kernel(float *__restric
 // rounds of loads per thread, S/16 workgroups in flight), then the 64 partial results are merged by a fixed
 // tree.  The merge of two (max, sum) pairs is the online-softmax rescaling.
 constexpr int CB_COLS = 16, CB_GROUPS = 1024 / CB_COLS;
-template <typename T>
+// PLAIN: the stand-alone column softmax; there are no targets, and colInv receives the sum itself (that op divides).
+template <typename T, bool PLAIN = false>
 __global__ __launch_bounds__(1024) void ce_combine_kernel(float *__restrict__ colM, float *__restrict__ colInv,
                                                           float *__restrict__ colLoss, const float *__restrict__ pm,
                                                           const float *__restrict__ pl,
@@ -206,8 +207,12 @@ __global__ __launch_bounds__(1024) void ce_combine_kernel(float *__restrict__ co
     }
     if (g == 0 && t < S) {
         const float M = sm[0][cl];
-        const float inv = 1.0f / sl[0][cl];
         colM[t] = M;
+        if constexpr (PLAIN) {
+            colInv[t] = sl[0][cl];
+            return;
+        }
+        const float inv = 1.0f / sl[0][cl];
         colInv[t] = inv;
         const int tgt = targets[t];
         float loss = 0.f;
@@ -281,6 +286,68 @@ __global__ __launch_bounds__(CE_THREADS) void ce_grad_kernel(T *dlogits, const T
             }
         }
     }
+}
+
+// probs = exp(l - M) / L: the second pass of the stand-alone column softmax (training/train_large_ane.m:508-516)
+template <int VEC>
+__global__ __launch_bounds__(CE_THREADS) void softmax_out_kernel(float *probs, const float *logits,
+                                                                 const float *__restrict__ colM,
+                                                                 const float *__restrict__ colL, int V, int S,
+                                                                 int rows_per_block) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = (blockIdx.y * 64 + lane) * VEC;
+    if (col >= S) return;
+    const int rb = gridDim.x - 1 - blockIdx.x;
+    const int v_lo = rb * rows_per_block;
+    const int v_hi = min(V, v_lo + rows_per_block);
+    float M[VEC], L[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) { M[j] = colM[col + j]; L[j] = colL[col + j]; }
+    for (int v = v_lo + wave; v < v_hi; v += CE_WAVES) {
+        float x[VEC], o[VEC];
+        ld_cols_nt<VEC>(x, logits + (size_t)v * S + col);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) o[j] = exp_neg(x[j] - M[j]) / L[j];
+        st_cols<VEC>(probs + (size_t)v * S + col, o);
+    }
+}
+
+// NLL on given probabilities (training/train_large_ane.m:519-530).  The loss is formed first, by one workgroup and
+// a fixed tree, so that the gradient pass may overwrite the probabilities in place.
+__global__ __launch_bounds__(CE_THREADS) void nll_loss_kernel(float *__restrict__ loss_out, const float *__restrict__ probs,
+                                                              const int32_t *__restrict__ targets, int V, int S) {
+    __shared__ float red[CE_THREADS];
+    float sl = 0.f;
+    for (int t = threadIdx.x; t < S; t += CE_THREADS) {
+        const int tg = targets[t];
+        if (tg >= 0 && tg < V) sl -= logf(probs[(size_t)tg * S + t] + 1e-10f);
+    }
+    red[threadIdx.x] = sl;
+    __syncthreads();
+    for (int off = CE_THREADS / 2; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) red[threadIdx.x] += red[threadIdx.x + off];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *loss_out = red[0] / (float)S;
+}
+
+// dlogits = (probs - onehot) * (1/S), one 128-bit access per lane; n4 = V*S/4 when VEC = 4
+template <int VEC>
+__global__ __launch_bounds__(256) void nll_grad_kernel(float *dlogits, const float *probs,
+                                                       const int32_t *__restrict__ targets, int V, int S, size_t n,
+                                                       float invS) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+    if (i >= n) return;
+    const int v = (int)(i / (size_t)S), t0 = (int)(i - (size_t)v * S);
+    float x[VEC], o[VEC];
+    ld_cols_nt<VEC>(x, probs + i);
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        float p = x[j];
+        if (targets[t0 + j] == v) p -= 1.0f;
+        o[j] = p * invS;
+    }
+    st_cols<VEC>(dlogits + i, o);
 }
 
 // resident workgroups of the second pass per compute unit (asked of the runtime once per storage type)
@@ -371,6 +438,54 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
 }
 
 }   // namespace
+
+MI355_API int mi355_softmax_cols_dev(float *probs, const float *logits, int V, int S) {
+    if (!mi355_ready("softmax_cols")) return -1;
+    if (!probs || !logits) return mi355_fail("softmax_cols: NULL pointer");
+    if (V <= 0 || S <= 0) return mi355_fail("softmax_cols: bad shape V=%d S=%d", V, S);
+    const int rpb = 4 * CE_TILE_ROWS;
+    const int nblk = (int)ceil_div((size_t)V, (size_t)rpb);
+    const bool vec_ok = (S % 4 == 0) && aligned16(logits) && aligned16(probs);
+    const int vec = vec_ok ? 4 : 1;
+    const int strips = (int)ceil_div((size_t)S, (size_t)64 * vec);
+    if (strips > 65535) return mi355_fail("softmax_cols: S too large");
+    auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const size_t part_b = al((size_t)nblk * S * sizeof(float)), col_b = al((size_t)S * sizeof(float));
+    char *ws = (char *)mi355_ws(2 * part_b + 2 * col_b);
+    if (!ws) return -1;
+    float *pm = (float *)ws, *pl = (float *)(ws + part_b);
+    float *colM = (float *)(ws + 2 * part_b), *colL = (float *)(ws + 2 * part_b + col_b);
+    const dim3 grid((unsigned)nblk, (unsigned)strips);
+    if (vec_ok) hipLaunchKernelGGL((ce_partial_kernel<4, float>), grid, dim3(CE_THREADS), 0, g_ctx.stream, pm, pl, logits, V, S, rpb);
+    else hipLaunchKernelGGL((ce_partial_kernel<1, float>), grid, dim3(CE_THREADS), 0, g_ctx.stream, pm, pl, logits, V, S, rpb);
+    LAUNCH_OK("softmax_cols partial");
+    hipLaunchKernelGGL((ce_combine_kernel<float, true>), dim3((unsigned)ceil_div((size_t)S, CB_COLS)), dim3(1024), 0,
+                       g_ctx.stream, colM, colL, nullptr, pm, pl, logits, nullptr, V, S, nblk);
+    LAUNCH_OK("softmax_cols combine");
+    if (vec_ok) hipLaunchKernelGGL(softmax_out_kernel<4>, grid, dim3(CE_THREADS), 0, g_ctx.stream, probs, logits, colM, colL, V, S, rpb);
+    else hipLaunchKernelGGL(softmax_out_kernel<1>, grid, dim3(CE_THREADS), 0, g_ctx.stream, probs, logits, colM, colL, V, S, rpb);
+    LAUNCH_OK("softmax_cols out");
+    return 0;
+}
+
+MI355_API int mi355_nll_from_probs_dev(float *dlogits, float *loss_dev, const float *probs, const int32_t *targets, int V,
+                                       int S) {
+    if (!mi355_ready("nll_from_probs")) return -1;
+    if (!dlogits || !loss_dev || !probs || !targets) return mi355_fail("nll_from_probs: NULL pointer");
+    if (V <= 0 || S <= 0) return mi355_fail("nll_from_probs: bad shape V=%d S=%d", V, S);
+    const size_t n = (size_t)V * S;
+    hipLaunchKernelGGL(nll_loss_kernel, dim3(1), dim3(CE_THREADS), 0, g_ctx.stream, loss_dev, probs, targets, V, S);
+    LAUNCH_OK("nll_from_probs loss");
+    const bool vec_ok = (S % 4 == 0) && aligned16(probs) && aligned16(dlogits);
+    if (vec_ok)
+        hipLaunchKernelGGL(nll_grad_kernel<4>, dim3((unsigned)ceil_div(n / 4, 256)), dim3(256), 0, g_ctx.stream, dlogits,
+                           probs, targets, V, S, n, 1.0f / (float)S);
+    else
+        hipLaunchKernelGGL(nll_grad_kernel<1>, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, g_ctx.stream, dlogits, probs,
+                           targets, V, S, n, 1.0f / (float)S);
+    LAUNCH_OK("nll_from_probs grad");
+    return 0;
+}
 
 MI355_API int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float *logits, const int32_t *targets, int V,
                                    int S, float grad_scale) {

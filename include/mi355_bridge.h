@@ -152,6 +152,13 @@ int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, int C, int S
 int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const float *x, const float *w,
                           int C, int S, int batch, float eps, int variant);
 
+/* Introspection, host-only (needs no GPU): the register tile that the RMSNorm entry points choose for a shape —
+ * op 0 = mi355_rmsnorm_fwd_dev, 1 = mi355_rmsnorm_bwd_dev, 2 = mi355_rmsnorm_bwd_residual_dev; aligned != 0 means
+ * 16-byte aligned tensors.  tile4 (may be NULL) receives {columns per lane, lanes per row segment, threads per
+ * workgroup, rows per lane held in registers (0 = rows are read twice)}.  0, or -1 if no kernel exists for the
+ * choice (a defect: the entry point would fail the same way). */
+int mi355_rmsnorm_tile(int op, int C, int S, int batch, int aligned, int *tile4);
+
 /* Weight-gradient accumulation mode.  By default dw / dwq / dwk are up to date (in stream order) when
  * the backward call that adds into them returns.  The loops read these gradients only at the optimizer
  * step, after the whole backward pass (training/training_dynamic/train.m:748-869); with
@@ -246,6 +253,17 @@ int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, 
  * (stories_cpu_ops.h:98).  dlogits may alias logits. */
 int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float *logits,
                          const int32_t *targets, int V, int S, float grad_scale);
+
+/* The two halves of that op as the static loop with ANE extras runs them when the classifier stays on the CPU
+ * (training/train_large_ane.m:499-530).
+ * mi355_softmax_cols_dev: probs[v][t] = exp(logits[v][t] - max_v) / sum_v exp(...), per column t — the scalar loop of
+ * train_large_ane.m:508-516 (which divides by the sum).  probs may alias logits.
+ * mi355_nll_from_probs_dev: *loss_dev = mean_t -logf(probs[tgt_t][t] + 1e-10f); dlogits = (probs - onehot) * (1/S) —
+ * train_large_ane.m:519-530.  The reference indexes with the target unchecked; here a target outside [0,V) adds no
+ * loss term and no one-hot (its column is still scaled by 1/S).  dlogits may alias probs. */
+int mi355_softmax_cols_dev(float *probs, const float *logits, int V, int S);
+int mi355_nll_from_probs_dev(float *dlogits, float *loss_dev, const float *probs, const int32_t *targets, int V,
+                             int S);
 
 /* Range diagnostics of the loops: out3_dev = {min x, max x, max |x|}.  Replaces vDSP_minv / vDSP_maxv /
  * vDSP_maxmgv — training/training_dynamic/train.m:664-666 (dq, dk, dv magnitudes) and :738-742 (range of x and
@@ -392,7 +410,9 @@ float mi355_cross_entropy_loss(float *dlogits, const float *logits, const uint16
                                int S);
 /* embed_lookup — training/stories_cpu_ops.h:112.  The reference reads the vocabulary size from the
  * compile-time VOCAB macro; it is an argument here.  The table is kept resident on the device, keyed
- * by its host address, and re-uploaded after mi355_host_table_invalidate(embed). */
+ * by its host address.  It is uploaded again after any host-pointer call of this library has written into
+ * that host array (mi355_adam_update on the table, as training/training_dynamic/train.m:869 does) and after
+ * mi355_host_table_invalidate(embed), which is for callers that change the array with code of their own. */
 void mi355_embed_lookup(float *x, const float *embed, const uint16_t *tokens, int vocab, int dim,
                         int seq);
 void mi355_host_table_invalidate(const float *embed);
@@ -411,6 +431,25 @@ void mi355_axpby(float *y, const float *a, const float *b, float alpha, size_t n
 /* adam_update — training/training_dynamic/cpu_ops.h:56 with the AdamState fields spelled out */
 void mi355_adam_update(float *w, const float *g, float *m, float *v, size_t n, int t, float lr, float b1,
                        float b2, float eps, float wd);
+
+/* Vocabulary compaction on host arrays — training/training_dynamic/cpu_ops.h:96-148, with the VocabMap fields
+ * and the size of the full table spelled out (include/mi355_cpu_ops.h wraps them in the reference's own
+ * names and struct).  The maps are caller-allocated: full_to_compact [full_vocab]; compact_to_full with room for
+ * full_vocab entries, of which the first compact_vocab are written.  mi355_vocab_map_build returns compact_vocab
+ * (-1 on failure); tokens >= full_vocab in the data are ignored.  compact_embed and update_full keep the full
+ * table resident on the device, keyed by its host address, like mi355_embed_lookup (and update_full keeps that
+ * copy current).  Map entries outside [0, full_vocab) are skipped. */
+int mi355_vocab_map_build(int *full_to_compact, int *compact_to_full, const uint16_t *data, size_t n_tokens,
+                          int full_vocab);
+/* vocab_compact_embed — cpu_ops.h:127-132: compact[c] = full_embed[compact_to_full[c]] */
+void mi355_vocab_compact_embed(float *compact, const float *full_embed, const int *compact_to_full, int compact_vocab,
+                               int full_vocab, int dim);
+/* vocab_scatter_grads — cpu_ops.h:135-142: full_gembed[compact_to_full[c]] += compact_gembed[c] */
+void mi355_vocab_scatter_grads(float *full_gembed, const float *compact_gembed, const int *compact_to_full,
+                               int compact_vocab, int full_vocab, int dim);
+/* vocab_update_full — cpu_ops.h:145-148: full_embed[compact_to_full[c]] = compact_embed[c] */
+void mi355_vocab_update_full(float *full_embed, const float *compact_embed, const int *compact_to_full,
+                             int compact_vocab, int full_vocab, int dim);
 
 #ifdef __cplusplus
 }

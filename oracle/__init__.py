@@ -51,6 +51,8 @@ def _load():
         "orc_embed_lookup": (C.c_int, [_f32p, _f32p, _i32p, C.c_int, C.c_int, C.c_int]),
         "orc_embed_backward": (None, [_f32p, _f32p, _i32p, C.c_int, C.c_int, C.c_int]),
         "orc_cross_entropy": (C.c_float, [_f32p, _f32p, _i32p, C.c_int, C.c_int, C.c_float]),
+        "orc_softmax_cols": (None, [_f32p, _f32p, C.c_int, C.c_int]),
+        "orc_nll_from_probs": (C.c_float, [_f32p, _f32p, _i32p, C.c_int, C.c_int]),
         "orc_minmax": (None, [_f32p, _f32p, C.c_size_t]),
         "orc_int8_scale": (C.c_float, [_f32p, C.c_size_t]),
         "orc_int8_quant": (None, [_i8p, _f32p, C.c_size_t, C.c_float, C.c_int]),
@@ -208,6 +210,24 @@ def cross_entropy(logits, targets, grad_scale=1.0):
     V, S = logits.shape
     dl = np.empty_like(logits)
     loss = lib.orc_cross_entropy(dl, logits, targets, V, S, grad_scale)
+    return float(loss), dl
+
+
+def softmax_cols(logits):
+    """Column softmax of logits [V,S] — train_large_ane.m:508-516."""
+    logits = _f32(logits)
+    V, S = logits.shape
+    p = np.empty_like(logits)
+    lib.orc_softmax_cols(p, logits, V, S)
+    return p
+
+
+def nll_from_probs(probs, targets):
+    """(loss, dlogits) from probabilities [V,S] — train_large_ane.m:519-530."""
+    probs = _f32(probs); targets = _i32(targets)
+    V, S = probs.shape
+    dl = np.empty_like(probs)
+    loss = lib.orc_nll_from_probs(dl, probs, targets, V, S)
     return float(loss), dl
 
 

@@ -349,6 +349,40 @@ ORC_API float orc_cross_entropy(float *dlogits, const float *logits, const int32
     return total / (float)S;
 }
 
+/* Column softmax as the static loop computes it when the classifier stays on the CPU —
+ * training/train_large_ane.m:508-516: per position t, maxv starts at -1e30f, every entry becomes
+ * expf(x - maxv) while the sum is accumulated in row order, then every entry is divided by the sum. */
+ORC_API void orc_softmax_cols(float *probs, const float *logits, int V, int S) {
+    for (int t = 0; t < S; t++) {
+        float maxv = -1e30f;
+        for (int v = 0; v < V; v++) { float val = logits[(size_t)v * S + t]; if (val > maxv) maxv = val; }
+        float sum = 0.0f;
+        for (int v = 0; v < V; v++) {
+            float e = expf(logits[(size_t)v * S + t] - maxv);
+            probs[(size_t)v * S + t] = e;
+            sum += e;
+        }
+        for (int v = 0; v < V; v++) probs[(size_t)v * S + t] /= sum;
+    }
+}
+
+/* NLL loss and gradient on given probabilities — training/train_large_ane.m:519-530:
+ * loss = -sum_t logf(probs[tgt_t, t] + 1e-10f) / S; dlogits = (probs - onehot) * (1/S) (vDSP_vsmul).
+ * The reference indexes with the target unchecked; a target outside [0,V) is given no loss term and no
+ * one-hot here. */
+ORC_API float orc_nll_from_probs(float *dlogits, const float *probs, const int32_t *targets, int V, int S) {
+    float total = 0.0f, invS = 1.0f / (float)S;
+    memmove(dlogits, probs, (size_t)V * S * sizeof(float));
+    for (int t = 0; t < S; t++) {
+        int tgt = targets[t];
+        if (tgt < 0 || tgt >= V) continue;
+        total -= logf(probs[(size_t)tgt * S + t] + 1e-10f);
+        dlogits[(size_t)tgt * S + t] -= 1.0f;
+    }
+    for (size_t i = 0; i < (size_t)V * S; i++) dlogits[i] = dlogits[i] * invS;
+    return total / (float)S;
+}
+
 /* Range diagnostics — training/training_dynamic/train.m:664-666 (vDSP_maxmgv) and :738-742 (vDSP_maxv,
  * vDSP_minv): out = {min, max, max |x|}.  NaNs are skipped. */
 ORC_API void orc_minmax(float *out3, const float *x, size_t n) {

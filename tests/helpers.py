@@ -5,19 +5,36 @@ import numpy as np
 TOL_F32 = 1e-5          # the fp32 parity bound of this path
 
 
-def rel_err(a, ref):
-    """max_i |a_i - ref_i| / max(|ref_i|, rms(ref)).
+def rel_err(a, ref, floor=1.0):
+    """max_i |a_i - ref_i| / max(|ref_i|, floor * rms(ref)).
 
-    Element-wise relative error, with the tensor's RMS as the floor of the denominator so that
-    entries that are (nearly) zero by cancellation are judged against the scale of the tensor."""
+    Element-wise relative error; `floor` (in units of the tensor's RMS) bounds the denominator from below.
+    floor = 1: entries that are small by cancellation are judged against the scale of the tensor — used only
+    for outputs whose formula subtracts nearly equal terms (RMSNorm dx, the rotation after a norm) or sums
+    thousands of signed terms (dw, loss gradients through GEMMs).  See err_std and err_elem for the others."""
     a = np.asarray(a, np.float64).ravel()
     ref = np.asarray(ref, np.float64).ravel()
     assert a.shape == ref.shape
     if a.size == 0:
         return 0.0
     rms = float(np.sqrt(np.mean(ref * ref)))
-    den = np.maximum(np.abs(ref), rms if rms > 0 else 1.0)
-    return float(np.max(np.abs(a - ref) / den))
+    den = np.maximum(np.abs(ref), floor * (rms if rms > 0 else 1.0))
+    den = np.maximum(den, 1.1754944e-38)        # entries below the smallest normal fp32 are judged against it
+    diff = np.abs(a - ref)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.where(diff == 0.0, 0.0, diff / den)
+    return float(np.max(q))
+
+
+def err_std(a, ref):
+    """The metric of this path: max |a - ref| / max(|ref|, 1e-3 * rms(ref))."""
+    return rel_err(a, ref, 1e-3)
+
+
+def err_elem(a, ref):
+    """Pure element-wise relative error (no floor): for outputs that are products of the inputs with no
+    subtraction (RMSNorm forward, SwiGLU forward, dh3, INT8 dequantize)."""
+    return rel_err(a, ref, 0.0)
 
 
 def normal(seed, shape, mean=0.0, std=1.0):

@@ -7,6 +7,7 @@ import subprocess
 import sys
 
 import numpy as np
+import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HDR = os.path.join(ROOT, "include", "mi355_bridge.h")
@@ -32,11 +33,21 @@ def test_library_exports_every_declared_symbol():
     assert not extra, extra
 
 
-def test_cpu_ops_header_compiles_as_c99(tmp_path):
-    src = tmp_path / "t.c"
-    src.write_text('#define VOCAB 32000\n#include "mi355_cpu_ops.h"\nint main(void){return 0;}\n')
-    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-Wno-unused-function", "-fsyntax-only", "-I",
-                        os.path.join(ROOT, "include"), str(src)], capture_output=True, text=True)
+@pytest.mark.parametrize("loop", ["dynamic_loop", "static_loop"])
+def test_reference_call_sites_compile_against_the_cpu_ops_header(tmp_path, loop):
+    """tests/callsites/*.c hold every CPU-op call of the reference's loops with the loops' own argument lists
+    (both adam_update forms, the VocabMap functions); they must compile as C99 with -Wall -Werror against
+    include/mi355_cpu_ops.h and link against the library."""
+    import ane_amd.bridge as br
+    src = os.path.join(ROOT, "tests", "callsites", loop + ".c")
+    exe = str(tmp_path / loop)
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-Wno-unused-function", "-I",
+                        os.path.join(ROOT, "include"), src, "-L", os.path.dirname(br.LIB_PATH), "-lmi355_ops", "-lm",
+                        "-o", exe], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    # the same unit as C++ and as Objective-C-free C11 with pedantic warnings
+    r = subprocess.run(["g++", "-x", "c++", "-std=c++17", "-Wall", "-Werror", "-Wno-unused-function", "-fsyntax-only",
+                        "-I", os.path.join(ROOT, "include"), src], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
 
 
@@ -53,6 +64,32 @@ def test_entry_points_fail_cleanly_without_a_gpu():
     br.lib.mi355_rmsnorm(y.ctypes.data, y.ctypes.data, y.ctypes.data, 2, 4)
     assert np.all(y == 3.0)
     br.lib.mi355_shutdown()
+
+
+def test_every_rmsnorm_shape_has_a_kernel():
+    """The tile picker may only choose tiles that are instantiated: every channel count from 1 to 4200, at column
+    counts on both sides of its thresholds (including 128 x 256 columns, where 16-lane strips of 512 threads win),
+    for all three entry points, aligned or not, and under every tuning knob."""
+    import ane_amd.bridge as br
+    tile = (ctypes.c_int * 4)()
+    shapes = [(256, 1), (256, 16), (256, 32), (256, 128), (256, 300), (64, 2), (37, 2), (20, 3), (4, 1), (1024, 64)]
+    seen = set()
+    try:
+        for lpr, thr in [(0, 0)] + [(l, t) for l in (4, 8, 16) for t in (256, 512, 1024)]:
+            br.lib.mi355_tune_set(b"rms_lpr", lpr); br.lib.mi355_tune_set(b"rms_threads", thr)
+            for C in list(range(1, 1100)) + list(range(1100, 4200, 37)) + [5000, 8192, 16384]:
+                if (lpr or thr) and C % 7:
+                    continue
+                for S, batch in shapes:
+                    for op in (0, 1, 2):
+                        for aligned in (1, 0):
+                            assert br.lib.mi355_rmsnorm_tile(op, C, S, batch, aligned, tile) == 0, \
+                                (op, C, S, batch, aligned, lpr, thr, list(tile), br.last_error())
+                            seen.add(tuple(tile))
+    finally:
+        br.lib.mi355_tune_set(b"rms_lpr", 0); br.lib.mi355_tune_set(b"rms_threads", 0)
+    assert (4, 16, 512, 8) in seen or (4, 16, 512, 16) in seen        # the tile that used to be missing
+    assert br.lib.mi355_rmsnorm_tile(3, 8, 8, 1, 1, None) == -1
 
 
 def test_bench_refuses_more_than_one_gpu():

@@ -23,7 +23,8 @@ def _rms_shapes():
         B = int(rng.integers(1, 5))
         out.append((B, C, S))
     # the last three have enough columns for the 128-byte strips (fp32 and bf16 pickers switch on strips x batch)
-    return out + [(1, 2048, 256), (3, 2049, 12), (2, 4096, 64), (7, 16, 1024), (32, 1024, 256), (40, 768, 256), (9, 600, 1024)]
+    return out + [(1, 2048, 256), (3, 2049, 12), (2, 4096, 64), (7, 16, 1024), (32, 1024, 256), (40, 768, 256), (9, 600, 1024),
+                  (128, 384, 256)]      # 32768 columns below 512 channels: 16-lane strips on 512 threads
 
 
 @pytest.mark.parametrize("B,C,S", _rms_shapes())
@@ -34,7 +35,7 @@ def test_rmsnorm_random_shapes(br, B, C, S):
     xd, wd, dyd, bd = (dev(br, a) for a in (x, w, dy, b2))
     yd, dxd, dwd = br.DevArray(x.shape), br.DevArray(x.shape), dev(br, dw0)
     br.check(br.lib.mi355_rmsnorm_fwd_dev(yd.ptr, xd.ptr, wd.ptr, C, S, B, 1e-5))
-    assert H.rel_err(yd.numpy(), O.rmsnorm(x, w)) <= TOL
+    assert H.err_elem(yd.numpy(), O.rmsnorm(x, w)) <= TOL
     br.check(br.lib.mi355_rmsnorm_bwd_dev(dxd.ptr, dwd.ptr, dyd.ptr, xd.ptr, wd.ptr, C, S, B, 1e-5, 0))
     rdx, rdw = O.rmsnorm_bwd(dy, x, w, dw=dw0)
     assert H.rel_err(dxd.numpy(), rdx) <= TOL and H.rel_err(dwd.numpy(), rdw) <= TOL
@@ -43,7 +44,12 @@ def test_rmsnorm_random_shapes(br, B, C, S):
     al = np.float32(24 ** 0.25)
     br.check(br.lib.mi355_residual_rmsnorm_fwd_dev(y2.ptr, yn.ptr, xd.ptr, bd.ptr, al, wd.ptr, C, S, B, 1e-5))
     r2 = O.axpby(x, b2, al, 0)
-    assert np.array_equal(y2.numpy(), r2) and H.rel_err(yn.numpy(), O.rmsnorm(r2, w)) <= TOL
+    assert np.array_equal(y2.numpy(), r2) and H.err_elem(yn.numpy(), O.rmsnorm(r2, w)) <= TOL
+    # backward with the residual riding along (8-row tiles, or the two-sweep variant)
+    dx3, dw3 = br.DevArray(x.shape), dev(br, dw0)
+    br.check(br.lib.mi355_rmsnorm_bwd_residual_dev(dx3.ptr, None, dw3.ptr, dyd.ptr, xd.ptr, wd.ptr, bd.ptr, 1.0, C, S, B,
+                                                   1e-5, 0))
+    assert H.rel_err(dx3.numpy(), O.axpby(rdx, b2, 0.0, 2)) <= TOL and H.rel_err(dw3.numpy(), rdw) <= TOL
 
 
 def _qk_shapes():
@@ -96,4 +102,66 @@ def test_softmax_ce_random_shapes(br, V, S):
     dl, lossd = br.DevArray(logits.shape), br.DevArray(1)
     br.check(br.lib.mi355_softmax_ce_dev(dl.ptr, lossd.ptr, ld.ptr, td.ptr, V, S, 1.0))
     rl, rd = O.cross_entropy(logits, tgt)
-    assert abs(float(lossd.numpy()[0]) - rl) <= TOL * max(abs(rl), 1e-3) and H.rel_err(dl.numpy(), rd) <= TOL
+    assert abs(float(lossd.numpy()[0]) - rl) <= TOL * max(abs(rl), 1e-3) and H.err_std(dl.numpy(), rd) <= TOL
+
+
+def _embed_cases():
+    """Seeded random shapes and id distributions for the gather and the ordered scatter-add: uniform ids, Zipf ids,
+    two or three hot tokens, ids of which a third are out of range, one token only; sequence lengths that are not
+    multiples of 4 or 64, row widths on both sides of the 128-bit and 256-float paths, vocabularies around the
+    planner's 2^18 limit, and every fifth case beyond its 16384 positions (library sort)."""
+    rng = np.random.default_rng(12345)
+    out = []
+    for case in range(36):
+        kind = int(rng.integers(0, 5))
+        S = int(rng.choice([1, 3, 4, 8, 16, 37, 64, 100, 256, 257, 512]))
+        B = int(rng.integers(1, max(2, min(300, 17000 // S))))
+        if case % 5 == 4:
+            B = max(1, 20000 // S)
+        D = int(rng.choice([1, 3, 4, 8, 20, 32, 33, 64, 96, 128, 256, 260, 768, 1024]))
+        if B * S * D > 12_000_000:
+            D = max(1, 12_000_000 // (B * S))
+        V = int(rng.choice([1, 2, 5, 37, 256, 1000, 32000, 151936, 262143, 262144, 400000]))
+        if V * D > 40_000_000:
+            V = max(1, 40_000_000 // D)
+        out.append((case, kind, V, D, B, S, int(rng.integers(1 << 30))))
+    return out
+
+
+@pytest.mark.parametrize("case,kind,V,D,B,S,seed", _embed_cases())
+def test_embed_gather_scatter_random_shapes(br, case, kind, V, D, B, S, seed):
+    print("[case] embed %d kind=%d V=%d D=%d B=%d S=%d" % (case, kind, V, D, B, S), flush=True)
+    rng = np.random.default_rng(seed)
+    N = B * S
+    if kind == 0: ids = rng.integers(0, V, N)
+    elif kind == 1: ids = H.zipf_ids(seed, N, V)
+    elif kind == 2: ids = rng.integers(0, max(1, min(V, 3)), N)
+    elif kind == 3: ids = np.where(rng.random(N) < 0.3, rng.integers(-5, V + 5, N), rng.integers(0, V, N))
+    else: ids = np.full(N, rng.integers(0, V))
+    ids = ids.astype(np.int32).reshape(B, S)
+    E = (rng.standard_normal((V, D)) * 0.02).astype(np.float32)
+    # gather: a copy, bit for bit; columns of skipped ids keep what the output held
+    x0 = np.full((B, D, S), 7.0, np.float32)
+    Ed, idd, xd = dev(br, E), dev(br, ids), dev(br, x0)
+    br.check(br.lib.mi355_embed_gather_dev(xd.ptr, Ed.ptr, idd.ptr, V, D, S, B))
+    want, _ = O.embed_lookup(E, ids, out=x0.copy())
+    assert xd.numpy().tobytes() == want.tobytes()
+    # scatter-add: the reference loop's order, bit for bit, by default; the opt-in tree order within each row's scale
+    dx = (rng.standard_normal((B, D, S)) * 3).astype(np.float32)
+    dE0 = rng.standard_normal((V, D)).astype(np.float32)
+    dxd, dEd = dev(br, dx), dev(br, dE0)
+    tree = case % 7 == 6
+    br.tune("scatter_tree", int(tree))
+    try:
+        br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, idd.ptr, V, D, S, B))
+    finally:
+        br.tune("scatter_tree", 0)
+    got, ref = dEd.numpy(), O.embed_backward(dE0, dx, ids)
+    if not tree:
+        assert got.tobytes() == ref.tobytes()
+    else:
+        # a reordered fp32 sum of n terms of scale 3: each row is judged against the size of its own partial sums
+        cnt = np.bincount(ids[(ids >= 0) & (ids < V)].ravel(), minlength=V).astype(np.float64)
+        scale = np.maximum(np.sqrt(np.mean(ref.astype(np.float64) ** 2, axis=1)), 3.0 * np.sqrt(np.maximum(cnt, 1.0)))
+        assert np.max(np.max(np.abs(got.astype(np.float64) - ref), axis=1) / scale) <= TOL
+        assert np.array_equal(got[cnt <= 96], ref[cnt <= 96])          # short segments keep the reference order

@@ -400,6 +400,41 @@ def test_cross_entropy_out_of_range_target_policy():
     assert abs(dl[:, 1].astype(np.float64).sum() - 1.0) < 1e-6      # skipped column = unscaled softmax
 
 
+def test_column_softmax_and_nll_on_probabilities():
+    """The halves of the op as training/train_large_ane.m:508-530 runs them: pinned by the float64 closed form, by
+    the column sums, by the recipe of training/test_classifier.m:132-134, and against the fused op (the two
+    formulations of the reference must agree: p*(1/sum) there, p/sum here)."""
+    V, S = 101, 6
+    x, _, _ = O.recipe_drand48(2, 999, V * S, 0)
+    logits = x.reshape(V, S)
+    p = O.softmax_cols(logits)
+    l64 = logits.astype(np.float64)
+    e = np.exp(l64 - l64.max(axis=0))
+    p64 = e / e.sum(axis=0)
+    assert H.err_elem(p, p64) < F32_FAITHFUL
+    assert np.allclose(p.astype(np.float64).sum(axis=0), 1.0, atol=1e-6)
+    assert np.all(p.argmax(axis=0) == logits.argmax(axis=0))
+    tgt = np.array([3, 100, 0, 57, 57, 1], np.int32)
+    loss, dl = O.nll_from_probs(p, tgt)
+    cols = np.arange(S)
+    assert abs(loss - (-np.log(p64[tgt, cols] + 1e-10).mean())) < 1e-6
+    d64 = p64.copy(); d64[tgt, cols] -= 1.0; d64 /= S
+    assert H.err_std(dl, d64) < F32_FAITHFUL
+    assert np.max(np.abs(dl.astype(np.float64).sum(axis=0))) < 1e-7
+    # same numbers as the fused op
+    floss, fdl = O.cross_entropy(logits, tgt)
+    assert abs(floss - loss) < 1e-6 and H.err_std(dl, fdl) < 1e-6
+    # hand-computable: two classes, logits (0, ln 3) -> probs (1/4, 3/4)
+    p2 = O.softmax_cols(np.array([[0.0], [np.log(3.0)]], np.float32))
+    assert np.allclose(p2[:, 0], [0.25, 0.75], rtol=1e-6)
+    l2, d2 = O.nll_from_probs(p2, np.array([1], np.int32))
+    assert abs(l2 - (-np.log(0.75 + 1e-10))) < 1e-6 and np.allclose(d2[:, 0], [0.25, -0.25], rtol=1e-6)
+    # a target outside the vocabulary: no loss term, no one-hot, column still scaled by 1/S
+    l3, d3 = O.nll_from_probs(p, np.array([3, V, 0, -1, 57, 1], np.int32))
+    assert np.allclose(d3[:, 1], p[:, 1] / S, rtol=1e-6) and np.allclose(d3[:, 3], p[:, 3] / S, rtol=1e-6)
+    assert abs(l3 - (-(np.log(p64[[3, 0, 57, 1], [0, 2, 4, 5]] + 1e-10)).sum() / S)) < 1e-6
+
+
 # ---------------------------------------------------------------------------------------------
 # INT8
 # ---------------------------------------------------------------------------------------------
