@@ -236,13 +236,15 @@ def test_swiglu_fwd_bwd(br, n):
     assert H.err_elem(od.numpy(), O.swiglu_fwd(h1, h3)) <= TOL
     r1, r3 = O.swiglu_bwd(d, h1, h3)
     t1, t3 = H.np_swiglu_bwd(d, h1, h3)
-    assert H.err_elem(d3.numpy(), r3) <= TOL and H.err_elem(d3.numpy(), t3) <= TOL
-    assert H.err_elem(od.numpy(), H.np_swiglu_fwd(h1, h3)) <= TOL
+    # against float64 the floor is 1e-3 of the tensor's scale: where sigmoid(-88) is a subnormal fp32 number the
+    # fp32 formula itself (oracle and GPU alike) is 1e-4 away from the exact value
+    assert H.err_elem(d3.numpy(), r3) <= TOL and H.err_std(d3.numpy(), t3) <= TOL
+    assert H.err_std(od.numpy(), H.np_swiglu_fwd(h1, h3)) <= TOL
     # dh1 carries the factor 1 + h1*(1 - sig), which passes through zero at h1 = -1.2785: element-wise relative
     # error away from that zero, the tensor's scale as the yardstick next to it (the subtraction cancels there)
     h64 = h1.astype(np.float64); sg = 1.0 / (1.0 + np.exp(-h64))
     away = np.abs(1.0 + h64 * (1.0 - sg)) > 0.05
-    assert H.err_elem(d1.numpy()[away], r1[away]) <= TOL and H.err_elem(d1.numpy()[away], t1[away]) <= TOL
+    assert H.err_elem(d1.numpy()[away], r1[away]) <= TOL and H.err_std(d1.numpy()[away], t1[away]) <= TOL
     assert H.rel_err(d1.numpy(), r1) <= TOL and H.rel_err(d1.numpy(), t1) <= TOL
     assert np.all(np.isfinite(od.numpy())) and np.all(np.isfinite(d1.numpy()))
 
