@@ -92,6 +92,7 @@ SIGNATURES = {
     "mi355_sumsq_accum_multi_dev": (_i, [_p, _p, _p, _i, _f]),
     "mi355_adam_update_multi_dev": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _f, _f, _f, _f, _f, _p, _i]),
     "mi355_rmsnorm_tile": (_i, [_i, _i, _i, _i, _i, _p]),
+    "mi355_softmax_ce_noalloc_dev": (_i, [_p, _p, _p, _p, _i, _i, _f]),
     "mi355_softmax_cols_dev": (_i, [_p, _p, _i, _i]),
     "mi355_nll_from_probs_dev": (_i, [_p, _p, _p, _p, _i, _i]),
     "mi355_vocab_map_build_dev": (_i, [_p, _p, _p, _p, _z, _i]),

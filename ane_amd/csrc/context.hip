@@ -54,6 +54,8 @@ void *mi355_ws(size_t bytes) {
     return p;
 }
 
+int mi355_ce_setup(void);        // softmax_ce.hip: locates its fixed scratch array on the current device
+
 MI355_API int mi355_init(void) {
     if (g_ctx.ready) return 0;
     int n = 0;
@@ -73,6 +75,7 @@ MI355_API int mi355_init(void) {
     g_ctx.ws = nullptr;
     g_ctx.ws_bytes = 0;
     g_ctx.ready = true;
+    if (mi355_ce_setup()) { g_ctx.ready = false; return -1; }
     g_err[0] = 0;
     return 0;
 }

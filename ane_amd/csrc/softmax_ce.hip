@@ -363,9 +363,20 @@ int grad_blocks_per_cu() {
     return cached;
 }
 
+// Scratch of mi355_softmax_ce_noalloc_dev: the first-pass partials and the three per-column arrays, in a
+// file-scope device array, so that the call needs no allocation.  One copy per GPU, held until the process ends.
+// In host code the array's name is only a handle for the symbol lookup below; kernels and copies use the address
+// that the lookup returns for the current device.
+constexpr size_t CE_SCRATCH_BYTES = (size_t)2 << 20;
+constexpr int CE_MAX_DEVICES = 16;
+}   // namespace
+static __device__ __align__(256) unsigned char scratch[CE_SCRATCH_BYTES];
+namespace {
+unsigned char *g_scratch_ptr[CE_MAX_DEVICES] = {};
+
 template <typename T>
 int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const int32_t *targets, int V, int S,
-           float grad_scale) {
+           float grad_scale, bool no_alloc = false) {
     if (!mi355_ready(who)) return -1;
     if (!dlogits || !loss_dev || !logits || !targets) return mi355_fail("%s: NULL pointer", who);
     if (V <= 0 || S <= 0) return mi355_fail("%s: bad shape V=%d S=%d", who, V, S);
@@ -413,7 +424,17 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
 
     auto al = [](size_t b) { return (b + 255) & ~(size_t)255; };
     const size_t part_b = al((size_t)nblk * S * sizeof(float)), col_b = al((size_t)S * sizeof(float));
-    char *ws = (char *)mi355_ws(2 * part_b + 3 * col_b);
+    char *ws;
+    if (no_alloc) {
+        if (2 * part_b + 3 * col_b > CE_SCRATCH_BYTES)
+            return mi355_fail("%s: V=%d S=%d needs %zu bytes of scratch, the fixed scratch holds %zu "
+                              "(use mi355_softmax_ce_dev, whose workspace grows)", who, V, S, 2 * part_b + 3 * col_b,
+                              CE_SCRATCH_BYTES);
+        ws = (g_ctx.device >= 0 && g_ctx.device < CE_MAX_DEVICES) ? (char *)g_scratch_ptr[g_ctx.device] : nullptr;
+        if (!ws) return mi355_fail("%s: the scratch array was not located at init", who);
+    } else {
+        ws = (char *)mi355_ws(2 * part_b + 3 * col_b);
+    }
     if (!ws) return -1;
     float *pm = (float *)ws, *pl = (float *)(ws + part_b);
     float *colM = (float *)(ws + 2 * part_b), *colInv = (float *)(ws + 2 * part_b + col_b);
@@ -438,6 +459,25 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
 }
 
 }   // namespace
+
+// Called by mi355_init with the device current: finds this device's copy of the scratch array, and asks the
+// runtime for the second pass's occupancy now so that the entry point below never has to.
+int mi355_ce_setup(void) {
+    const int dev = g_ctx.device;
+    if (dev < 0 || dev >= CE_MAX_DEVICES) return mi355_fail("init: device index %d beyond %d", dev, CE_MAX_DEVICES);
+    unsigned char *ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return mi355_fail("init: hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+    (void)grad_blocks_per_cu<float>();
+    return 0;
+}
+
+// The same op with its scratch in the fixed device array: no hipMalloc, no hipFree, no workspace growth.
+MI355_API int mi355_softmax_ce_noalloc_dev(float *dlogits, float *loss_dev, const float *logits, const int32_t *targets,
+                                           int V, int S, float grad_scale) {
+    return ce_run<float>("softmax_ce_noalloc", dlogits, loss_dev, logits, targets, V, S, grad_scale, true);
+}
 
 MI355_API int mi355_softmax_cols_dev(float *probs, const float *logits, int V, int S) {
     if (!mi355_ready("softmax_cols")) return -1;

@@ -254,6 +254,16 @@ int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, 
 int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float *logits,
                          const int32_t *targets, int V, int S, float grad_scale);
 
+/* mi355_softmax_ce_dev for callers that may not allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and the same
+ * bits out, but the scratch (first-pass partials, per-column max / sum / loss) lives in a fixed 2 MiB device array
+ * of the library, located once by mi355_init: the call performs no hipMalloc, no hipFree and no workspace growth.
+ * Limit: 2 * ceil(V / rows per workgroup) * S * 4 + 3 * S * 4 bytes (rounded up to 256 each) must fit 2 MiB —
+ * [151936, 256] needs 0.93 MiB — otherwise the call fails with a message and launches nothing.  Every call on a
+ * GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race. */
+int mi355_softmax_ce_noalloc_dev(float *dlogits, float *loss_dev, const float *logits, const int32_t *targets,
+                                 int V, int S, float grad_scale);
+
 /* The two halves of that op as the static loop with ANE extras runs them when the classifier stays on the CPU
  * (training/train_large_ane.m:499-530).
  * mi355_softmax_cols_dev: probs[v][t] = exp(logits[v][t] - max_v) / sum_v exp(...), per column t — the scalar loop of
