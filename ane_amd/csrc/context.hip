@@ -85,6 +85,7 @@ void mi355_dw_free(void);       // queued weight-gradient reductions and their a
 void mi355_blas_free(void);     // rocBLAS handle of mi355_sgemm_dev
 void mi355_ckpt_free(void);     // pinned staging buffer of the checkpoint reader/writer
 void mi355_graph_shutdown(void);  // capture stream
+void mi355_norm_free(void);       // exchange area of the clustered RMSNorm
 
 MI355_API void mi355_shutdown(void) {
     if (!g_ctx.ready) return;
@@ -94,6 +95,7 @@ MI355_API void mi355_shutdown(void) {
     mi355_blas_free();
     mi355_ckpt_free();
     mi355_graph_shutdown();
+    mi355_norm_free();
     if (g_ctx.ws) (void)hipFree(g_ctx.ws);
     g_ctx = Mi355Ctx{};
 }
@@ -148,6 +150,7 @@ MI355_API int mi355_tune_set(const char *key, int value) {
         {"ew_unroll", &g_ctx.ew_unroll},
         {"ce_rows", &g_ctx.ce_rows}, {"ce_rows2", &g_ctx.ce_rows2}, {"buf_phase", &g_ctx.buf_phase}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
         {"gemm_splitk", &g_ctx.gemm_splitk}, {"scatter_tree", &g_ctx.scatter_tree},
+        {"rms_cluster", &g_ctx.rms_cluster}, {"rms_cluster_spin", &g_ctx.rms_cluster_spin},
     };
     for (auto &t : tab)
         if (strcmp(t.k, key) == 0) { *t.v = value; return 0; }

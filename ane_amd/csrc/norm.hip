@@ -13,6 +13,7 @@
 // a second kernel, so the result is deterministic and needs no floating-point atomics.
 #include "common.h"
 #include "tile.h"
+#include "norm_cluster.h"
 
 namespace {
 
@@ -469,6 +470,40 @@ NormCfg plan_tile(int op, int C, int S, int batch, bool vec_ok) {
         }                                                                                             \
     } while (0)
 
+int cluster_spin_ticks(void) {
+    return g_ctx.rms_cluster_spin == 0 ? 200000 : (g_ctx.rms_cluster_spin < 0 ? 0 : g_ctx.rms_cluster_spin);
+}
+
+// The single-workgroup tiles are chosen by hand (knobs) or the shape does not cluster: csplit == 0.
+ClusterPlan plan_cluster(int C, int S, int batch, bool vec_ok, int max_rpt) {
+    if (g_ctx.rms_lpr || g_ctx.rms_threads) return ClusterPlan{0, 0, 0, 0, 0, 0};
+    return cluster_plan(C, S, batch, vec_ok, max_rpt);
+}
+
+template <bool FUSE>
+void launch_fwd_cluster(const ClusterPlan &cp, float *yn, float *y_res, const float *a, const float *b, float alpha,
+                        const float *w, int C, int S, float eps) {
+    const float invC = 1.0f / (float)C;
+    if (cp.rpt == 4)
+        hipLaunchKernelGGL((rms_fwd_cluster_kernel<4, 1024, FUSE>), dim3(cp.nblk), dim3(1024), 0, g_ctx.stream, yn, y_res,
+                           a, b, alpha, w, C, S, cp.strips, cp.nblk, cp.csplit, cp.rows_pm, eps, invC, g_cluster_ws,
+                           cluster_spin_ticks());
+    else
+        hipLaunchKernelGGL((rms_fwd_cluster_kernel<8, 1024, FUSE>), dim3(cp.nblk), dim3(1024), 0, g_ctx.stream, yn, y_res,
+                           a, b, alpha, w, C, S, cp.strips, cp.nblk, cp.csplit, cp.rows_pm, eps, invC, g_cluster_ws,
+                           cluster_spin_ticks());
+}
+
+// The backward tiles hold two (with the residual three) operands per row: four rows per lane fill the registers.
+template <bool RES>
+void launch_bwd_cluster(const ClusterPlan &cp, float *dx, float *part, const float *dy, const float *x, const float *w,
+                        int C, int S, float eps, int variant, const float *res, float *dx2, float alpha2) {
+    const float invC = 1.0f / (float)C;
+    hipLaunchKernelGGL((rms_bwd_cluster_kernel<4, 1024, RES>), dim3(cp.nblk), dim3(1024), 0, g_ctx.stream, dx, part, dy,
+                       x, w, C, S, cp.strips, cp.nblk, cp.csplit, cp.rows_pm, eps, invC, variant, res, dx2, alpha2,
+                       g_cluster_ws, cluster_spin_ticks());
+}
+
 }   // namespace
 
 // Host-only: which tile an entry point would run for a shape, and whether that tile exists.
@@ -485,6 +520,13 @@ MI355_API int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, in
     if (!y || !x || !w) return mi355_fail("rmsnorm_fwd: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_fwd: bad shape C=%d S=%d batch=%d", C, S, batch);
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(y);
+    const ClusterPlan cp = plan_cluster(C, S, batch, vec_ok, 8);
+    if (cp.csplit) {
+        if (!cluster_ws_ready()) return -1;
+        launch_fwd_cluster<false>(cp, y, nullptr, x, nullptr, 0.f, w, C, S, eps);
+        LAUNCH_OK("rmsnorm_fwd");
+        return 0;
+    }
     NormCfg cfg = plan_tile(0, C, S, batch, vec_ok);
     NORM_DISPATCH(launch_fwd, cfg, y, x, w, C, S, batch, eps);
     LAUNCH_OK("rmsnorm_fwd");
@@ -497,7 +539,21 @@ MI355_API int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const
     if (!dx || !dw || !dy || !x || !w) return mi355_fail("rmsnorm_bwd: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_bwd: bad shape C=%d S=%d batch=%d", C, S, batch);
     if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd: variant must be 0 or 1");
+    if (dx == x) return mi355_fail("rmsnorm_bwd: dx must not alias x (dx may alias dy)");
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(dy) && aligned16(dx);
+    // in place on dy the single-workgroup tile is used: a cluster member that has to recompute another member's
+    // sums (its bounded wait expired) would read rows that their owner has already overwritten
+    const ClusterPlan cp = dx == dy ? ClusterPlan{0, 0, 0, 0, 0, 0} : plan_cluster(C, S, batch, vec_ok, 4);
+    if (cp.csplit) {
+        if (!cluster_ws_ready()) return -1;
+        const int nrows = cp.nblk / cp.csplit;
+        float *part = mi355_dw_partials((size_t)nrows * C, dw, nullptr);
+        if (!part) return -1;
+        launch_bwd_cluster<false>(cp, dx, part, dy, x, w, C, S, eps, variant, nullptr, nullptr, 0.f);
+        LAUNCH_OK("rmsnorm_bwd");
+        if (mi355_dw_submit(dw, part, nrows, C)) return -1;
+        return mi355_dw_op_end();
+    }
     NormCfg cfg = plan_tile(1, C, S, batch, vec_ok);
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
@@ -519,8 +575,20 @@ MI355_API int mi355_rmsnorm_bwd_residual_dev(float *dx, float *dx_scaled, float 
     if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd_residual: variant must be 0 or 1");
     if (dx_scaled && (dx_scaled == dx || dx_scaled == dy || dx_scaled == x || dx_scaled == res))
         return mi355_fail("rmsnorm_bwd_residual: dx_scaled must not alias another operand");
+    if (dx == x) return mi355_fail("rmsnorm_bwd_residual: dx must not alias x (dx may alias res or dy)");
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(res) &&
                         (!dx_scaled || aligned16(dx_scaled));
+    const ClusterPlan cp = dx == dy ? ClusterPlan{0, 0, 0, 0, 0, 0} : plan_cluster(C, S, batch, vec_ok, 4);
+    if (cp.csplit) {
+        if (!cluster_ws_ready()) return -1;
+        const int nrows = cp.nblk / cp.csplit;
+        float *part = mi355_dw_partials((size_t)nrows * C, dw, nullptr);
+        if (!part) return -1;
+        launch_bwd_cluster<true>(cp, dx, part, dy, x, w, C, S, eps, variant, res, dx_scaled, alpha);
+        LAUNCH_OK("rmsnorm_bwd_residual");
+        if (mi355_dw_submit(dw, part, nrows, C)) return -1;
+        return mi355_dw_op_end();
+    }
     NormCfg cfg = plan_tile(2, C, S, batch, vec_ok);
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
@@ -541,6 +609,14 @@ MI355_API int mi355_residual_rmsnorm_fwd_dev(float *y, float *yn, const float *a
     if (yn == y || yn == a || yn == b) return mi355_fail("residual_rmsnorm_fwd: yn must not alias y, a or b");
     const bool vec_ok = (S % 4 == 0) && aligned16(y) && aligned16(yn) && aligned16(a) && aligned16(b);
     const float invC = 1.0f / (float)C;
+    // in place (y over a or b) the single-workgroup tile is used, for the reason given in mi355_rmsnorm_bwd_dev
+    const ClusterPlan cp = (y == a || y == b) ? ClusterPlan{0, 0, 0, 0, 0, 0} : plan_cluster(C, S, batch, vec_ok, 8);
+    if (cp.csplit) {
+        if (!cluster_ws_ready()) return -1;
+        launch_fwd_cluster<true>(cp, yn, y, a, b, alpha, w, C, S, eps);
+        LAUNCH_OK("residual_rmsnorm_fwd");
+        return 0;
+    }
 #define RES_RMS(VEC, LPR, THR, CAP)                                                                              \
     do {                                                                                                         \
         const int strips = (int)ceil_div((size_t)S, (size_t)(LPR) * (VEC));                                      \

@@ -31,6 +31,9 @@ PEAK_HBM_GBS = 8000.0      # MI355X published HBM3E peak
 # runs summarised in profiles/qwen3_sweep_pmc_fetch_write.md (FETCH_SIZE x 1.9992 + WRITE_SIZE x 0.9992, the
 # factors the same counters need to read 50.33 MB for a plain 50.33 MB copy).  Not measured live.
 MEASURED_TRAFFIC_BYTES = {"swiglu_bwd": 251.56e6}
+# the same for the three launches of the ordered scatter-add at BASELINE.json config 2
+# (profiles/embed_config2_pmc_fetch_write.md)
+SCATTER_TRAFFIC_BYTES = 176.14e6
 
 # Qwen3-0.6B (training/training_dynamic/models/qwen3_06b.h:6-16), batch 16
 Q3 = dict(C=1024, H=3072, heads=16, kv_heads=8, hd=128, S=256, batch=16, layers=28, V=151936, theta=1e6,
@@ -401,16 +404,16 @@ def zipf_ids(seed, n, vocab, s=1.1):
     return np.minimum(np.searchsorted(cdf, u, side="right"), vocab - 1).astype(np.int32)
 
 
-def bench_embed(br, args):
-    """BASELINE.json config 2: vocab 32000 x dim 768 table, 64 sequences x 256 Zipf(1.1) ids; gather + ordered scatter-add."""
+def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
+    """BASELINE.json config 2: vocab 32000 x dim 768 table, 64 sequences x 256 Zipf(1.1) ids; gather + ordered
+    scatter-add.  Returns the JSON object of that workload."""
     V, D, B, S = 32000, 768, 64, 256
     N = B * S
     ids = zipf_ids(0, N, V).reshape(B, S)
     U = int(np.unique(ids).size)
     E = br.DevArray((V, D)); br.check(br.lib.mi355_fill_normal_dev(E.ptr, E.size, 1, 0.0, 0.02))
     idd = br.DevArray.from_numpy(ids)
-    nbuf = 6                                               # rotate buffers so operands are cold
-    xs = [br.DevArray((B, D, S)) for _ in range(nbuf)]
+    xs = [br.DevArray((B, D, S)) for _ in range(nbuf)]     # rotate buffers so operands are cold
     gs = [br.DevArray((B, D, S)) for _ in range(nbuf)]
     dEs = [br.DevArray((V, D)) for _ in range(nbuf)]
     for i, g in enumerate(gs):
@@ -425,42 +428,44 @@ def bench_embed(br, args):
         for g, dE in zip(gs, dEs):
             br.check(br.lib.mi355_embed_scatter_add_dev(dE.ptr, g.ptr, idd.ptr, V, D, S, B))
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         gather(); scatter()
-    t_g = time_region(br, gather, args.steps) / nbuf
-    t_s = time_region(br, scatter, args.steps) / nbuf
+    t_g = time_region(br, gather, steps) / nbuf
+    t_s = time_region(br, scatter, steps) / nbuf
     br.tune("scatter_tree", 1)          # the opt-in fixed-tree order for long segments (deterministic, not bit-identical)
     scatter()
-    t_s_tree = time_region(br, scatter, args.steps) / nbuf
+    t_s_tree = time_region(br, scatter, steps) / nbuf
     br.tune("scatter_tree", 0)
 
     def copy():                         # y = 1.0*a over one activation slab: the streaming rate next to the two ops, and
         for x, g in zip(xs, gs):        # the known-size dispatch that scales the traffic counters of the profile
             br.check(br.lib.mi355_axpby_dev(x.ptr, g.ptr, None, 1.0, g.size, 1))
     copy()
-    t_c = time_region(br, copy, args.steps) / nbuf
-    b_g = 8 * D * N + 4 * N
+    t_c = time_region(br, copy, steps) / nbuf
+    b_g = 8 * D * N + 4 * N                 # the definition's bytes: every gathered row read once, written once
+    b_g_moved = 4 * D * U + 4 * D * N + 4 * N   # what has to cross HBM: each distinct row once, the output, the ids
     b_s = 4 * D * N + 8 * D * U + 4 * N
+    row = lambda op, ms, nbytes, **kw: dict(op=op, ms=ms, alg_mb=nbytes / 1e6, gbs=nbytes / ms / 1e6,
+                                            frac=nbytes / ms / 1e6 / PEAK_HBM_GBS, **kw)
     out = {"metric": "embedding gather + ordered scatter-add (BASELINE.json config 2)", "value": N / ((t_g + t_s) / 1e3),
-           "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": t_g + t_s,
+           "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": t_g + t_s,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32+i32", "data": "synthetic",
            "config": {"workload": "embedding table [32000,768] fp32, 64x256 Zipf(1.1) ids, seed 0", "unique_ids": U,
                       "hottest_id_count": int(np.bincount(ids.ravel()).max())},
-           "ops": [dict(op="embed_gather", ms=t_g, alg_mb=b_g / 1e6, gbs=b_g / t_g / 1e6, frac=b_g / t_g / 1e6 / PEAK_HBM_GBS),
-                   dict(op="embed_scatter_add", ms=t_s, alg_mb=b_s / 1e6, gbs=b_s / t_s / 1e6,
-                        frac=b_s / t_s / 1e6 / PEAK_HBM_GBS),
-                   dict(op="embed_scatter_add (scatter_tree=1)", ms=t_s_tree, alg_mb=b_s / 1e6, gbs=b_s / t_s_tree / 1e6,
-                        frac=b_s / t_s_tree / 1e6 / PEAK_HBM_GBS),
-                   dict(op="copy of one activation slab", ms=t_c, alg_mb=8 * D * N / 1e6, gbs=8 * D * N / t_c / 1e6,
-                        frac=8 * D * N / t_c / 1e6 / PEAK_HBM_GBS)],
+           "ops": [row("embed_gather", t_g, b_g, hbm_mb=b_g_moved / 1e6, hbm_frac=b_g_moved / t_g / 1e6 / PEAK_HBM_GBS,
+                       note="alg_mb counts every gathered row; hbm_mb counts each distinct row once (the rest are cache hits)"),
+                   row("embed_scatter_add", t_s, b_s, traffic_mb=SCATTER_TRAFFIC_BYTES / 1e6,
+                       traffic_source="profiles/embed_config2_pmc_fetch_write.md"),
+                   row("embed_scatter_add (scatter_tree=1)", t_s_tree, b_s),
+                   row("copy of one activation slab", t_c, 8 * D * N)],
            "roofline": dict(bound="hbm", kernel="embed_scatter_add (3 launches)", achieved=b_s / t_s / 1e6, peak=PEAK_HBM_GBS,
                             unit="GB/s", frac=b_s / t_s / 1e6 / PEAK_HBM_GBS,
-                            # chunk_sort 0.16 + rank_transpose 101.67 + seg_sum 74.31 MB (FETCH_SIZE + WRITE_SIZE, scaled)
-                            traffic=176.14e6, traffic_source="profiles/embed_config2_pmc_fetch_write.md",
+                            traffic=SCATTER_TRAFFIC_BYTES, traffic_source="profiles/embed_config2_pmc_fetch_write.md",
                             alg_bytes_per_launch=b_s, avg_launch_ms=t_s)}
-    if args.cpu_layers > 0:
+    if with_cpu:
         import oracle as O
         Eh = E.numpy(); g0 = gs[0].numpy()
+        gather()                            # the copy above went over the gathered slabs
         t0 = time.perf_counter(); ref_x, _ = O.embed_lookup(Eh, ids); t_cg = time.perf_counter() - t0
         # every dE buffer has accumulated the same number of times: compare one fresh pass
         dE0 = br.DevArray((V, D)); br.check(br.lib.mi355_embed_scatter_add_dev(dE0.ptr, gs[0].ptr, idd.ptr, V, D, S, B))
@@ -469,14 +474,17 @@ def bench_embed(br, args):
                                    "scatter_add_bit_exact": bool(dE0.numpy().tobytes() == ref_dE.tobytes())}
         out["cpu_baseline"] = dict(value=N / (t_cg + t_cs), unit="tokens/s", cores=1, kind="port",
                                    sample="the whole config-2 workload once: gather %.3f s + scatter-add %.3f s" % (t_cg, t_cs))
-    print(json.dumps(out))
+    return out
 
 
-def bench_optimizer(br, args):
+def bench_embed(br, args):
+    print(json.dumps(measure_embed(br, args.steps, args.warmup, args.cpu_layers > 0)))
+
+
+def measure_optimizer(br, steps, warmup, nset=8):
     """Optimizer tail of training/training_dynamic/train.m:748-877 on one Qwen3-0.6B layer's matrices
     (Wq,Wk,Wv,Wo,W1,W2,W3 = 15.7 M parameters) x 8 rotating sets: norm sweep + fused AdamW sweep."""
     sizes = [2048 * 1024, 1024 * 1024, 1024 * 1024, 1024 * 2048, 3072 * 1024, 1024 * 3072, 3072 * 1024]
-    nset = 8
     A = br.DevArray
     sets = []
     seed = 1
@@ -510,20 +518,24 @@ def bench_optimizer(br, args):
             br.check(br.lib.mi355_adam_update_multi_dev(pw, pg, pm, pv, narr, wdarr, k, 3, 3e-4, 0.9, 0.95, 1e-8, gsc,
                                                         cs.ptr, 1))
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         norm_pass(); adam_pass()
-    t_n = time_region(br, norm_pass, args.steps) / nset
-    t_a = time_region(br, adam_pass, args.steps) / nset
+    t_n = time_region(br, norm_pass, steps) / nset
+    t_a = time_region(br, adam_pass, steps) / nset
     P = sum(sizes)
     b_n, b_a = 4 * P, 32 * P           # read g | read w,g,m,v + write w,m,v,g(=0)
     out = {"metric": "optimizer tail (scaled global norm + clip + AdamW + gradient clear), parameters/s",
-           "value": P / ((t_n + t_a) / 1e3), "unit": "parameters/s", "n_gpus": 1, "steps": args.steps,
-           "warmup": args.warmup, "ms_per_step": t_n + t_a, "higher_is_better": True, "scaling": "weak",
+           "value": P / ((t_n + t_a) / 1e3), "unit": "parameters/s", "n_gpus": 1, "steps": steps,
+           "warmup": warmup, "ms_per_step": t_n + t_a, "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
            "config": {"workload": "one Qwen3-0.6B layer's 7 weight matrices (%d parameters), fp32 w/g/m/v" % P},
            "ops": [dict(op="sumsq_accum (7 tensors)", ms=t_n, alg_mb=b_n / 1e6, gbs=b_n / t_n / 1e6, frac=b_n / t_n / 1e6 / PEAK_HBM_GBS),
                    dict(op="adam_update (7 tensors)", ms=t_a, alg_mb=b_a / 1e6, gbs=b_a / t_a / 1e6, frac=b_a / t_a / 1e6 / PEAK_HBM_GBS)]}
-    print(json.dumps(out))
+    return out
+
+
+def bench_optimizer(br, args):
+    print(json.dumps(measure_optimizer(br, args.steps, args.warmup)))
 
 
 def bench_host(br, args):
@@ -690,6 +702,9 @@ def main():
                          "(BASELINE.json configs 0/1: one [C,256] sequence per op, 12 layers, RoPE without QK-norm); "
                          "embed = BASELINE.json config 2; optimizer = the Adam tail (each prints its own JSON line)")
     ap.add_argument("--batch", type=int, default=0, help="sequences per op (default: 16 for qwen3, 1 for stories110m)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="default workload only: skip the other BASELINE.json configurations (embedding config 2, the "
+                         "Stories110M shapes of configs 0/1, the optimizer tail) that a default run appends to its line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path needs no collectives); run with --gpus 1")
@@ -788,6 +803,35 @@ def main():
         out["cpu_baseline"] = cpu
         out["parity_vs_oracle_on_sample"] = {"max_rel_err": parity, "int8_bit_exact": int8_exact}
         out["gpu_over_cpu"] = out["value"] / cpu["value"]
+    default_run = (args.workload == "qwen3" and not (args.fuse or bf16 or args.graph or args.share_buffers or args.batch
+                                                      or args.headline_only or args.tune or args.buf_phase))
+    if default_run:
+        # The other BASELINE.json configurations, measured in the same run (they cost milliseconds): their rows join
+        # `ops` under a prefix, their own JSON objects go to `other_workloads`.
+        del wl
+        rnd = lambda r: {k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}
+        other = {}
+        emb = measure_embed(br, max(3, args.steps // 2), 2, args.cpu_layers > 0)
+        other["embedding_config2"] = emb
+        out["ops"] += [rnd(dict(r, op="config2: " + r["op"])) for r in emb["ops"]]
+        cfg1 = dict(S110)
+        wl1 = Workload(br, cfg1, cfg1["layers"])
+        for _ in range(2):
+            wl1.step()
+        br.sync()
+        ms1 = time_region(br, wl1.step, args.steps)
+        tab1 = per_op_table(br, wl1, args.op_reps)
+        other["stories110m_configs_0_1"] = {
+            "workload": "the same sweep at the Stories110M shapes (BASELINE.json configs 0/1): 12 layers, one [C,256] "
+                        "sequence per op (the reference's calling pattern), RoPE theta 1e4 without QK-norm, "
+                        "softmax-CE [32000,256]; every op is one kernel boundary here",
+            "ms_per_step": ms1, "tokens_per_s": cfg1["batch"] * cfg1["S"] / (ms1 / 1e3), "ops": [rnd(r) for r in tab1]}
+        out["ops"] += [rnd(dict(r, op="stories110m: " + r["op"])) for r in tab1]
+        del wl1
+        opt = measure_optimizer(br, max(3, args.steps // 2), 2, nset=4)
+        other["optimizer_tail"] = opt
+        out["ops"] += [rnd(dict(r, op="optimizer: " + r["op"])) for r in opt["ops"]]
+        out["other_workloads"] = other
     print(json.dumps(out))
 
 

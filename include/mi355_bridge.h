@@ -148,7 +148,7 @@ int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, int C, int S
  * training/training_dynamic/cpu_ops.h:24-54.  dx is assigned, dw[C] is accumulated (+=).
  * variant 0 = the reference CPU op: dx = ((dy - x*dot)*rr)*w;
  * variant 1 = the textbook gradient (training/backward.h:28-42, training/ane_rmsnorm_bwd.h:56-74):
- * dx = (dy*w)*rr - (x*dot)*rr.  Both use dot = rr^2/C * sum_c dy*x*w. */
+ * dx = (dy*w)*rr - (x*dot)*rr.  Both use dot = rr^2/C * sum_c dy*x*w.  dx may alias dy; it must not alias x. */
 int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const float *x, const float *w,
                           int C, int S, int batch, float eps, int variant);
 
@@ -175,15 +175,16 @@ int mi355_dw_flush(void);
  * rmsnorm_bwd + the add loop of train.m:714-721.  The adds and the scale are the separate passes' own, in their
  * order: the result equals mi355_rmsnorm_bwd_dev followed by mi355_axpby_dev (modes 2 and 1) bit for bit when
  * both run on the same tile shape (they do below 32 x 256 columns), and to the rounding of the column sums
- * otherwise.  dx may alias res or dy. */
+ * otherwise.  dx may alias res or dy; it must not alias x. */
 int mi355_rmsnorm_bwd_residual_dev(float *dx, float *dx_scaled, float *dw, const float *dy, const float *x,
                                    const float *w, const float *res, float alpha, int C, int S, int batch, float eps,
                                    int variant);
 
 /* Residual add fused with the RMSNorm that follows it in the loops: vDSP_vsma + rmsnorm at
  * training/training_dynamic/train.m:460-461 (and a layer's x_next feeding the next rmsnorm at :417).
- * y = a + alpha*b (as mode 0 of mi355_axpby_dev); yn = rmsnorm(y, w).  One launch instead of two; the
- * results are bit-identical to the two separate calls.  y may alias a or b; yn must not alias anything. */
+ * y = a + alpha*b (as mode 0 of mi355_axpby_dev); yn = rmsnorm(y, w).  One launch instead of two; y is bit-identical
+ * to the separate call, yn too when y aliases neither input (in place another tile shape is used, and yn then
+ * agrees to the rounding of the column sums).  y may alias a or b; yn must not alias anything. */
 int mi355_residual_rmsnorm_fwd_dev(float *y, float *yn, const float *a, const float *b, float alpha,
                                    const float *w, int C, int S, int batch, float eps);
 
