@@ -83,18 +83,75 @@ __device__ __forceinline__ v4f ld4_nt(const float *p) {
     return __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
 }
 
-// sum over the lanes {l ^ m : m in multiples of STEP below 64}, i.e. lanes that share (l % STEP)
+// Value of lane (l ^ M) of a wave64, through the cheapest path the ISA has for each distance: a DPP quad permute
+// inside the adder for 1 and 2, ds_swizzle in bit-mask mode (the LDS crossbar, no address register, no LDS memory)
+// for 4, 8 and 16, v_permlane32_swap for 32.
+template <int M>
+__device__ __forceinline__ float lane_xor(float v) {
+    static_assert(M == 1 || M == 2 || M == 4 || M == 8 || M == 16 || M == 32, "lane distance");
+    const int iv = __float_as_int(v);
+    int r;
+    if constexpr (M == 1) r = __builtin_amdgcn_update_dpp(0, iv, 0xB1, 0xF, 0xF, true);          // quad_perm:[1,0,3,2]
+    else if constexpr (M == 2) r = __builtin_amdgcn_update_dpp(0, iv, 0x4E, 0xF, 0xF, true);     // quad_perm:[2,3,0,1]
+    else if constexpr (M == 4) r = __builtin_amdgcn_ds_swizzle(iv, (4 << 10) | 0x1F);            // swizzle(SWAP,4)
+    else if constexpr (M == 8) r = __builtin_amdgcn_ds_swizzle(iv, (8 << 10) | 0x1F);
+    else if constexpr (M == 16) r = __builtin_amdgcn_ds_swizzle(iv, (16 << 10) | 0x1F);
+    else {
+        typedef unsigned lane_pair __attribute__((ext_vector_type(2)));
+        // {v with its upper half replaced by the lower half, v with its lower half replaced by the upper half}
+        const lane_pair p = __builtin_amdgcn_permlane32_swap((unsigned)iv, (unsigned)iv, false, false);
+        r = (int)((__lane_id() & 32) ? p[0] : p[1]);
+    }
+    return __int_as_float(r);
+}
+// DPP mirrors within half a row (lane i <-> 7-i) and a row (i <-> 15-i): in a butterfly whose earlier steps have
+// made the lanes of each group of 4 (of 8) agree, the mirrored lane holds what lane i^4 (i^8) holds.
+__device__ __forceinline__ float dpp_half_mirror(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float dpp_row_mirror(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));
+}
+
+// sum over the lanes {l ^ m : m in multiples of STEP below 64}, i.e. lanes that share (l % STEP); every lane of a
+// class adds the same pairs in the same order, so all of them end with the same bits
 template <int STEP>
 __device__ __forceinline__ float wave_sum_stride(float v) {
-#pragma unroll
-    for (int m = STEP; m < 64; m <<= 1) v += __shfl_xor(v, m, 64);
+    if constexpr (STEP <= 1) v += lane_xor<1>(v);
+    if constexpr (STEP <= 2) v += lane_xor<2>(v);
+    if constexpr (STEP <= 4) v += lane_xor<4>(v);
+    if constexpr (STEP <= 8) v += lane_xor<8>(v);
+    if constexpr (STEP <= 16) v += lane_xor<16>(v);
+    if constexpr (STEP <= 32) v += lane_xor<32>(v);
     return v;
 }
 // sum over groups of G adjacent lanes (G a power of two <= 64)
 template <int G>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-    for (int m = 1; m < G; m <<= 1) v += __shfl_xor(v, m, 64);
+    if constexpr (G >= 2) v += lane_xor<1>(v);
+    if constexpr (G >= 4) v += lane_xor<2>(v);
+    if constexpr (G >= 8) v += dpp_half_mirror(v);
+    if constexpr (G >= 16) v += dpp_row_mirror(v);
+    if constexpr (G >= 32) v += lane_xor<16>(v);
+    if constexpr (G >= 64) v += lane_xor<32>(v);
+    return v;
+}
+
+// whole-wave reductions on the same lane exchanges; every lane ends with the result
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, lane_xor<1>(v)); v = fmaxf(v, lane_xor<2>(v)); v = fmaxf(v, lane_xor<4>(v));
+    v = fmaxf(v, lane_xor<8>(v)); v = fmaxf(v, lane_xor<16>(v)); v = fmaxf(v, lane_xor<32>(v));
+    return v;
+}
+__device__ __forceinline__ float wave_min(float v) {
+    v = fminf(v, lane_xor<1>(v)); v = fminf(v, lane_xor<2>(v)); v = fminf(v, lane_xor<4>(v));
+    v = fminf(v, lane_xor<8>(v)); v = fminf(v, lane_xor<16>(v)); v = fminf(v, lane_xor<32>(v));
+    return v;
+}
+// sum with the far lanes first (32, 16, ... 1)
+__device__ __forceinline__ float wave_sum_far_first(float v) {
+    v += lane_xor<32>(v); v += lane_xor<16>(v); v += lane_xor<8>(v);
+    v += lane_xor<4>(v); v += lane_xor<2>(v); v += lane_xor<1>(v);
     return v;
 }
 

@@ -209,8 +209,7 @@ __global__ __launch_bounds__(EW_THREADS) void absmax_kernel(float *__restrict__ 
     } else {
         for (size_t i = tid; i < n; i += stride) m = fmaxf(m, fabsf(x[i]));
     }
-#pragma unroll
-    for (int k = 1; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
+    m = wave_max(m);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -224,8 +223,7 @@ __global__ __launch_bounds__(1024) void scale_from_partials_kernel(float *scale,
     __shared__ float red[16];
     float m = 0.f;
     for (int i = threadIdx.x; i < nblk; i += 1024) m = fmaxf(m, part[i]);
-#pragma unroll
-    for (int k = 1; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
+    m = wave_max(m);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -256,11 +254,8 @@ __global__ __launch_bounds__(EW_THREADS) void minmax_kernel(float *__restrict__ 
     } else {
         for (size_t i = tid; i < n; i += stride) { lo = fminf(lo, x[i]); hi = fmaxf(hi, x[i]); }
     }
-#pragma unroll
-    for (int k = 1; k < 64; k <<= 1) {
-        lo = fminf(lo, __shfl_xor(lo, k, 64));
-        hi = fmaxf(hi, __shfl_xor(hi, k, 64));
-    }
+    lo = wave_min(lo);
+    hi = wave_max(hi);
     if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = lo; red[1][threadIdx.x >> 6] = hi; }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -274,11 +269,8 @@ __global__ __launch_bounds__(1024) void minmax_final_kernel(float *out, const fl
     __shared__ float red[2][16];
     float lo = INFINITY, hi = -INFINITY;
     for (int i = threadIdx.x; i < nblk; i += 1024) { lo = fminf(lo, part[2 * i]); hi = fmaxf(hi, part[2 * i + 1]); }
-#pragma unroll
-    for (int k = 1; k < 64; k <<= 1) {
-        lo = fminf(lo, __shfl_xor(lo, k, 64));
-        hi = fmaxf(hi, __shfl_xor(hi, k, 64));
-    }
+    lo = wave_min(lo);
+    hi = wave_max(hi);
     if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = lo; red[1][threadIdx.x >> 6] = hi; }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -345,8 +337,7 @@ __global__ __launch_bounds__(EW_THREADS) void quant_dyn_kernel(int *__restrict__
     if (threadIdx.x < 64) {
         float m = 0.f;
         for (int i = threadIdx.x; i < nblk; i += 64) m = fmaxf(m, part[i]);
-#pragma unroll
-        for (int k = 1; k < 64; k <<= 1) m = fmaxf(m, __shfl_xor(m, k, 64));
+        m = wave_max(m);
         if (threadIdx.x == 0) red = m;
     }
     __syncthreads();

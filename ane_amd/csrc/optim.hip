@@ -33,8 +33,7 @@ __global__ __launch_bounds__(OPT_THREADS) void sumsq_partial_kernel(float *__res
         for (size_t i = tid; i < n; i += stride) { float t = g[i] * pre; s0 += t * t; }
     }
     float s = (s0 + s1) + (s2 + s3);
-#pragma unroll
-    for (int k = 32; k >= 1; k >>= 1) s += __shfl_xor(s, k, 64);
+    s = wave_sum_far_first(s);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
     __syncthreads();
     if (threadIdx.x == 0) part[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
@@ -133,8 +132,7 @@ __global__ __launch_bounds__(OPT_THREADS) void sumsq_partial_mt_kernel(float *__
     if (blockIdx.x == 0)
         for (size_t i = n4 * 4 + threadIdx.x; i < n; i += OPT_THREADS) { float t = g[i] * pre; s0 += t * t; }
     float s = (s0 + s1) + (s2 + s3);
-#pragma unroll
-    for (int k = 32; k >= 1; k >>= 1) s += __shfl_xor(s, k, 64);
+    s = wave_sum_far_first(s);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
     __syncthreads();
     if (threadIdx.x == 0) part[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
