@@ -42,6 +42,20 @@ bool mi355_ready(const char *who);
 bool mi355_outside_capture(const char *who);
 // Workspace of at least `bytes` (256-byte aligned), NULL on failure.
 void *mi355_ws(size_t bytes);
+// Exchange area for kernels whose workgroups pass values to one another inside one launch (the clustered
+// RMSNorm, the single-launch INT8 scale): 8-byte slots {fp32 value, tag}, XCH_SLOT_STRIDE per workgroup number, and
+// one launch counter per workgroup number; norm_cluster.h describes the protocol.  Allocated and zeroed on first
+// use (not possible during a graph capture); false with the error recorded on failure.
+constexpr int XCH_SLOT_STRIDE = 128;
+constexpr int XCH_MAX_BLOCKS = 2048;
+struct Mi355Exchange {
+    unsigned long long *slots;     // [XCH_MAX_BLOCKS][XCH_SLOT_STRIDE]
+    unsigned *cnt;                 // [XCH_MAX_BLOCKS] launches completed by each workgroup number
+    int *fallbacks;                // workgroups whose bounded wait expired, ever (diagnostic)
+};
+bool mi355_exchange(Mi355Exchange *out);
+// Ticks of the 100 MHz clock that such a kernel waits for a partner before it does the partner's work itself.
+int mi355_exchange_spin_ticks(void);
 // Runs every queued weight-gradient reduction (dw_reduce.hip).
 extern "C" int mi355_dw_flush(void);
 

@@ -54,6 +54,33 @@ void *mi355_ws(size_t bytes) {
     return p;
 }
 
+static Mi355Exchange g_xch = {nullptr, nullptr, nullptr};
+
+bool mi355_exchange(Mi355Exchange *out) {
+    if (!g_xch.slots) {
+        if (!mi355_outside_capture("first use of a kernel whose workgroups exchange partial results (its exchange area "
+                                   "is allocated)"))
+            return false;
+        const size_t slot_b = (size_t)XCH_MAX_BLOCKS * XCH_SLOT_STRIDE * sizeof(unsigned long long);
+        const size_t cnt_b = (size_t)XCH_MAX_BLOCKS * sizeof(unsigned);
+        char *p = nullptr;
+        hipError_t e = hipMalloc((void **)&p, slot_b + cnt_b + 256);
+        if (e != hipSuccess) { mi355_fail("exchange area hipMalloc: %s", hipGetErrorString(e)); return false; }
+        // tags and counters must start equal: all zero
+        e = hipMemsetAsync(p, 0, slot_b + cnt_b + 256, g_ctx.stream);
+        if (e != hipSuccess) { (void)hipFree(p); mi355_fail("exchange area clear: %s", hipGetErrorString(e)); return false; }
+        g_xch.slots = (unsigned long long *)p;
+        g_xch.cnt = (unsigned *)(p + slot_b);
+        g_xch.fallbacks = (int *)(p + slot_b + cnt_b);
+    }
+    *out = g_xch;
+    return true;
+}
+
+int mi355_exchange_spin_ticks(void) {
+    return g_ctx.rms_cluster_spin == 0 ? 200000 : (g_ctx.rms_cluster_spin < 0 ? 0 : g_ctx.rms_cluster_spin);
+}
+
 int mi355_ce_setup(void);        // softmax_ce.hip: locates its fixed scratch array on the current device
 
 MI355_API int mi355_init(void) {
@@ -85,7 +112,6 @@ void mi355_dw_free(void);       // queued weight-gradient reductions and their a
 void mi355_blas_free(void);     // rocBLAS handle of mi355_sgemm_dev
 void mi355_ckpt_free(void);     // pinned staging buffer of the checkpoint reader/writer
 void mi355_graph_shutdown(void);  // capture stream
-void mi355_norm_free(void);       // exchange area of the clustered RMSNorm
 
 MI355_API void mi355_shutdown(void) {
     if (!g_ctx.ready) return;
@@ -95,7 +121,8 @@ MI355_API void mi355_shutdown(void) {
     mi355_blas_free();
     mi355_ckpt_free();
     mi355_graph_shutdown();
-    mi355_norm_free();
+    if (g_xch.slots) (void)hipFree(g_xch.slots);
+    g_xch = Mi355Exchange{nullptr, nullptr, nullptr};
     if (g_ctx.ws) (void)hipFree(g_ctx.ws);
     g_ctx = Mi355Ctx{};
 }

@@ -218,6 +218,83 @@ __global__ __launch_bounds__(EW_THREADS) void absmax_kernel(float *__restrict__ 
     }
 }
 
+// The per-tensor scale in ONE launch: every workgroup publishes its maximum through the exchange area (an 8-byte
+// relaxed agent-scope atomic {value, launch tag}; the protocol is described in norm_cluster.h) and workgroup 0
+// gathers them and writes scale = max|x|/127 (1 for an all-zero tensor).  At most 1024 workgroups, one per compute
+// unit in practice, so all of them are resident together; if a maximum does not arrive within the bounded wait,
+// workgroup 0 takes the maximum of the whole tensor itself.  The maximum is exact in any order.
+// (Workgroup 0 reads the others' launch counters when it starts.  The others do not wait for it, so one that had
+// finished before workgroup 0 started would be taken for absent and cost the bounded wait; workgroups are
+// dispatched in index order and need microseconds for their share, so workgroup 0 is running long before.)
+__global__ __launch_bounds__(1024) void absmax_scale_kernel(float *__restrict__ scale, const float *__restrict__ x,
+                                                            size_t n, size_t n4, bool vec, Mi355Exchange ws,
+                                                            int spin_ticks) {
+    __shared__ float red[16];
+    __shared__ int failed;
+    const int nblk = (int)gridDim.x, blk = (int)blockIdx.x, t = (int)threadIdx.x;
+    if (t == 0) failed = 0;
+    unsigned want = 0;
+    if (blk == 0 && t < nblk) want = ws.cnt[t] + 1u;
+    const unsigned my_tag = ws.cnt[blk] + 1u;
+    auto tensor_max = [&](size_t first, size_t stride) {
+        float m = 0.f;
+        if (vec) {
+            for (size_t i = first; i < n4; i += stride) {
+                const v4f v = ld4_nt(x + 4 * i);
+#pragma unroll
+                for (int j = 0; j < 4; j++) m = fmaxf(m, fabsf(v[j]));
+            }
+            if (first < 1024)       // the few elements behind the last whole group of four
+                for (size_t i = n4 * 4 + first; i < n; i += 1024) m = fmaxf(m, fabsf(x[i]));
+        } else {
+            for (size_t i = first; i < n; i += stride) m = fmaxf(m, fabsf(x[i]));
+        }
+        return m;
+    };
+    auto block_max = [&](float m) {          // maximum over the workgroup, in every thread
+        m = wave_max(m);
+        __syncthreads();
+        if ((t & 63) == 0) red[t >> 6] = m;
+        __syncthreads();
+        float r = red[0];
+#pragma unroll
+        for (int k = 1; k < 16; k++) r = fmaxf(r, red[k]);
+        return r;
+    };
+    float m = block_max(tensor_max((size_t)blk * 1024 + t, (size_t)nblk * 1024));
+    if (t == 0)
+        __hip_atomic_store(&ws.slots[(size_t)blk * XCH_SLOT_STRIDE], ((unsigned long long)my_tag << 32) | __float_as_uint(m),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (blk == 0) {
+        float g = 0.f;
+        if (t < nblk) {
+            const unsigned long long *sp = &ws.slots[(size_t)t * XCH_SLOT_STRIDE];
+            const long long t0 = wall_clock64();
+            unsigned long long pk;
+            bool ok = false;
+            for (;;) {
+                pk = __hip_atomic_load(sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((unsigned)(pk >> 32) == want) { ok = true; break; }
+                if (wall_clock64() - t0 >= (long long)spin_ticks) break;
+                __builtin_amdgcn_s_sleep(2);
+            }
+            if (!ok) failed = 1;
+            g = __uint_as_float((unsigned)pk);
+        }
+        g = block_max(g);
+        if (failed) {
+            if (t == 0) atomicAdd(ws.fallbacks, 1);
+            g = block_max(tensor_max((size_t)t, 1024));
+        }
+        if (t == 0) {
+            float s = g / 127.0f;
+            if (s == 0.0f) s = 1.0f;
+            *scale = s;
+        }
+    }
+    if (t == 0) ws.cnt[blk] = my_tag;
+}
+
 __global__ __launch_bounds__(1024) void scale_from_partials_kernel(float *scale, const float *__restrict__ part,
                                                                    int nblk) {
     __shared__ float red[16];
@@ -637,12 +714,16 @@ MI355_API int mi355_int8_scale_dev(float *scale_dev, const float *x, size_t n) {
     if (n == 0) return mi355_fail("int8_scale: empty tensor");
     const bool vec = aligned16(x);
     const size_t n4 = vec ? n / 4 : 0;
-    size_t blocks = ceil_div(vec ? (n4 ? n4 : 1) : n, (size_t)EW_THREADS);
-    if (blocks > 4096) blocks = 4096;
-    float *part = (float *)mi355_ws(blocks * sizeof(float));
-    if (!part) return -1;
-    hipLaunchKernelGGL(absmax_kernel, dim3((unsigned)blocks), dim3(EW_THREADS), 0, g_ctx.stream, part, x, n, n4, vec);
-    hipLaunchKernelGGL(scale_from_partials_kernel, dim3(1), dim3(1024), 0, g_ctx.stream, scale_dev, part, (int)blocks);
+    // one workgroup of 1024 threads per compute unit, fewer for small tensors (at least 4 accesses per thread)
+    const size_t per_block = (size_t)1024 * 4;
+    size_t blocks = ceil_div(vec ? (n4 ? n4 : 1) : n, per_block);
+    const size_t cus = g_ctx.num_cu > 0 ? (size_t)g_ctx.num_cu : 256;
+    if (blocks > cus) blocks = cus;
+    if (blocks > 1024) blocks = 1024;
+    Mi355Exchange xch;
+    if (!mi355_exchange(&xch)) return -1;
+    hipLaunchKernelGGL(absmax_scale_kernel, dim3((unsigned)blocks), dim3(1024), 0, g_ctx.stream, scale_dev, x, n, n4, vec, xch,
+                       mi355_exchange_spin_ticks());
     LAUNCH_OK("int8_scale");
     return 0;
 }

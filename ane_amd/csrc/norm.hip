@@ -470,9 +470,9 @@ NormCfg plan_tile(int op, int C, int S, int batch, bool vec_ok) {
         }                                                                                             \
     } while (0)
 
-int cluster_spin_ticks(void) {
-    return g_ctx.rms_cluster_spin == 0 ? 200000 : (g_ctx.rms_cluster_spin < 0 ? 0 : g_ctx.rms_cluster_spin);
-}
+int cluster_spin_ticks(void) { return mi355_exchange_spin_ticks(); }
+ClusterWs g_cluster_ws = {nullptr, nullptr, nullptr};
+bool cluster_ws_ready(void) { return mi355_exchange(&g_cluster_ws); }
 
 // The single-workgroup tiles are chosen by hand (knobs) or the shape does not cluster: csplit == 0.
 ClusterPlan plan_cluster(int C, int S, int batch, bool vec_ok, int max_rpt) {

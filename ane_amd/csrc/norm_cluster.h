@@ -32,15 +32,11 @@ namespace {
 
 constexpr int CL_LPR = 16;                 // lanes per row piece: 16 x 16 B = 256 B
 constexpr int CL_W = CL_LPR * 4;           // columns per strip
-constexpr int CL_SLOT_STRIDE = 2 * CL_W;   // 8-byte slots per workgroup: two quantities per column
-constexpr int CL_MAX_BLOCKS = 2048;        // workgroups per launch that the slot area covers
+constexpr int CL_SLOT_STRIDE = XCH_SLOT_STRIDE;   // 8-byte slots per workgroup: two quantities per column
+constexpr int CL_MAX_BLOCKS = XCH_MAX_BLOCKS;     // workgroups per launch that the slot area covers
 constexpr int CL_MAX_SPLIT = 8;
-
-struct ClusterWs {
-    unsigned long long *slots;     // [CL_MAX_BLOCKS][CL_SLOT_STRIDE] {fp32 value, tag}
-    unsigned *cnt;                 // [CL_MAX_BLOCKS] launches completed by each workgroup number
-    int *fallbacks;                // number of workgroups that gave up waiting, ever (diagnostic)
-};
+static_assert(CL_SLOT_STRIDE >= 2 * CL_W, "two quantities per column must fit a workgroup's slots");
+typedef Mi355Exchange ClusterWs;
 
 // Per-thread partial sums acc[q][j] (q < NV quantities, j < 4 columns of this lane) -> per-column sums of the
 // workgroup in wsum[q*CL_W + column], valid for all threads after the barrier.  lds: NW*NV*CL_W floats.
@@ -365,25 +361,6 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_cluster_kernel(float *dx, flo
     if (threadIdx.x == 0) ws.cnt[g.blk] = my_tag;
 }
 
-ClusterWs g_cluster_ws = {nullptr, nullptr, nullptr};
-
-// The slot area, allocated and cleared on first use (tags and counters must start equal: all zero).
-bool cluster_ws_ready(void) {
-    if (g_cluster_ws.slots) return true;
-    if (!mi355_outside_capture("first use of the clustered RMSNorm (its exchange area is allocated)")) return false;
-    const size_t slot_b = (size_t)CL_MAX_BLOCKS * CL_SLOT_STRIDE * sizeof(unsigned long long);
-    const size_t cnt_b = (size_t)CL_MAX_BLOCKS * sizeof(unsigned);
-    char *p = nullptr;
-    hipError_t e = hipMalloc((void **)&p, slot_b + cnt_b + 256);
-    if (e != hipSuccess) { mi355_fail("cluster exchange area hipMalloc: %s", hipGetErrorString(e)); return false; }
-    e = hipMemsetAsync(p, 0, slot_b + cnt_b + 256, g_ctx.stream);
-    if (e != hipSuccess) { (void)hipFree(p); mi355_fail("cluster exchange area clear: %s", hipGetErrorString(e)); return false; }
-    g_cluster_ws.slots = (unsigned long long *)p;
-    g_cluster_ws.cnt = (unsigned *)(p + slot_b);
-    g_cluster_ws.fallbacks = (int *)(p + slot_b + cnt_b);
-    return true;
-}
-
 // How a shape is split: csplit members of rows_pm rows each; rpt rows per lane.  csplit = 0: not clustered.
 struct ClusterPlan {
     int csplit, rows_pm, rpt, threads, strips, nblk;
@@ -423,8 +400,3 @@ ClusterPlan cluster_plan(int C, int S, int batch, bool vec_ok, int max_rpt) {
 }
 
 }   // namespace
-
-void mi355_norm_free(void) {
-    if (g_cluster_ws.slots) (void)hipFree(g_cluster_ws.slots);
-    g_cluster_ws = ClusterWs{nullptr, nullptr, nullptr};
-}

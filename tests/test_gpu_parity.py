@@ -606,6 +606,27 @@ def test_int8_quantize_dynamic_equals_scale_then_quant(br, n, rounding):
     assert s2.numpy()[0] == 1.0 and not q2.numpy()[:min(n, 64)].any()
 
 
+@pytest.mark.parametrize("n", [1024 * 4096, 4099, 5, 3 * 1024 * 1024 + 1])
+def test_int8_scale_single_launch_and_its_expired_wait(br, n):
+    """The scale comes from one launch whose workgroups hand their maxima to workgroup 0; with the bounded wait set
+    to expire at once workgroup 0 takes the maximum itself.  Same bits either way, also on an unaligned tensor."""
+    x = H.normal(140, n + 1) * np.float32(2.5)
+    x[n // 2] = np.float32(-123.25)
+    xd = dev(br, x); sd = br.DevArray(1)
+    try:
+        for spin in (0, -1):
+            br.tune("rms_cluster_spin", spin)
+            for off in (0, 1):                       # off = 1: the address is not 16-byte aligned (scalar path)
+                sd.upload(np.zeros(1, np.float32))
+                br.check(br.lib.mi355_int8_scale_dev(sd.ptr, xd.ptr + 4 * off, n))
+                assert sd.numpy()[0] == np.float32(O.int8_scale(x[off:off + n])), (spin, off)
+    finally:
+        br.tune("rms_cluster_spin", 0)
+    z = dev(br, np.zeros(4096, np.float32))
+    br.check(br.lib.mi355_int8_scale_dev(sd.ptr, z.ptr, 4096))
+    assert sd.numpy()[0] == 1.0
+
+
 @pytest.mark.parametrize("n", [1024 * 4096, 2048 * 256 * 16, 13, 1, 4099])
 def test_minmax_exact(br, n):
     say("minmax n=%d" % n)
