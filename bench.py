@@ -30,10 +30,18 @@ PEAK_HBM_GBS = 8000.0      # MI355X published HBM3E peak
 # HBM-side bytes per dispatch of the dominant kernel at the default workload, from the two rocprofv3 --pmc
 # runs summarised in profiles/qwen3_sweep_pmc_fetch_write.md (FETCH_SIZE x 1.9992 + WRITE_SIZE x 0.9992, the
 # factors the same counters need to read 50.33 MB for a plain 50.33 MB copy).  Not measured live.
-MEASURED_TRAFFIC_BYTES = {"swiglu_bwd": 251.56e6}
-# the same for the three launches of the ordered scatter-add at BASELINE.json config 2
-# (profiles/embed_config2_pmc_fetch_write.md)
-SCATTER_TRAFFIC_BYTES = 176.14e6
+MEASURED_TRAFFIC_BYTES = {"swiglu_bwd": 251.60e6}
+# the same for the three launches of softmax-CE on [151936,256] (partials 156.62 + combine 2.06 + gradient 311.39 MB:
+# the logits are read twice), and per op of the sweep (same profile)
+CE_TRAFFIC_BYTES = 470.07e6
+OP_TRAFFIC_BYTES = {"rmsnorm_fwd": 34.04e6, "rmsnorm_bwd": 51.43e6 + 1.62e6 / 2, "qknorm_rope_fwd": 100.99e6,
+                    "qknorm_rope_bwd": 152.08e6, "swiglu_fwd": 150.97e6, "swiglu_bwd": 251.60e6, "residual": 50.33e6,
+                    "residual_rmsnorm_fwd": 67.64e6, "rmsnorm_bwd_residual": 85.04e6, "scale_copy": 100.66e6,
+                    "softmax_ce": CE_TRAFFIC_BYTES, "int8_scale": 16.91e6, "int8_quant": 20.99e6, "int8_dequant": 20.99e6}
+# the same for BASELINE.json config 2 (profiles/embed_config2_pmc_fetch_write.md): the three launches of the ordered
+# scatter-add (chunk sort 0.16 + ranks and transpose 101.70 + segment sums 74.32 MB) and the gather
+SCATTER_TRAFFIC_BYTES = 176.18e6
+GATHER_TRAFFIC_BYTES = 70.14e6
 
 # Qwen3-0.6B (training/training_dynamic/models/qwen3_06b.h:6-16), batch 16
 Q3 = dict(C=1024, H=3072, heads=16, kv_heads=8, hd=128, S=256, batch=16, layers=28, V=151936, theta=1e6,
@@ -61,6 +69,7 @@ def alg_bytes(cfg, a=4):
         "swiglu_bwd": 5 * a * H * St,
         "residual": 3 * a * C * St,
         "scale_copy": 2 * a * H * St,        # y = alpha*a over an [H,St] tensor: a plain copy-shaped stream (train.m:523,595)
+        "copy, bytes of rmsnorm_fwd": 2 * a * C * St,     # the same over [C,St]: the streaming rate at the size of the small ops
         # residual + the RMSNorm after it in one launch; as two ops the same work is 12CSt + 8CSt + 4C
         "residual_rmsnorm_fwd": 4 * a * C * St + 4 * C,
         # RMSNorm backward + the backward residual + the scaled copy in one launch (train.m:586-595); as three ops
@@ -210,6 +219,8 @@ class Workload:
                                                   self.alpha, d["w_att"].ptr, C, S, B, 1e-5))
         elif name == "scale_copy":     # dffn = alpha*dy shaped stream over the SwiGLU-sized buffers
             ck(lib.mi355_axpby_dev(self.scratch_h.ptr, d["dsilu"].ptr, None, self.alpha, n_h, 1))
+        elif name == "copy_c":         # the same stream over an RMSNorm-sized tensor: what a plain copy of those bytes takes
+            ck(lib.mi355_axpby_dev(self.scratch_c.ptr, d["x"].ptr, None, self.alpha, n_c, 1))
         elif name == "swiglu_fwd":
             ck(lib.mi355_swiglu_fwd_dev(d["gate"].ptr, d["h1"].ptr, d["h3"].ptr, n_h))
         elif name == "residual2":
@@ -288,7 +299,7 @@ def per_op_table(br, wl, reps):
     names = {"rmsnorm_fwd": "rmsnorm_fwd", "rmsnorm_bwd": "rmsnorm_bwd", "qknorm_rope_fwd": "qknorm_rope_fwd",
              "qknorm_rope_bwd": "qknorm_rope_bwd", "swiglu_fwd": "swiglu_fwd", "swiglu_bwd": "swiglu_bwd",
              "residual1": "residual", "res_rms1": "residual_rmsnorm_fwd", "rms_bwd_res": "rmsnorm_bwd_residual",
-             "scale_copy": "scale_copy"}
+             "scale_copy": "scale_copy", "copy_c": "copy, bytes of rmsnorm_fwd"}
     table = []
     if wl.bf16:
         del names["res_rms1"]          # the fused residual + RMSNorm ops exist for fp32 storage only
@@ -443,7 +454,6 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
     copy()
     t_c = time_region(br, copy, steps) / nbuf
     b_g = 8 * D * N + 4 * N                 # the definition's bytes: every gathered row read once, written once
-    b_g_moved = 4 * D * U + 4 * D * N + 4 * N   # what has to cross HBM: each distinct row once, the output, the ids
     b_s = 4 * D * N + 8 * D * U + 4 * N
     row = lambda op, ms, nbytes, **kw: dict(op=op, ms=ms, alg_mb=nbytes / 1e6, gbs=nbytes / ms / 1e6,
                                             frac=nbytes / ms / 1e6 / PEAK_HBM_GBS, **kw)
@@ -452,9 +462,13 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32+i32", "data": "synthetic",
            "config": {"workload": "embedding table [32000,768] fp32, 64x256 Zipf(1.1) ids, seed 0", "unique_ids": U,
                       "hottest_id_count": int(np.bincount(ids.ravel()).max())},
-           "ops": [row("embed_gather", t_g, b_g, hbm_mb=b_g_moved / 1e6, hbm_frac=b_g_moved / t_g / 1e6 / PEAK_HBM_GBS,
-                       note="alg_mb counts every gathered row; hbm_mb counts each distinct row once (the rest are cache hits)"),
+           "ops": [row("embed_gather", t_g, b_g, traffic_mb=GATHER_TRAFFIC_BYTES / 1e6,
+                       traffic_frac=GATHER_TRAFFIC_BYTES / t_g / 1e6 / PEAK_HBM_GBS,
+                       note="alg_mb counts every gathered row as read; the %d distinct rows are re-read from cache, so the "
+                            "bytes that move (traffic_mb, rocprofv3 counters) are fewer and traffic_frac is the roofline "
+                            "figure" % U),
                    row("embed_scatter_add", t_s, b_s, traffic_mb=SCATTER_TRAFFIC_BYTES / 1e6,
+                       traffic_frac=SCATTER_TRAFFIC_BYTES / t_s / 1e6 / PEAK_HBM_GBS,
                        traffic_source="profiles/embed_config2_pmc_fetch_write.md"),
                    row("embed_scatter_add (scatter_tree=1)", t_s_tree, b_s),
                    row("copy of one activation slab", t_c, 8 * D * N)],
@@ -772,6 +786,13 @@ def main():
                     traffic_source="profiles/qwen3_sweep_pmc_fetch_write.md", alg_bytes_per_launch=ab[dom["op"]],
                     avg_launch_ms=dom["ms"])
 
+    if (cfg["name"], cfg["batch"], bf16) == ("qwen3-0.6b", 16, False):
+        # HBM-side bytes per launch from the committed rocprofv3 counter runs, next to the algorithmic bytes
+        for r in table:
+            tb = OP_TRAFFIC_BYTES.get(r["op"])
+            if tb:
+                r["traffic_mb"] = tb / 1e6
+                r["traffic_frac"] = tb / r["ms"] / 1e6 / PEAK_HBM_GBS
     out = {
         "metric": "layer-op tokens/s at %s shape (fused-op HBM GB/s and %% of peak in `ops`)" % (
             "Qwen3-0.6B" if cfg["name"] == "qwen3-0.6b" else "Stories110M"),
