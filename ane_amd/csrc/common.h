@@ -97,9 +97,10 @@ __device__ __forceinline__ v4f ld4_nt(const float *p) {
     return __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
 }
 
-// Value of lane (l ^ M) of a wave64, through the cheapest path the ISA has for each distance: a DPP quad permute
-// inside the adder for 1 and 2, ds_swizzle in bit-mask mode (the LDS crossbar, no address register, no LDS memory)
-// for 4, 8 and 16, v_permlane32_swap for 32.
+// Value of lane (l ^ M) of a wave64, through the cheapest path measured for each distance: a DPP quad permute inside
+// the adder for 1 and 2, ds_bpermute for 4, 8 and 16, v_permlane32_swap for 32.  (ds_swizzle in bit-mask mode also
+// reaches 4, 8 and 16, without an address register, but the 16-wave RMSNorm tile ran 0.2-0.3 us slower with it
+// than with ds_bpermute: 10.4-10.7 against 10.0-10.5 us; v_permlane32_swap and ds_bpermute were equal for 32.)
 template <int M>
 __device__ __forceinline__ float lane_xor(float v) {
     static_assert(M == 1 || M == 2 || M == 4 || M == 8 || M == 16 || M == 32, "lane distance");
@@ -107,9 +108,7 @@ __device__ __forceinline__ float lane_xor(float v) {
     int r;
     if constexpr (M == 1) r = __builtin_amdgcn_update_dpp(0, iv, 0xB1, 0xF, 0xF, true);          // quad_perm:[1,0,3,2]
     else if constexpr (M == 2) r = __builtin_amdgcn_update_dpp(0, iv, 0x4E, 0xF, 0xF, true);     // quad_perm:[2,3,0,1]
-    else if constexpr (M == 4) r = __builtin_amdgcn_ds_swizzle(iv, (4 << 10) | 0x1F);            // swizzle(SWAP,4)
-    else if constexpr (M == 8) r = __builtin_amdgcn_ds_swizzle(iv, (8 << 10) | 0x1F);
-    else if constexpr (M == 16) r = __builtin_amdgcn_ds_swizzle(iv, (16 << 10) | 0x1F);
+    else if constexpr (M == 4 || M == 8 || M == 16) return __shfl_xor(v, M, 64);                 // ds_bpermute_b32
     else {
         typedef unsigned lane_pair __attribute__((ext_vector_type(2)));
         // {v with its upper half replaced by the lower half, v with its lower half replaced by the upper half}

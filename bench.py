@@ -841,7 +841,7 @@ def main():
             wl1.step()
         br.sync()
         ms1 = time_region(br, wl1.step, args.steps)
-        tab1 = per_op_table(br, wl1, args.op_reps)
+        tab1 = [r for r in per_op_table(br, wl1, args.op_reps) if not r["op"].startswith("int8")]   # (same tensor as above)
         other["stories110m_configs_0_1"] = {
             "workload": "the same sweep at the Stories110M shapes (BASELINE.json configs 0/1): 12 layers, one [C,256] "
                         "sequence per op (the reference's calling pattern), RoPE theta 1e4 without QK-norm, "

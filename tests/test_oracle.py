@@ -101,6 +101,28 @@ def test_rmsnorm_bwd_golden_and_variants():
     a, _ = O.rmsnorm_bwd(dy, x, one, variant=0)
     b, _ = O.rmsnorm_bwd(dy, x, one, variant=1)
     assert H.rel_err(a, b) < 1e-6
+    # What the reference's operand order does to the exact gradient, derived from training/stories_cpu_ops.h:35-46
+    # without retyping its formula: it multiplies the whole bracket by w instead of dy alone, so
+    #   variant0 = variant1 + x * (1 - w) * (rr^2 / C) * sum_c dy*y,   y = the forward output, rr^2 = 1/(mean x^2 + eps).
+    # Variant 1 is pinned by finite differences below and y by the forward tests, so a dropped term, a wrong sign or
+    # a misplaced w in the oracle's variant 0 fails here.
+    x64, dy64, w64 = x.astype(np.float64), dy.astype(np.float64), w.astype(np.float64)
+    y64 = O.rmsnorm(x, w).astype(np.float64)
+    rr2 = 1.0 / (np.mean(x64 * x64, axis=0, keepdims=True) + 1e-5)
+    corr = x64 * (1.0 - w64)[:, None] * (rr2 / x.shape[0]) * np.sum(dy64 * y64, axis=0, keepdims=True)
+    assert H.rel_err(dx0, dx1.astype(np.float64) + corr) < 1e-5
+    assert np.max(np.abs(corr)) > 1e-3 * np.max(np.abs(dx1))            # the correction is not a rounding artefact
+    # and variant 1 with dw against central differences of L = sum dy * rmsnorm(x, w), at a few entries
+    def loss(xx, ww):
+        return float(np.sum(dy64 * H.np_rmsnorm(xx, ww)))
+    h = 1e-5
+    rng = np.random.default_rng(5)
+    for _ in range(6):
+        c, t = int(rng.integers(x.shape[0])), int(rng.integers(x.shape[1]))
+        xp, xm = x64.copy(), x64.copy(); xp[c, t] += h; xm[c, t] -= h
+        assert abs((loss(xp, w64) - loss(xm, w64)) / (2 * h) - dx1[c, t]) < 2e-4 * max(1.0, abs(dx1[c, t]))
+        wp, wm = w64.copy(), w64.copy(); wp[c] += h; wm[c] -= h
+        assert abs((loss(x64, wp) - loss(x64, wm)) / (2 * h) - dw0[c]) < 2e-4 * max(1.0, abs(dw0[c]))
 
 
 def test_rmsnorm_bwd_assigns_dx_accumulates_dw_over_batch():
