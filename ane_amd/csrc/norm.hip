@@ -475,9 +475,9 @@ ClusterWs g_cluster_ws = {nullptr, nullptr, nullptr};
 bool cluster_ws_ready(void) { return mi355_exchange(&g_cluster_ws); }
 
 // The single-workgroup tiles are chosen by hand (knobs) or the shape does not cluster: csplit == 0.
-ClusterPlan plan_cluster(int C, int S, int batch, bool vec_ok, int max_rpt) {
+ClusterPlan plan_cluster(int C, int S, int batch, bool vec_ok, int max_rpt, int rounds = 1) {
     if (g_ctx.rms_lpr || g_ctx.rms_threads) return ClusterPlan{0, 0, 0, 0, 0, 0, false};
-    return cluster_plan(C, S, batch, vec_ok, max_rpt);
+    return cluster_plan(C, S, batch, vec_ok, max_rpt, rounds);
 }
 
 template <int RPT, bool FUSE, bool EXACT>
@@ -519,11 +519,20 @@ void launch_bwd_cluster(const ClusterPlan &cp, float *dx, float *part, const flo
 }   // namespace
 
 // Host-only: which tile an entry point would run for a shape, and whether that tile exists.
-MI355_API int mi355_rmsnorm_tile(int op, int C, int S, int batch, int aligned, int *tile4) {
+MI355_API int mi355_rmsnorm_tile(int op, int C, int S, int batch, int aligned, int *tile5) {
     if (op < 0 || op > 2 || C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_tile: bad arguments");
-    const NormCfg cfg = plan_tile(op, C, S, batch, aligned && S % 4 == 0);
-    if (tile4) { tile4[0] = cfg.vec; tile4[1] = cfg.lpr; tile4[2] = cfg.threads; tile4[3] = cfg.cap; }
+    const bool vec_ok = aligned && S % 4 == 0;
+    // the single-workgroup tile is also what an in-place call of a clustered shape runs: it has to exist either way
+    const NormCfg cfg = plan_tile(op, C, S, batch, vec_ok);
     if (!norm_tile_exists(cfg)) return mi355_fail("rmsnorm: no kernel for tile key %d", norm_key(cfg));
+    const ClusterPlan cp = plan_cluster(C, S, batch, vec_ok, op == 0 ? 8 : 4, op == 2 ? 2 : 1);
+    if (tile5) {
+        if (cp.csplit) { tile5[0] = 4; tile5[1] = CL_LPR; tile5[2] = cp.threads; tile5[3] = cp.rpt; tile5[4] = cp.csplit; }
+        else { tile5[0] = cfg.vec; tile5[1] = cfg.lpr; tile5[2] = cfg.threads; tile5[3] = cfg.cap; tile5[4] = 0; }
+    }
+    if (cp.csplit && (cp.nblk > CL_MAX_BLOCKS || cp.rows_pm > (cp.threads / CL_LPR) * cp.rpt || (cp.rpt != 4 && cp.rpt != 8) ||
+                      (op != 0 && cp.rpt != 4)))
+        return mi355_fail("rmsnorm: inconsistent cluster plan for C=%d S=%d batch=%d", C, S, batch);
     return 0;
 }
 
@@ -590,7 +599,7 @@ MI355_API int mi355_rmsnorm_bwd_residual_dev(float *dx, float *dx_scaled, float 
     if (dx == x) return mi355_fail("rmsnorm_bwd_residual: dx must not alias x (dx may alias res or dy)");
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(res) &&
                         (!dx_scaled || aligned16(dx_scaled));
-    const ClusterPlan cp = dx == dy ? ClusterPlan{0, 0, 0, 0, 0, 0, false} : plan_cluster(C, S, batch, vec_ok, 4);
+    const ClusterPlan cp = dx == dy ? ClusterPlan{0, 0, 0, 0, 0, 0, false} : plan_cluster(C, S, batch, vec_ok, 4, 2);
     if (cp.csplit) {
         if (!cluster_ws_ready()) return -1;
         const int nrows = cp.nblk / cp.csplit;

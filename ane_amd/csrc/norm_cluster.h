@@ -368,8 +368,12 @@ struct ClusterPlan {
 };
 
 // Clustering pays when whole-C strips of 64 columns would leave most compute units idle: tall tensors
-// (C >= 512) whose 64-column strips number fewer than the compute units.
-ClusterPlan cluster_plan(int C, int S, int batch, bool vec_ok, int max_rpt) {
+// (C >= 512) whose 64-column strips number fewer than the compute units.  Measured at C = 1024 with 32 x 256 and
+// 64 x 256 columns: a launch of more workgroups than compute units (two rounds of 1024-thread workgroups) loses to
+// the single-workgroup tiles with 128-byte strips (forward 30.0 against 29.1 us, backward 22.3 against 19.9 us),
+// except for the backward with the residual, whose single-workgroup tile is the weakest (32.7 against 43.7 us).
+// rounds: how many workgroups per compute unit a launch may have (1: all resident at once).
+ClusterPlan cluster_plan(int C, int S, int batch, bool vec_ok, int max_rpt, int rounds) {
     ClusterPlan p = {0, 0, 0, 0, 0, 0, false};
     if (!vec_ok || C < 512 || g_ctx.rms_cluster < 0) return p;
     const long strips = (long)ceil_div((size_t)S, CL_W);
@@ -378,7 +382,7 @@ ClusterPlan cluster_plan(int C, int S, int batch, bool vec_ok, int max_rpt) {
     const int threads = 1024, rps = threads / CL_LPR;
     int split = 0;
     for (int s = 2; s <= CL_MAX_SPLIT; s *= 2) {
-        if (clusters * s > CL_MAX_BLOCKS || clusters * s > 2L * cus) break;
+        if (clusters * s > CL_MAX_BLOCKS || clusters * s > (long)rounds * cus) break;
         const int rows = (int)ceil_div((size_t)C, (size_t)s);
         if (rows > rps * max_rpt) continue;                      // does not fit the registers yet: split further
         split = s;

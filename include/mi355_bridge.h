@@ -112,8 +112,9 @@ int mi355_qknorm_rope_bwd_bf16_dev(uint16_t *dq, uint16_t *dk, float *dwq, float
 /* Graphs: record a launch-bound sequence of device-resident ops once, replay it as one submission.  No
  * counterpart in the reference (its ops are synchronous CPU calls).  Between begin and end the *_dev ops are
  * recorded instead of run; calls that allocate, wait or touch the host (buf_alloc/free/read/write, sync,
- * set_stream, workspace growth, a first-time RoPE table, embed_scatter_add beyond 16384 positions, sgemm,
- * ckpt_*) fail with -1 and end in a failed capture, so run the sequence once eagerly first.  mi355_graph_launch
+ * set_stream, workspace growth, a first-time RoPE table, the first clustered RMSNorm or INT8 scale of the process
+ * (their exchange area is allocated then), embed_scatter_add beyond 16384 positions, sgemm, ckpt_*, the
+ * host-pointer drop-ins) fail with -1 and end in a failed capture, so run the sequence once eagerly first.  mi355_graph_launch
  * enqueues the replay on the bridge stream; it fails if a workspace was reallocated since the recording (record
  * again).  Accumulating ops (dw +=) accumulate on every replay. */
 typedef struct mi355_graph mi355_graph;
@@ -154,10 +155,11 @@ int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const float *x,
 
 /* Introspection, host-only (needs no GPU): the register tile that the RMSNorm entry points choose for a shape —
  * op 0 = mi355_rmsnorm_fwd_dev, 1 = mi355_rmsnorm_bwd_dev, 2 = mi355_rmsnorm_bwd_residual_dev; aligned != 0 means
- * 16-byte aligned tensors.  tile4 (may be NULL) receives {columns per lane, lanes per row segment, threads per
- * workgroup, rows per lane held in registers (0 = rows are read twice)}.  0, or -1 if no kernel exists for the
- * choice (a defect: the entry point would fail the same way). */
-int mi355_rmsnorm_tile(int op, int C, int S, int batch, int aligned, int *tile4);
+ * 16-byte aligned tensors.  tile5 (may be NULL) receives {columns per lane, lanes per row piece, threads per
+ * workgroup, rows per lane held in registers (0 = rows are read twice), workgroups that share the rows of one strip
+ * (0 = one workgroup owns all C rows; 2, 4 or 8 = the clustered kernels, which out-of-place calls of tall shapes
+ * run)}.  0, or -1 if no kernel exists for the choice (a defect: the entry point would fail the same way). */
+int mi355_rmsnorm_tile(int op, int C, int S, int batch, int aligned, int *tile5);
 
 /* Weight-gradient accumulation mode.  By default dw / dwq / dwk are up to date (in stream order) when
  * the backward call that adds into them returns.  The loops read these gradients only at the optimizer

@@ -22,6 +22,9 @@
 #ifndef MI355_CPU_OPS_H
 #define MI355_CPU_OPS_H
 
+#include <stdlib.h>
+#include <string.h>
+
 #include "mi355_bridge.h"
 
 #ifndef VOCAB
@@ -75,8 +78,6 @@ static inline void adam_update(float *w, const float *g, AdamState *s, int t, fl
  * freed by the caller.  The size of the full table, which the reference's vocab_compact_embed does not
  * take, comes from VOCAB.  Tokens >= full_vocab in the data, which the reference's scan would write out of
  * bounds for, are ignored.  If the GPU cannot be used compact_vocab is 0. */
-#include <stdlib.h>
-#include <string.h>
 typedef struct {
     int compact_vocab;          /* number of tokens that occur */
     int *full_to_compact;       /* [full_vocab] -> compact id, -1 if unused */

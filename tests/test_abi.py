@@ -71,7 +71,7 @@ def test_every_rmsnorm_shape_has_a_kernel():
     counts on both sides of its thresholds (including 128 x 256 columns, where 16-lane strips of 512 threads win),
     for all three entry points, aligned or not, and under every tuning knob."""
     import ane_amd.bridge as br
-    tile = (ctypes.c_int * 4)()
+    tile = (ctypes.c_int * 5)()
     shapes = [(256, 1), (256, 16), (256, 32), (256, 128), (256, 300), (64, 2), (37, 2), (20, 3), (4, 1), (1024, 64)]
     seen = set()
     try:
@@ -88,7 +88,10 @@ def test_every_rmsnorm_shape_has_a_kernel():
                             seen.add(tuple(tile))
     finally:
         br.lib.mi355_tune_set(b"rms_lpr", 0); br.lib.mi355_tune_set(b"rms_threads", 0)
-    assert (4, 16, 512, 8) in seen or (4, 16, 512, 16) in seen        # the tile that used to be missing
+    assert (4, 16, 512, 8, 0) in seen or (4, 16, 512, 16, 0) in seen  # the tile that used to be missing
+    assert br.lib.mi355_rmsnorm_tile(0, 1024, 256, 16, 1, tile) == 0 and tuple(tile) == (4, 16, 1024, 4, 4)   # Qwen3: 4 x 256 rows
+    assert br.lib.mi355_rmsnorm_tile(1, 768, 256, 1, 1, tile) == 0 and tile[4] == 8                           # Stories110M
+    assert br.lib.mi355_rmsnorm_tile(0, 1024, 256, 64, 1, tile) == 0 and tile[4] == 0                         # enough columns
     assert br.lib.mi355_rmsnorm_tile(3, 8, 8, 1, 1, None) == -1
 
 
