@@ -9,93 +9,13 @@
 // One lane handles 8 contiguous elements: one 128-bit access on the bf16 side.
 #include "common.h"
 #include "tile.h"
+#include "norm_cluster.h"
 
 #include <math.h>
 
 namespace {
 
-typedef uint16_t bf16_t;
-typedef unsigned int v4u __attribute__((ext_vector_type(4)));
-
 constexpr int BT = 256;
-
-__device__ __forceinline__ float bf_to_f(unsigned bits16) { return __uint_as_float(bits16 << 16); }
-// round to nearest even; NaN stays NaN (quiet bit forced)
-__device__ __forceinline__ unsigned f_to_bf(float f) {
-    const unsigned u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
-
-// VEC bf16 values -> VEC floats.  VEC = 8: one 128-bit access, element 2j in the low half of word j.
-template <int VEC, bool NT>
-__device__ __forceinline__ void ldb(float (&r)[VEC], const bf16_t *p) {
-    if constexpr (VEC == 8) {
-        const v4u *q = reinterpret_cast<const v4u *>(p);
-        const v4u w = NT ? __builtin_nontemporal_load(q) : *q;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            r[2 * j] = bf_to_f(w[j] & 0xffffu);
-            r[2 * j + 1] = bf_to_f(w[j] >> 16);
-        }
-    } else {
-        static_assert(VEC == 1, "bf16 rows are read 8 columns or 1 column at a time");
-        r[0] = bf_to_f(*p);
-    }
-}
-template <int VEC>
-__device__ __forceinline__ void stb(bf16_t *p, const float (&r)[VEC]) {
-    if constexpr (VEC == 8) {
-        v4u w;
-#pragma unroll
-        for (int j = 0; j < 4; j++) w[j] = f_to_bf(r[2 * j]) | (f_to_bf(r[2 * j + 1]) << 16);
-        __builtin_nontemporal_store(w, reinterpret_cast<v4u *>(p));
-    } else {
-        *p = (bf16_t)f_to_bf(r[0]);
-    }
-}
-
-// Register tiles keep the bf16 words packed (half the registers of an fp32 tile) and widen them at each use.
-template <int VEC> struct RawT { typedef unsigned type; };
-template <> struct RawT<8> { typedef v4u type; };
-template <int VEC, bool NT>
-__device__ __forceinline__ typename RawT<VEC>::type ld_raw(const bf16_t *p) {
-    if constexpr (VEC == 8) {
-        const v4u *q = reinterpret_cast<const v4u *>(p);
-        return NT ? __builtin_nontemporal_load(q) : *q;
-    } else {
-        return (unsigned)*p;
-    }
-}
-template <int VEC>
-__device__ __forceinline__ void unpack(float (&r)[VEC], const typename RawT<VEC>::type &w) {
-    if constexpr (VEC == 8) {
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            r[2 * j] = bf_to_f(w[j] & 0xffffu);
-            r[2 * j + 1] = bf_to_f(w[j] >> 16);
-        }
-    } else {
-        r[0] = bf_to_f(w);
-    }
-}
-// Tells the compiler nothing about the words' contents from here on, so that the widened copies made before a
-// reduction are dropped instead of being kept alive across it (they would double the register tile).
-template <int VEC>
-__device__ __forceinline__ void forget(typename RawT<VEC>::type &w) {
-    if constexpr (VEC == 8) {
-        unsigned a = w[0], b = w[1], c = w[2], d = w[3];
-        asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
-        w[0] = a; w[1] = b; w[2] = c; w[3] = d;
-    } else {
-        asm volatile("" : "+v"(w));
-    }
-}
-template <int VEC>
-__device__ __forceinline__ typename RawT<VEC>::type raw_zero() {
-    if constexpr (VEC == 8) { v4u z = {0u, 0u, 0u, 0u}; return z; }
-    else return 0u;
-}
 
 // ---- converts (rectangles, as the fp16 staging converts) ----
 template <int VEC>
@@ -675,6 +595,24 @@ BfCfg pick_bf(int C, bool vec_ok, int S, int batch) {
     return BfCfg{8, lpr, threads, 0};
 }
 
+// Clustered variants (norm_cluster.h, bf16 storage: strips of 128 columns, 2 or 4 rows per lane).  Not when the
+// single-workgroup tile is chosen by hand through the rms_lpr / rms_threads knobs.
+Mi355Exchange g_bf_cluster_ws = {nullptr, nullptr, nullptr};
+ClusterPlan plan_cluster_bf(int C, int S, int batch, bool vec_ok) {
+    if (g_ctx.rms_lpr || g_ctx.rms_threads) return NO_CLUSTER;
+    return cluster_plan(C, S, batch, vec_ok, StoreBf16::VEC, 2, 4, 1);
+}
+#define BF_CLUSTER_FWD(RPT, EXACT)                                                                                   \
+    hipLaunchKernelGGL((rms_fwd_cluster_kernel<StoreBf16, RPT, 1024, false, EXACT>), dim3(cp.nblk), dim3(1024), 0,   \
+                       g_ctx.stream, y, (uint16_t *)nullptr, x, (const uint16_t *)nullptr, 0.f, w, C, S, cp.strips,  \
+                       cp.nblk, cp.csplit, cp.rows_pm, eps, 1.0f / (float)C, g_bf_cluster_ws,                        \
+                       mi355_exchange_spin_ticks())
+#define BF_CLUSTER_BWD(RPT, EXACT)                                                                                   \
+    hipLaunchKernelGGL((rms_bwd_cluster_kernel<StoreBf16, RPT, 1024, false, EXACT>), dim3(cp.nblk), dim3(1024), 0,   \
+                       g_ctx.stream, dx, part, dy, x, w, C, S, cp.strips, cp.nblk, cp.csplit, cp.rows_pm, eps,       \
+                       1.0f / (float)C, variant, (const uint16_t *)nullptr, (uint16_t *)nullptr, 0.f,                \
+                       g_bf_cluster_ws, mi355_exchange_spin_ticks())
+
 #define BF_CASE(KERNEL, V, L, T, CP, nblk, ...)                                                                      \
     case (V) * 1000000 + (L) * 10000 + ((T) / 256) * 100 + (CP):                                                     \
         hipLaunchKernelGGL((KERNEL<V, L, T, CP>), dim3(nblk), dim3(T), 0, g_ctx.stream, __VA_ARGS__);                \
@@ -782,7 +720,20 @@ MI355_API int mi355_rmsnorm_fwd_bf16_dev(uint16_t *y, const uint16_t *x, const f
     if (!mi355_ready("rmsnorm_fwd_bf16")) return -1;
     if (!y || !x || !w) return mi355_fail("rmsnorm_fwd_bf16: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_fwd_bf16: bad shape C=%d S=%d batch=%d", C, S, batch);
-    const BfCfg cfg = pick_bf(C, S % 8 == 0 && aligned16(x) && aligned16(y), S, batch);
+    const bool vec_ok = S % 8 == 0 && aligned16(x) && aligned16(y);
+    // tall shapes whose strips would leave compute units idle split the channel axis over clusters of workgroups,
+    // as the fp32 op does (norm_cluster.h); in place the single-workgroup tile is used
+    const ClusterPlan cp = y == x ? NO_CLUSTER : plan_cluster_bf(C, S, batch, vec_ok);
+    if (cp.csplit) {
+        if (!mi355_exchange(&g_bf_cluster_ws)) return -1;
+        if (cp.rpt == 2 && cp.exact) BF_CLUSTER_FWD(2, true);
+        else if (cp.rpt == 2) BF_CLUSTER_FWD(2, false);
+        else if (cp.exact) BF_CLUSTER_FWD(4, true);
+        else BF_CLUSTER_FWD(4, false);
+        LAUNCH_OK("rmsnorm_fwd_bf16");
+        return 0;
+    }
+    const BfCfg cfg = pick_bf(C, vec_ok, S, batch);
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
     BF_DISPATCH(rms_fwd_bf16_kernel, cfg, nblk, y, x, w, C, S, strips, nblk, eps, 1.0f / (float)C);
@@ -796,7 +747,22 @@ MI355_API int mi355_rmsnorm_bwd_bf16_dev(uint16_t *dx, float *dw, const uint16_t
     if (!dx || !dw || !dy || !x || !w) return mi355_fail("rmsnorm_bwd_bf16: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_bwd_bf16: bad shape C=%d S=%d batch=%d", C, S, batch);
     if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd_bf16: variant must be 0 or 1");
-    const BfCfg cfg = pick_bf(C, S % 8 == 0 && aligned16(x) && aligned16(dy) && aligned16(dx), S, batch);
+    const bool vec_ok = S % 8 == 0 && aligned16(x) && aligned16(dy) && aligned16(dx);
+    const ClusterPlan cp = (dx == dy || dx == x) ? NO_CLUSTER : plan_cluster_bf(C, S, batch, vec_ok);
+    if (cp.csplit) {
+        if (!mi355_exchange(&g_bf_cluster_ws)) return -1;
+        const int nrows = cp.nblk / cp.csplit;
+        float *part = mi355_dw_partials((size_t)nrows * C, dw, nullptr);
+        if (!part) return -1;
+        // (four rows per lane without the masks would need more than the 128 registers a lane has)
+        if (cp.rpt == 2 && cp.exact) BF_CLUSTER_BWD(2, true);
+        else if (cp.rpt == 2) BF_CLUSTER_BWD(2, false);
+        else BF_CLUSTER_BWD(4, false);
+        LAUNCH_OK("rmsnorm_bwd_bf16");
+        if (mi355_dw_submit(dw, part, nrows, C)) return -1;
+        return mi355_dw_op_end();
+    }
+    const BfCfg cfg = pick_bf(C, vec_ok, S, batch);
     const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
     const int nblk = strips * batch;
     float *part = mi355_dw_partials((size_t)nblk * C, dw, nullptr);

@@ -46,7 +46,7 @@ void *mi355_ws(size_t bytes);
 // RMSNorm, the single-launch INT8 scale): 8-byte slots {fp32 value, tag}, XCH_SLOT_STRIDE per workgroup number, and
 // one launch counter per workgroup number; norm_cluster.h describes the protocol.  Allocated and zeroed on first
 // use (not possible during a graph capture); false with the error recorded on failure.
-constexpr int XCH_SLOT_STRIDE = 128;
+constexpr int XCH_SLOT_STRIDE = 256;
 constexpr int XCH_MAX_BLOCKS = 2048;
 struct Mi355Exchange {
     unsigned long long *slots;     // [XCH_MAX_BLOCKS][XCH_SLOT_STRIDE]

@@ -476,14 +476,14 @@ bool cluster_ws_ready(void) { return mi355_exchange(&g_cluster_ws); }
 
 // The single-workgroup tiles are chosen by hand (knobs) or the shape does not cluster: csplit == 0.
 ClusterPlan plan_cluster(int C, int S, int batch, bool vec_ok, int max_rpt, int rounds = 1) {
-    if (g_ctx.rms_lpr || g_ctx.rms_threads) return ClusterPlan{0, 0, 0, 0, 0, 0, false};
-    return cluster_plan(C, S, batch, vec_ok, max_rpt, rounds);
+    if (g_ctx.rms_lpr || g_ctx.rms_threads) return NO_CLUSTER;
+    return cluster_plan(C, S, batch, vec_ok, StoreF32::VEC, 4, max_rpt, rounds);
 }
 
 template <int RPT, bool FUSE, bool EXACT>
 void launch_fwd_cluster_as(const ClusterPlan &cp, float *yn, float *y_res, const float *a, const float *b, float alpha,
                            const float *w, int C, int S, float eps) {
-    hipLaunchKernelGGL((rms_fwd_cluster_kernel<RPT, 1024, FUSE, EXACT>), dim3(cp.nblk), dim3(1024), 0, g_ctx.stream, yn,
+    hipLaunchKernelGGL((rms_fwd_cluster_kernel<StoreF32, RPT, 1024, FUSE, EXACT>), dim3(cp.nblk), dim3(1024), 0, g_ctx.stream, yn,
                        y_res, a, b, alpha, w, C, S, cp.strips, cp.nblk, cp.csplit, cp.rows_pm, eps, 1.0f / (float)C,
                        g_cluster_ws, cluster_spin_ticks());
 }
@@ -501,7 +501,7 @@ void launch_fwd_cluster(const ClusterPlan &cp, float *yn, float *y_res, const fl
 template <bool RES, bool EXACT>
 void launch_bwd_cluster_as(const ClusterPlan &cp, float *dx, float *part, const float *dy, const float *x, const float *w,
                            int C, int S, float eps, int variant, const float *res, float *dx2, float alpha2) {
-    hipLaunchKernelGGL((rms_bwd_cluster_kernel<4, 1024, RES, EXACT>), dim3(cp.nblk), dim3(1024), 0, g_ctx.stream, dx, part,
+    hipLaunchKernelGGL((rms_bwd_cluster_kernel<StoreF32, 4, 1024, RES, EXACT>), dim3(cp.nblk), dim3(1024), 0, g_ctx.stream, dx, part,
                        dy, x, w, C, S, cp.strips, cp.nblk, cp.csplit, cp.rows_pm, eps, 1.0f / (float)C, variant, res, dx2,
                        alpha2, g_cluster_ws, cluster_spin_ticks());
 }
@@ -541,7 +541,8 @@ MI355_API int mi355_rmsnorm_fwd_dev(float *y, const float *x, const float *w, in
     if (!y || !x || !w) return mi355_fail("rmsnorm_fwd: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_fwd: bad shape C=%d S=%d batch=%d", C, S, batch);
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(y);
-    const ClusterPlan cp = plan_cluster(C, S, batch, vec_ok, 8);
+    // in place the single-workgroup tile is used, for the reason given in mi355_rmsnorm_bwd_dev
+    const ClusterPlan cp = y == x ? NO_CLUSTER : plan_cluster(C, S, batch, vec_ok, 8);
     if (cp.csplit) {
         if (!cluster_ws_ready()) return -1;
         launch_fwd_cluster<false>(cp, y, nullptr, x, nullptr, 0.f, w, C, S, eps);
@@ -564,7 +565,7 @@ MI355_API int mi355_rmsnorm_bwd_dev(float *dx, float *dw, const float *dy, const
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(dy) && aligned16(dx);
     // in place on dy the single-workgroup tile is used: a cluster member that has to recompute another member's
     // sums (its bounded wait expired) would read rows that their owner has already overwritten
-    const ClusterPlan cp = dx == dy ? ClusterPlan{0, 0, 0, 0, 0, 0, false} : plan_cluster(C, S, batch, vec_ok, 4);
+    const ClusterPlan cp = dx == dy ? NO_CLUSTER : plan_cluster(C, S, batch, vec_ok, 4);
     if (cp.csplit) {
         if (!cluster_ws_ready()) return -1;
         const int nrows = cp.nblk / cp.csplit;
@@ -599,7 +600,7 @@ MI355_API int mi355_rmsnorm_bwd_residual_dev(float *dx, float *dx_scaled, float 
     if (dx == x) return mi355_fail("rmsnorm_bwd_residual: dx must not alias x (dx may alias res or dy)");
     const bool vec_ok = (S % 4 == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(res) &&
                         (!dx_scaled || aligned16(dx_scaled));
-    const ClusterPlan cp = dx == dy ? ClusterPlan{0, 0, 0, 0, 0, 0, false} : plan_cluster(C, S, batch, vec_ok, 4, 2);
+    const ClusterPlan cp = dx == dy ? NO_CLUSTER : plan_cluster(C, S, batch, vec_ok, 4, 2);
     if (cp.csplit) {
         if (!cluster_ws_ready()) return -1;
         const int nrows = cp.nblk / cp.csplit;
@@ -631,7 +632,7 @@ MI355_API int mi355_residual_rmsnorm_fwd_dev(float *y, float *yn, const float *a
     const bool vec_ok = (S % 4 == 0) && aligned16(y) && aligned16(yn) && aligned16(a) && aligned16(b);
     const float invC = 1.0f / (float)C;
     // in place (y over a or b) the single-workgroup tile is used, for the reason given in mi355_rmsnorm_bwd_dev
-    const ClusterPlan cp = (y == a || y == b) ? ClusterPlan{0, 0, 0, 0, 0, 0, false} : plan_cluster(C, S, batch, vec_ok, 8);
+    const ClusterPlan cp = (y == a || y == b) ? NO_CLUSTER : plan_cluster(C, S, batch, vec_ok, 8);
     if (cp.csplit) {
         if (!cluster_ws_ready()) return -1;
         launch_fwd_cluster<true>(cp, yn, y, a, b, alpha, w, C, S, eps);

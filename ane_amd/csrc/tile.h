@@ -40,6 +40,89 @@ __device__ __forceinline__ void stv(float *p, const float (&r)[VEC]) {
     }
 }
 
+// ---- bfloat16 storage: values travel as uint16_t bit patterns (the upper half of the fp32 pattern) and are
+// widened to fp32 on load, rounded to nearest even on store ----
+typedef uint16_t bf16_t;
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bf_to_f(unsigned bits16) { return __uint_as_float(bits16 << 16); }
+// round to nearest even; NaN stays NaN (quiet bit forced)
+__device__ __forceinline__ unsigned f_to_bf(float f) {
+    const unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+// VEC bf16 values -> VEC floats.  VEC = 8: one 128-bit access, element 2j in the low half of word j.
+template <int VEC, bool NT>
+__device__ __forceinline__ void ldb(float (&r)[VEC], const bf16_t *p) {
+    if constexpr (VEC == 8) {
+        const v4u *q = reinterpret_cast<const v4u *>(p);
+        const v4u w = NT ? __builtin_nontemporal_load(q) : *q;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            r[2 * j] = bf_to_f(w[j] & 0xffffu);
+            r[2 * j + 1] = bf_to_f(w[j] >> 16);
+        }
+    } else {
+        static_assert(VEC == 1, "bf16 rows are read 8 columns or 1 column at a time");
+        r[0] = bf_to_f(*p);
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void stb(bf16_t *p, const float (&r)[VEC]) {
+    if constexpr (VEC == 8) {
+        v4u w;
+#pragma unroll
+        for (int j = 0; j < 4; j++) w[j] = f_to_bf(r[2 * j]) | (f_to_bf(r[2 * j + 1]) << 16);
+        __builtin_nontemporal_store(w, reinterpret_cast<v4u *>(p));
+    } else {
+        *p = (bf16_t)f_to_bf(r[0]);
+    }
+}
+
+// Register tiles keep the bf16 words packed (half the registers of an fp32 tile) and widen them at each use.
+template <int VEC> struct RawT { typedef unsigned type; };
+template <> struct RawT<8> { typedef v4u type; };
+template <int VEC, bool NT>
+__device__ __forceinline__ typename RawT<VEC>::type ld_raw(const bf16_t *p) {
+    if constexpr (VEC == 8) {
+        const v4u *q = reinterpret_cast<const v4u *>(p);
+        return NT ? __builtin_nontemporal_load(q) : *q;
+    } else {
+        return (unsigned)*p;
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void unpack(float (&r)[VEC], const typename RawT<VEC>::type &w) {
+    if constexpr (VEC == 8) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            r[2 * j] = bf_to_f(w[j] & 0xffffu);
+            r[2 * j + 1] = bf_to_f(w[j] >> 16);
+        }
+    } else {
+        r[0] = bf_to_f(w);
+    }
+}
+// Tells the compiler nothing about the words' contents from here on, so that the widened copies made before a
+// reduction are dropped instead of being kept alive across it (they would double the register tile).
+template <int VEC>
+__device__ __forceinline__ void forget(typename RawT<VEC>::type &w) {
+    if constexpr (VEC == 8) {
+        unsigned a = w[0], b = w[1], c = w[2], d = w[3];
+        asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+        w[0] = a; w[1] = b; w[2] = c; w[3] = d;
+    } else {
+        asm volatile("" : "+v"(w));
+    }
+}
+template <int VEC>
+__device__ __forceinline__ typename RawT<VEC>::type raw_zero() {
+    if constexpr (VEC == 8) { v4u z = {0u, 0u, 0u, 0u}; return z; }
+    else return 0u;
+}
+
 // Sum acc[q][j] over all threads of the block that share the same lane column (tid % LPR).
 // Every thread ends with the full per-column totals.  lds: NW*NV*LPR*VEC floats.
 template <int VEC, int LPR, int THREADS, int NV>

@@ -82,6 +82,50 @@ def test_rmsnorm_bf16(br, B, C, S):
         assert H.rel_err(dwd.numpy(), rdw) <= 1e-5                      # fp32 in, fp32 sums, fp32 out
 
 
+@pytest.mark.parametrize("B,C,S", [(16, 1024, 256), (1, 768, 256), (2, 1000, 200), (3, 520, 136), (1, 2048, 8)])
+def test_rmsnorm_bf16_clustered_every_split_and_the_expired_wait(br, B, C, S):
+    """The bf16-storage norm with the channel axis split over 2, 4 or 8 cooperating workgroups (and the library's own
+    choice): against the oracle, equal to the bit whatever the split's bounded wait does, and run-to-run."""
+    print("[case] bf16 rmsnorm clustered B=%d C=%d S=%d" % (B, C, S), flush=True)
+    (xb, x), (dyb, dy) = bf(H.normal(230, (B, C, S))), bf(H.normal(231, (B, C, S)))
+    w = H.normal(232, C, 1.0, 0.02); dw0 = H.normal(233, C)
+    xd, dyd, wd = dev(br, xb), dev(br, dyb), dev(br, w)
+    ry = O.rmsnorm(x, w)
+    rdx, rdw = O.rmsnorm_bwd(dy, x, w, dw=dw0)
+
+    def run_all():
+        y, dx = br.DevArray(x.shape, np.uint16), br.DevArray(x.shape, np.uint16)
+        dwd = dev(br, dw0)
+        br.check(br.lib.mi355_rmsnorm_fwd_bf16_dev(y.ptr, xd.ptr, wd.ptr, C, S, B, 1e-5))
+        br.check(br.lib.mi355_rmsnorm_bwd_bf16_dev(dx.ptr, dwd.ptr, dyd.ptr, xd.ptr, wd.ptr, C, S, B, 1e-5, 0))
+        return [a.numpy() for a in (y, dx, dwd)]
+
+    try:
+        for split in (0, 2, 4, 8):
+            br.tune("rms_cluster", split); br.tune("rms_cluster_spin", 0)
+            got = run_all()
+            y, dx, dwv = got
+            assert H.rel_err(O.cvt_bf16_f32(y), ry) <= TOL16, split
+            assert H.rel_err(O.cvt_bf16_f32(dx), rdx) <= TOL16 and H.rel_err(dwv, rdw) <= 1e-5, split
+            again = run_all()
+            assert all(a.tobytes() == b.tobytes() for a, b in zip(got, again)), split
+            br.tune("rms_cluster_spin", -1)                              # the wait expires before it starts
+            alone = run_all()
+            assert all(a.tobytes() == b.tobytes() for a, b in zip(got, alone)), split
+    finally:
+        br.tune("rms_cluster", 0); br.tune("rms_cluster_spin", 0)
+    br.tune("rms_cluster", -1)                                           # never clustered: the single-workgroup tiles
+    try:
+        y, dx, dwv = run_all()
+        assert H.rel_err(O.cvt_bf16_f32(y), ry) <= TOL16 and H.rel_err(O.cvt_bf16_f32(dx), rdx) <= TOL16
+    finally:
+        br.tune("rms_cluster", 0)
+    # in place (dx over dy) the single-workgroup tile runs
+    dy2 = dev(br, dyb); dwd = dev(br, dw0)
+    br.check(br.lib.mi355_rmsnorm_bwd_bf16_dev(dy2.ptr, dwd.ptr, dy2.ptr, xd.ptr, wd.ptr, C, S, B, 1e-5, 0))
+    assert H.rel_err(back(dy2), rdx) <= TOL16
+
+
 def test_bf16_bad_arguments(br):
     a = br.DevArray(64, np.uint16); w = br.DevArray(8)
     assert br.lib.mi355_rmsnorm_fwd_bf16_dev(a.ptr, a.ptr, None, 8, 8, 1, 1e-5) == -1
