@@ -178,6 +178,7 @@ MI355_API int mi355_tune_set(const char *key, int value) {
         {"ce_rows", &g_ctx.ce_rows}, {"ce_rows2", &g_ctx.ce_rows2}, {"buf_phase", &g_ctx.buf_phase}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
         {"gemm_splitk", &g_ctx.gemm_splitk}, {"scatter_tree", &g_ctx.scatter_tree},
         {"rms_cluster", &g_ctx.rms_cluster}, {"rms_cluster_spin", &g_ctx.rms_cluster_spin},
+        {"ce_resident", &g_ctx.ce_resident},
     };
     for (auto &t : tab)
         if (strcmp(t.k, key) == 0) { *t.v = value; return 0; }

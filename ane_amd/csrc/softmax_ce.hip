@@ -16,6 +16,7 @@
 #include "common.h"
 
 #include <math.h>
+#include <type_traits>
 
 namespace {
 
@@ -350,6 +351,372 @@ __global__ __launch_bounds__(256) void nll_grad_kernel(float *dlogits, const flo
     st_cols<VEC>(dlogits + i, o);
 }
 
+// ---- the one-launch form: logits stay on the chip between the two passes ---------------------------------------
+// The register files and the LDS of the chip together hold more than the logits of the classifier
+// ([151936][256] fp32 = 156 MB; 256 compute units x (512 KB of registers + 160 KB of LDS) = 172 MB), so one launch
+// with ONE workgroup of 1024 threads per compute unit can read most rows once: a workgroup owns a block of rows of
+// one 64-column strip (256-byte row pieces), keeps the first CR row steps in registers and the next in LDS, and
+// reads only the remainder a second time.  The (max, sum exp) partials of the workgroups of a strip (its members)
+// are exchanged through tagged 8-byte slots as in the clustered RMSNorm (norm_cluster.h): one relaxed agent-scope
+// atomic {fp32 value, launch tag} per slot, a launch counter per workgroup number, nothing to clear, a bounded
+// wait.  A member whose wait for a partner expires recomputes that partner's partial from memory with the same
+// operations in the same order (same bits), so every member of a strip normalises with identical column sums.
+constexpr int CR_THREADS = 1024;
+constexpr int CR_W = 64;                     // columns per strip
+constexpr int CR_RPS = CR_THREADS / 16;      // rows per step: 16 lanes x 16 B per row piece
+constexpr int CR_NW = CR_THREADS / 64;
+constexpr int CR_MAX_SPLIT = 64;             // members per strip
+constexpr int CR_MAX_STRIPS = 16;
+constexpr int CR_LOSS_SLOT = 2 * CR_W;       // after the 64 maxima and 64 sums
+constexpr int CR_STRIDE = 136;               // slots per workgroup number
+constexpr int CR_MAX_WG = 512;
+constexpr int CR_SUB = 4;                    // rows per lane and online step beyond the register rows
+constexpr int CR_K_REG = 20, CR_K_LDS = 7;   // row steps kept in registers (80 of a lane's 128) and in LDS (112 KB)
+constexpr int CR_MAX_STEPS = 64;             // beyond that most rows would be read twice anyway
+constexpr size_t CR_XCH_BYTES = (size_t)CR_MAX_WG * CR_STRIDE * 8 + (size_t)CR_MAX_WG * 4 + 256;
+
+struct CeXch {
+    unsigned long long *slots;     // [CR_MAX_WG][CR_STRIDE]
+    unsigned *cnt;                 // [CR_MAX_WG] launches completed by each workgroup number
+    int *fallbacks;                // workgroups whose bounded wait expired, ever (diagnostic)
+};
+struct CrGeo {
+    const float *logits;
+    int V, S, strips, csplit, Rm, K;   // Rm rows per member, K = ceil(Rm / CR_RPS) row steps
+};
+
+// (m, l) <- (m, l) merged with N more values: the online-softmax step
+template <int N>
+__device__ __forceinline__ void online_update(float &m, float &l, const float (&x)[N]) {
+    float tm = x[0];
+#pragma unroll
+    for (int k = 1; k < N; k++) tm = fmaxf(tm, x[k]);
+    const float nm = fmaxf(m, tm);
+    if (nm > -INFINITY) {
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < N; k++) s += exp_neg_fast(x[k] - nm);     // exp(-inf) = 0 for masked rows
+        l = l * exp_neg(m - nm) + s;
+        m = nm;
+    }
+}
+__device__ __forceinline__ void merge_pair(float &m, float &l, float m1, float l1) {
+    const float nm = fmaxf(m, m1);
+    if (nm > -INFINITY) {
+        l = l * exp_neg(m - nm) + l1 * exp_neg(m1 - nm);
+        m = nm;
+    }
+}
+
+// The (max, sum exp) partial of member p of a strip over its rows, for the 64 columns of the strip: valid in
+// threads 0..63 (thread t = column t) on return.  KEEP: this workgroup's own rows; the first K_REG steps stay in
+// xr, the next K_LDS in lrow.  Otherwise nothing is kept and the first K_REG steps are read twice (their maximum,
+// then their sum in the same order), which gives the same bits with four rows in flight instead of K_REG.
+template <int K_REG, int K_LDS, bool KEEP>
+__device__ __forceinline__ void cr_member_partial(const CrGeo &g, int strip, int p, v4f (&xr)[K_REG], v4f (*lrow)[CR_THREADS],
+                                                  float (*wm)[CR_W], float (*wl)[CR_W], float &Mout, float &Lout) {
+    static_assert(K_REG % CR_SUB == 0, "the register rows are re-read four at a time");
+    const int lc = threadIdx.x & 15, row0 = threadIdx.x >> 4, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int v_lo = p * g.Rm;
+    // this lane holds the member's rows row0 + 64k; they exist while 64k < lim
+    const int lim = min(g.V, v_lo + g.Rm) - v_lo - row0;
+    // a row piece = (uniform address of row v_lo + 64k of the strip) + (this lane's fixed 32-bit offset)
+    const float *base = g.logits + ((size_t)v_lo * g.S + (size_t)strip * CR_W);
+    const unsigned loff = (unsigned)row0 * (unsigned)g.S + (unsigned)lc * 4u;
+    const size_t step = (size_t)CR_RPS * g.S;
+    const v4f ninf = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    float m[4], l[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) { m[j] = -INFINITY; l[j] = 0.f; }
+    if constexpr (KEEP) {
+#pragma unroll
+        for (int k = 0; k < K_REG; k++) {
+            xr[k] = CR_RPS * k < lim ? ld4(base + k * step + loff) : ninf;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float t[K_REG];
+#pragma unroll
+            for (int k = 0; k < K_REG; k++) t[k] = xr[k][j];
+            online_update<K_REG>(m[j], l[j], t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        for (int k0 = K_REG; k0 < g.K; k0 += CR_SUB) {
+            v4f t[CR_SUB];
+#pragma unroll
+            for (int u = 0; u < CR_SUB; u++) {
+                t[u] = CR_RPS * (k0 + u) < lim ? ld4(base + (k0 + u) * step + loff) : ninf;
+                if (k0 + u < K_REG + K_LDS) lrow[k0 + u - K_REG][threadIdx.x] = t[u];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float x4[CR_SUB];
+#pragma unroll
+                for (int u = 0; u < CR_SUB; u++) x4[u] = t[u][j];
+                online_update<CR_SUB>(m[j], l[j], x4);
+            }
+        }
+    } else {
+        // one column and one row at a time: the same operations on the same values in the same order with a
+        // handful of registers, because the caller's own rows stay live in theirs
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            auto at = [&](int k) {
+                return CR_RPS * k < lim ? base[k * step + loff + j] : -INFINITY;
+            };
+            float mj = -INFINITY, lj = 0.f, tm = -INFINITY, s = 0.f;
+#pragma unroll 1
+            for (int k = 0; k < K_REG; k++) tm = fmaxf(tm, at(k));
+            const float nm = fmaxf(mj, tm);
+            if (nm > -INFINITY) {
+#pragma unroll 1
+                for (int k = 0; k < K_REG; k++) s += exp_neg_fast(at(k) - nm);
+                lj = lj * exp_neg(mj - nm) + s;
+                mj = nm;
+            }
+#pragma unroll 1
+            for (int k0 = K_REG; k0 < g.K; k0 += CR_SUB) {
+                float x4[CR_SUB];
+#pragma unroll
+                for (int u = 0; u < CR_SUB; u++) x4[u] = at(k0 + u);
+                online_update<CR_SUB>(mj, lj, x4);
+            }
+            m[j] = mj;
+            l[j] = lj;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // the four row groups of a wave, then the sixteen waves in order
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        merge_pair(m[j], l[j], lane_xor<16>(m[j]), lane_xor<16>(l[j]));
+        merge_pair(m[j], l[j], lane_xor<32>(m[j]), lane_xor<32>(l[j]));
+    }
+    if (lane < 16) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) { wm[wave][lc * 4 + j] = m[j]; wl[wave][lc * 4 + j] = l[j]; }
+    }
+    __syncthreads();
+    if (threadIdx.x < CR_W) {
+        float M = wm[0][threadIdx.x], L = wl[0][threadIdx.x];
+#pragma unroll
+        for (int w = 1; w < CR_NW; w++) merge_pair(M, L, wm[w][threadIdx.x], wl[w][threadIdx.x]);
+        Mout = M;
+        Lout = L;
+    }
+    __syncthreads();
+}
+
+// The members' partials in tot[p][0 = max, 1 = sum][column] -> the strip's column maxima and sums, merged in a
+// fixed order (sixteen groups of members, then the groups); valid in threads 0..63 on return.
+__device__ __forceinline__ void cr_merge_members(int csplit, const float (*tot)[2][CR_W], float (*wm)[CR_W], float (*wl)[CR_W],
+                                                 float &Mout, float &Lout) {
+    const int c = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int mpg = (csplit + CR_NW - 1) / CR_NW;
+    float M = -INFINITY, L = 0.f;
+    for (int q = 0; q < mpg; q++) {
+        const int p = grp * mpg + q;
+        if (p < csplit) merge_pair(M, L, tot[p][0][c], tot[p][1][c]);
+    }
+    wm[grp][c] = M;
+    wl[grp][c] = L;
+    __syncthreads();
+    if (threadIdx.x < CR_W) {
+        M = wm[0][threadIdx.x]; L = wl[0][threadIdx.x];
+#pragma unroll
+        for (int w = 1; w < CR_NW; w++) merge_pair(M, L, wm[w][threadIdx.x], wl[w][threadIdx.x]);
+        Mout = M;
+        Lout = L;
+    }
+    __syncthreads();
+}
+
+// Sum over the strip's columns of -log(p[target] + 1e-10), by wave 0 (every lane of it ends with the sum).
+__device__ __forceinline__ float cr_strip_loss(const CrGeo &g, int strip, const int32_t *targets, float M, float inv) {
+    const int t = strip * CR_W + threadIdx.x;
+    const int tg = targets[t];
+    float loss = 0.f;
+    if (tg >= 0 && tg < g.V) {
+        const float p = exp_neg(g.logits[(size_t)tg * g.S + t] - M) * inv;
+        loss = -logf(p + 1e-10f);
+    }
+    return wave_sum_far_first(loss);
+}
+
+// One bounded wait for a tagged slot.  false: the tag did not arrive within spin_ticks.
+__device__ __forceinline__ bool cr_wait_slot(const unsigned long long *sp, unsigned want, int spin_ticks, float &value) {
+    const long long t0 = wall_clock64();
+    for (;;) {
+        const unsigned long long pk = __hip_atomic_load(sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((unsigned)(pk >> 32) == want) { value = __uint_as_float((unsigned)pk); return true; }
+        if (wall_clock64() - t0 >= (long long)spin_ticks) return false;
+        __builtin_amdgcn_s_sleep(2);
+    }
+}
+
+// grid: strips * csplit workgroups, all resident at once (one per compute unit).  Workgroup b: strip b % strips,
+// member b / strips, so that the workgroups that read the pieces of one row are neighbours in time.
+template <int K_REG, int K_LDS>
+__global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restrict__ dlogits, const float *__restrict__ logits,
+                                                                 const int32_t *__restrict__ targets, int V, int S,
+                                                                 int strips, int csplit, int Rm, int K, float invS,
+                                                                 float grad_scale, float *__restrict__ loss_out, CeXch ws,
+                                                                 int spin_ticks) {
+    __shared__ v4f lrow[K_LDS][CR_THREADS];
+    __shared__ float wm[CR_NW][CR_W], wl[CR_NW][CR_W];
+    __shared__ float tot[CR_MAX_SPLIT][2][CR_W];
+    __shared__ float fM[CR_W], fInv[CR_W];
+    __shared__ float strip_loss[CR_MAX_STRIPS];
+    __shared__ unsigned want[CR_MAX_SPLIT], want_leader[CR_MAX_STRIPS];
+    __shared__ int failed[CR_MAX_SPLIT];
+    const int tid = threadIdx.x;
+    const int b = blockIdx.x;
+    const int strip = b % strips, me = b / strips;
+    const CrGeo g = {logits, V, S, strips, csplit, Rm, K};
+    if (tid < csplit) { want[tid] = ws.cnt[tid * strips + strip] + 1u; failed[tid] = 0; }
+    if (tid < strips) want_leader[tid] = ws.cnt[tid] + 1u;          // member 0 of strip s is workgroup s
+    const unsigned my_tag = ws.cnt[b] + 1u;
+    __syncthreads();
+
+    // ---- pass 1: this member's rows, kept; its partial published
+    v4f xr[K_REG];
+    float Mp = -INFINITY, Lp = 0.f;
+    cr_member_partial<K_REG, K_LDS, true>(g, strip, me, xr, lrow, wm, wl, Mp, Lp);
+    if (tid < CR_W) {
+        unsigned long long *mine = ws.slots + (size_t)b * CR_STRIDE;
+        __hip_atomic_store(mine + tid, ((unsigned long long)my_tag << 32) | __float_as_uint(Mp), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + CR_W + tid, ((unsigned long long)my_tag << 32) | __float_as_uint(Lp), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // ---- every member's partial: 128 slots each
+    for (int i = tid; i < csplit * 2 * CR_W; i += CR_THREADS) {
+        const int p = i >> 7, r = i & 127;
+        float val = 0.f;
+        if (!cr_wait_slot(ws.slots + (size_t)(p * strips + strip) * CR_STRIDE + r, want[p], spin_ticks, val)) failed[p] = 1;
+        tot[p][r >> 6][r & 63] = val;
+    }
+    __syncthreads();
+    bool counted = false;
+    for (int p = 0; p < csplit; p++) {
+        if (failed[p]) {                                             // the same for every thread: read after the barrier
+            if (tid == 0 && !counted) { atomicAdd(ws.fallbacks, 1); counted = true; }
+            float M2 = -INFINITY, L2 = 0.f;
+            cr_member_partial<K_REG, K_LDS, false>(g, strip, p, xr, lrow, wm, wl, M2, L2);
+            if (tid < CR_W) { tot[p][0][tid] = M2; tot[p][1][tid] = L2; }
+        }
+    }
+    __syncthreads();
+    float Mc = 0.f, Lc = 1.f;
+    cr_merge_members(csplit, tot, wm, wl, Mc, Lc);
+    if (tid < CR_W) {
+        const float inv = 1.0f / Lc;
+        fM[tid] = Mc;
+        fInv[tid] = inv;
+        if (me == 0) {                                               // the strip's leader also forms its loss term
+            const float ls = cr_strip_loss(g, strip, targets, Mc, inv);
+            if (tid == 0) {
+                strip_loss[strip] = ls;
+                __hip_atomic_store(ws.slots + (size_t)b * CR_STRIDE + CR_LOSS_SLOT,
+                                   ((unsigned long long)my_tag << 32) | __float_as_uint(ls), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- pass 2: dlogits = (exp(l - M) / L - onehot) / S * grad_scale; the rows read last come first
+    {
+        const int lc = tid & 15;
+        int row0 = tid >> 4;
+        asm volatile("" : "+v"(row0));     // the row masks are formed again here instead of being kept from pass 1
+        const int v_lo = me * Rm;
+        const int lim = min(V, v_lo + Rm) - v_lo - row0;           // this lane's rows row0 + 64k exist while 64k < lim
+        const float *src = logits + ((size_t)v_lo * S + (size_t)strip * CR_W);
+        float *dst = dlogits + ((size_t)v_lo * S + (size_t)strip * CR_W);
+        const unsigned loff = (unsigned)row0 * (unsigned)S + (unsigned)lc * 4u;
+        const size_t step = (size_t)CR_RPS * S;
+        float M[4], inv[4], sc[4];
+        int tk[4];                         // the target's row is this lane's row 64k when tk == 64k
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            M[j] = fM[lc * 4 + j];
+            inv[j] = fInv[lc * 4 + j];
+            const int tg = targets[strip * CR_W + lc * 4 + j];
+            const bool ok = tg >= 0 && tg < V;
+            tk[j] = ok ? tg - v_lo - row0 : -1;
+            sc[j] = ok ? invS : 1.0f;      // an out-of-range target leaves the column unscaled (stories_cpu_ops.h:98)
+        }
+        auto emit = [&](int k, const v4f &x) {
+            v4f o;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float pj = exp_neg(x[j] - M[j]) * inv[j];
+                if (tk[j] == CR_RPS * k) pj -= 1.0f;
+                pj = pj * sc[j];
+                if (grad_scale != 1.0f) pj = pj * grad_scale;
+                o[j] = pj;
+            }
+            st4_nt(dst + k * step + loff, o);
+        };
+        for (int k0 = K_REG + K_LDS; k0 < K; k0 += CR_SUB) {
+            v4f t[CR_SUB];
+#pragma unroll
+            for (int u = 0; u < CR_SUB; u++)
+                if (CR_RPS * (k0 + u) < lim) t[u] = ld4_nt(src + (k0 + u) * step + loff);
+#pragma unroll
+            for (int u = 0; u < CR_SUB; u++)
+                if (CR_RPS * (k0 + u) < lim) emit(k0 + u, t[u]);
+        }
+#pragma unroll
+        for (int k = 0; k < K_LDS; k++) {
+            if (CR_RPS * (K_REG + k) < lim) emit(K_REG + k, lrow[k][tid]);
+            __builtin_amdgcn_sched_barrier(0);       // one row at a time: the scheduler would otherwise hold them all
+        }
+#pragma unroll
+        for (int k = 0; k < K_REG; k++) {
+            if (CR_RPS * k < lim) emit(k, xr[k]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // ---- the loss: workgroup 0 adds the strips' terms in order; by now the other leaders have long published
+    if (b == 0) {
+        __syncthreads();
+        if (tid < strips) failed[tid] = 0;
+        __syncthreads();
+        if (tid > 0 && tid < strips) {
+            float val = 0.f;
+            if (!cr_wait_slot(ws.slots + (size_t)tid * CR_STRIDE + CR_LOSS_SLOT, want_leader[tid], spin_ticks, val)) failed[tid] = 1;
+            strip_loss[tid] = val;
+        }
+        __syncthreads();
+        for (int s2 = 1; s2 < strips; s2++) {
+            if (failed[s2]) {                                        // that strip's loss term from memory, the same way
+                for (int p = 0; p < csplit; p++) {
+                    float M2 = -INFINITY, L2 = 0.f;
+                    cr_member_partial<K_REG, K_LDS, false>(g, s2, p, xr, lrow, wm, wl, M2, L2);
+                    if (tid < CR_W) { tot[p][0][tid] = M2; tot[p][1][tid] = L2; }
+                }
+                __syncthreads();
+                float M3 = 0.f, L3 = 1.f;
+                cr_merge_members(csplit, tot, wm, wl, M3, L3);
+                if (tid < CR_W) {
+                    const float ls = cr_strip_loss(g, s2, targets, M3, 1.0f / L3);
+                    if (tid == 0) strip_loss[s2] = ls;
+                }
+                __syncthreads();
+            }
+        }
+        if (tid == 0) {
+            float total = 0.f;
+            for (int s2 = 0; s2 < strips; s2++) total += strip_loss[s2];
+            *loss_out = total / (float)S;
+        }
+    }
+    if (tid == 0) ws.cnt[b] = my_tag;
+}
+
 // resident workgroups of the second pass per compute unit (asked of the runtime once per storage type)
 template <typename T>
 int grad_blocks_per_cu() {
@@ -367,10 +734,14 @@ int grad_blocks_per_cu() {
 // file-scope device array, so that the call needs no allocation.  One copy per GPU, held until the process ends.
 // In host code the array's name is only a handle for the symbol lookup below; kernels and copies use the address
 // that the lookup returns for the current device.
+// Behind them, in the same array, lies the exchange area of the one-launch kernel (slots and launch counters, which
+// must start at zero: the array is zero-initialised when the code object is loaded, and nothing ever clears it).
 constexpr size_t CE_SCRATCH_BYTES = (size_t)2 << 20;
+constexpr size_t CE_XCH_AREA = (size_t)1 << 20;
+static_assert(CR_XCH_BYTES <= CE_XCH_AREA, "the exchange area must fit behind the partials");
 constexpr int CE_MAX_DEVICES = 16;
 }   // namespace
-static __device__ __align__(256) unsigned char scratch[CE_SCRATCH_BYTES];
+static __device__ __align__(256) unsigned char scratch[CE_SCRATCH_BYTES + CE_XCH_AREA];
 namespace {
 unsigned char *g_scratch_ptr[CE_MAX_DEVICES] = {};
 
@@ -384,6 +755,31 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
     // compute units evenly (at least 1.75 per unit, and the last round of them as full as possible); ties go to
     // the larger block, which leaves fewer partials to merge.  At V = 151936 on 256 units: 320 rows, 475
     // workgroups (87 us for the op; 256 rows and 594 workgroups: 91 us; 384 rows and 396: 97 us).
+    if constexpr (std::is_same<T, float>::value) {
+        // The one-launch form: fp32, whole 64-column strips, out of place (a member that recomputes a partner's
+        // partial reads the partner's logits), and a vocabulary for which it pays (ce_resident: 0 = V >= 4096,
+        // 1 = any V, -1 = never).  One workgroup per compute unit at most, so that all of them are resident at once.
+        const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
+        const int strips_r = S / CR_W;
+        unsigned char *base = (g_ctx.device >= 0 && g_ctx.device < CE_MAX_DEVICES) ? g_scratch_ptr[g_ctx.device] : nullptr;
+        if (g_ctx.ce_resident >= 0 && base && S % CR_W == 0 && strips_r <= CR_MAX_STRIPS && (const void *)dlogits != (const void *)logits &&
+            aligned16(logits) && aligned16(dlogits) && (V >= 4096 || g_ctx.ce_resident > 0)) {
+            const int csplit = cu / strips_r < CR_MAX_SPLIT ? cu / strips_r : CR_MAX_SPLIT;
+            const int Rm = csplit > 0 ? (int)ceil_div((size_t)V, (size_t)csplit) : 0;
+            const int K = (int)ceil_div((size_t)Rm, (size_t)CR_RPS);
+            if (csplit >= 2 && csplit * strips_r <= CR_MAX_WG && csplit * strips_r <= cu && K <= CR_MAX_STEPS) {
+                CeXch xch;
+                xch.slots = (unsigned long long *)(base + CE_SCRATCH_BYTES);
+                xch.cnt = (unsigned *)(base + CE_SCRATCH_BYTES + (size_t)CR_MAX_WG * CR_STRIDE * 8);
+                xch.fallbacks = (int *)(base + CE_SCRATCH_BYTES + (size_t)CR_MAX_WG * CR_STRIDE * 8 + (size_t)CR_MAX_WG * 4);
+                hipLaunchKernelGGL((ce_resident_kernel<CR_K_REG, CR_K_LDS>), dim3((unsigned)(csplit * strips_r)), dim3(CR_THREADS), 0,
+                                   g_ctx.stream, (float *)dlogits, (const float *)logits, targets, V, S, strips_r, csplit, Rm, K,
+                                   1.0f / (float)S, grad_scale, loss_dev, xch, mi355_exchange_spin_ticks());
+                LAUNCH_OK("softmax_ce (one launch)");
+                return 0;
+            }
+        }
+    }
     int rpb = g_ctx.ce_rows;
     if (rpb <= 0) {
         const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;

@@ -703,6 +703,46 @@ def test_softmax_ce_deterministic(br):
     assert res[0] == res[1]
 
 
+@pytest.mark.parametrize("V,S", [(4099, 64), (32000, 256), (151936, 256), (700, 128), (40, 64), (9000, 1024), (5000, 192),
+                                 (70000, 64)])
+def test_softmax_ce_one_launch_and_its_expired_wait(br, V, S):
+    """The form that keeps the logits on the chip between the passes (one workgroup per compute unit, partials
+    exchanged inside the launch), forced for every shape it accepts: against the oracle; run to run and with the
+    bounded wait set to expire at once (partners' partials recomputed from memory) the same bits; and close to the
+    three-launch form, which sums in another order."""
+    say("softmax_ce one launch V=%d S=%d" % (V, S))
+    logits = H.normal(77, (V, S), 0, 2.0)
+    tgt = np.random.default_rng(78).integers(0, V, S).astype(np.int32)
+    tgt[1] = V; tgt[S - 2] = -1                                         # out-of-range targets are skipped
+    ld, td = dev(br, logits), dev(br, tgt)
+
+    def run(scale):
+        dd = br.DevArray(logits.shape); lossd = br.DevArray(1)
+        br.check(br.lib.mi355_softmax_ce_dev(dd.ptr, lossd.ptr, ld.ptr, td.ptr, V, S, scale))
+        return lossd.numpy().copy(), dd.numpy()
+
+    try:
+        br.tune("ce_resident", 1); br.tune("rms_cluster_spin", 0)
+        for scale in (1.0, 256.0):
+            loss, dl = run(scale)
+            rl, rd = O.cross_entropy(logits, tgt, scale)
+            assert abs(float(loss[0]) - rl) <= TOL * abs(rl) + 1e-12
+            assert H.err_std(dl, rd) <= TOL
+        loss, dl = run(1.0)
+        loss2, dl2 = run(1.0)
+        assert loss.tobytes() == loss2.tobytes() and dl.tobytes() == dl2.tobytes()
+        br.tune("rms_cluster_spin", -1)                                  # the wait expires before it starts
+        loss3, dl3 = run(1.0)
+        assert loss.tobytes() == loss3.tobytes() and dl.tobytes() == dl3.tobytes()
+        br.tune("rms_cluster_spin", 0)
+        br.tune("ce_resident", -1)                                       # the three-launch form
+        loss4, dl4 = run(1.0)
+        assert abs(float(loss4[0]) - float(loss[0])) <= 2e-6 * abs(float(loss[0]))
+        assert H.err_std(dl4, dl) <= 2e-6
+    finally:
+        br.tune("ce_resident", 0); br.tune("rms_cluster_spin", 0)
+
+
 # ---------------------------------------------------------------------------------------------
 # INT8: bit-exact
 # ---------------------------------------------------------------------------------------------
