@@ -355,8 +355,9 @@ __global__ __launch_bounds__(256) void nll_grad_kernel(float *dlogits, const flo
 // The register files and the LDS of the chip together hold more than the logits of the classifier
 // ([151936][256] fp32 = 156 MB; 256 compute units x (512 KB of registers + 160 KB of LDS) = 172 MB), so one launch
 // with ONE workgroup of 1024 threads per compute unit can read most rows once: a workgroup owns a block of rows of
-// one 64-column strip (256-byte row pieces), keeps the first CR row steps in registers and the next in LDS, and
-// reads only the remainder a second time.  The (max, sum exp) partials of the workgroups of a strip (its members)
+// one 64-column strip (256-byte row pieces), keeps its last 16 row steps in registers and the 9 before them in LDS
+// (25 of the 38 steps of the Qwen3 vocabulary; all of them for 32000 rows), and reads only the remainder a second
+// time.  Measured at [151936][256]: 69 us against 84 us for the three launches.  The (max, sum exp) partials of the workgroups of a strip (its members)
 // are exchanged through tagged 8-byte slots as in the clustered RMSNorm (norm_cluster.h): one relaxed agent-scope
 // atomic {fp32 value, launch tag} per slot, a launch counter per workgroup number, nothing to clear, a bounded
 // wait.  A member whose wait for a partner expires recomputes that partner's partial from memory with the same
@@ -371,7 +372,7 @@ constexpr int CR_LOSS_SLOT = 2 * CR_W;       // after the 64 maxima and 64 sums
 constexpr int CR_STRIDE = 136;               // slots per workgroup number
 constexpr int CR_MAX_WG = 512;
 constexpr int CR_SUB = 4;                    // rows per lane and online step beyond the register rows
-constexpr int CR_K_REG = 20, CR_K_LDS = 7;   // row steps kept in registers (80 of a lane's 128) and in LDS (112 KB)
+constexpr int CR_K_REG = 16, CR_K_LDS = 9;   // row steps kept in registers (64 of a lane's 128) and in LDS (144 KB)
 constexpr int CR_MAX_STEPS = 64;             // beyond that most rows would be read twice anyway
 constexpr size_t CR_XCH_BYTES = (size_t)CR_MAX_WG * CR_STRIDE * 8 + (size_t)CR_MAX_WG * 4 + 256;
 
@@ -408,46 +409,57 @@ __device__ __forceinline__ void merge_pair(float &m, float &l, float m1, float l
     }
 }
 
+// Sixteen (max, sum) pairs of one column -> their merge: the maximum, then the sums rescaled to it (sixteen
+// independent exponentials) and added in order.
+__device__ __forceinline__ void cr_merge16(const float (*wm)[CR_W], const float (*wl)[CR_W], int c, float &M, float &L) {
+    float mm[CR_NW];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < CR_NW; w++) { mm[w] = wm[w][c]; mx = fmaxf(mx, mm[w]); }
+    float acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < CR_NW; w++) acc += wl[w][c] * exp_neg(mm[w] - mx);     // an empty part has sum 0
+    M = mx;
+    L = acc;
+}
+
 // The (max, sum exp) partial of member p of a strip over its rows, for the 64 columns of the strip: valid in
-// threads 0..63 (thread t = column t) on return.  KEEP: this workgroup's own rows; the first K_REG steps stay in
-// xr, the next K_LDS in lrow.  Otherwise nothing is kept and the first K_REG steps are read twice (their maximum,
-// then their sum in the same order), which gives the same bits with four rows in flight instead of K_REG.
-template <int K_REG, int K_LDS, bool KEEP>
+// threads 0..63 (thread t = column t) on return.  Of a member's K row steps the last K_REG are the register rows,
+// the K_LDS before them the LDS rows, and the first kL = K - K_REG - K_LDS the rows that are read twice.  A lane
+// folds its rows into its running (max, sum) four at a time, in row order: the rows before the register rows, then
+// the register rows.  KEEP: this workgroup's own rows; the loads run ahead of the arithmetic.
+// Otherwise nothing is kept: one column and one
+// group of four rows at a time, the same operations on the same values in the same order (same bits) in a handful
+// of registers, because the caller's own rows stay live in theirs.
+template <int K_REG, int K_LDS, bool KEEP, bool NT = false>
 __device__ __forceinline__ void cr_member_partial(const CrGeo &g, int strip, int p, v4f (&xr)[K_REG], v4f (*lrow)[CR_THREADS],
                                                   float (*wm)[CR_W], float (*wl)[CR_W], float &Mout, float &Lout) {
-    static_assert(K_REG % CR_SUB == 0, "the register rows are re-read four at a time");
+    static_assert(K_REG % CR_SUB == 0, "the register rows fold four at a time");
     const int lc = threadIdx.x & 15, row0 = threadIdx.x >> 4, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int v_lo = p * g.Rm;
-    // this lane holds the member's rows row0 + 64k; they exist while 64k < lim
+    constexpr int rs = CR_RPS;                                    // rows between a lane's consecutive rows
+    // this lane holds the member's rows row0 + rs*k; they exist while rs*k < lim
     const int lim = min(g.V, v_lo + g.Rm) - v_lo - row0;
-    // a row piece = (uniform address of row v_lo + 64k of the strip) + (this lane's fixed 32-bit offset)
+    const int kR = max(0, g.K - K_REG), kL = max(0, kR - K_LDS);
+    // a row piece = (uniform address of row v_lo + rs*k of the strip) + (this lane's fixed 32-bit offset)
     const float *base = g.logits + ((size_t)v_lo * g.S + (size_t)strip * CR_W);
     const unsigned loff = (unsigned)row0 * (unsigned)g.S + (unsigned)lc * 4u;
-    const size_t step = (size_t)CR_RPS * g.S;
+    const size_t step = (size_t)rs * g.S;
     const v4f ninf = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
     float m[4], l[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) { m[j] = -INFINITY; l[j] = 0.f; }
     if constexpr (KEEP) {
-#pragma unroll
-        for (int k = 0; k < K_REG; k++) {
-            xr[k] = CR_RPS * k < lim ? ld4(base + k * step + loff) : ninf;
-        }
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float t[K_REG];
-#pragma unroll
-            for (int k = 0; k < K_REG; k++) t[k] = xr[k][j];
-            online_update<K_REG>(m[j], l[j], t);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        for (int k0 = K_REG; k0 < g.K; k0 += CR_SUB) {
-            v4f t[CR_SUB];
+        // rows that stay on the chip may be read past the cache (they are not read again); the others stay cached
+        auto loadg = [&](v4f (&t)[CR_SUB], int k0) {
 #pragma unroll
             for (int u = 0; u < CR_SUB; u++) {
-                t[u] = CR_RPS * (k0 + u) < lim ? ld4(base + (k0 + u) * step + loff) : ninf;
-                if (k0 + u < K_REG + K_LDS) lrow[k0 + u - K_REG][threadIdx.x] = t[u];
+                const int k = k0 + u;
+                if (k < kR && rs * k < lim) t[u] = (NT && k >= kL) ? ld4_nt(base + k * step + loff) : ld4(base + k * step + loff);
+                else t[u] = ninf;
             }
+        };
+        auto foldg = [&](const v4f (&t)[CR_SUB]) {
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 float x4[CR_SUB];
@@ -455,32 +467,59 @@ __device__ __forceinline__ void cr_member_partial(const CrGeo &g, int strip, int
                 for (int u = 0; u < CR_SUB; u++) x4[u] = t[u][j];
                 online_update<CR_SUB>(m[j], l[j], x4);
             }
+        };
+        auto keepg = [&](const v4f (&t)[CR_SUB], int k0) {
+#pragma unroll
+            for (int u = 0; u < CR_SUB; u++)
+                if (k0 + u >= kL && k0 + u < kR) lrow[k0 + u - kL][threadIdx.x] = t[u];
+        };
+        // the register rows are asked for first and folded last: they are in flight while the other rows stream
+        // through two groups of four
+#pragma unroll
+        for (int i = 0; i < K_REG; i++) {
+            const int k = kR + i;
+            xr[i] = rs * k < lim ? (NT ? ld4_nt(base + k * step + loff) : ld4(base + k * step + loff)) : ninf;
+        }
+        {
+            v4f ta[CR_SUB], tb[CR_SUB];
+            loadg(ta, 0);
+            loadg(tb, CR_SUB);
+            for (int k0 = 0; k0 < kR; k0 += 2 * CR_SUB) {
+                keepg(ta, k0);
+                foldg(ta);
+                loadg(ta, k0 + 2 * CR_SUB);
+                if (k0 + CR_SUB < kR) {
+                    keepg(tb, k0 + CR_SUB);
+                    foldg(tb);
+                }
+                loadg(tb, k0 + 3 * CR_SUB);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < K_REG / CR_SUB; c++) {
+            v4f t[CR_SUB];
+#pragma unroll
+            for (int u = 0; u < CR_SUB; u++) t[u] = xr[c * CR_SUB + u];
+            foldg(t);
         }
     } else {
-        // one column and one row at a time: the same operations on the same values in the same order with a
-        // handful of registers, because the caller's own rows stay live in theirs
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            auto at = [&](int k) {
-                return CR_RPS * k < lim ? base[k * step + loff + j] : -INFINITY;
-            };
-            float mj = -INFINITY, lj = 0.f, tm = -INFINITY, s = 0.f;
+            float mj = -INFINITY, lj = 0.f;
+            auto part = [&](int kbeg, int kend) {
 #pragma unroll 1
-            for (int k = 0; k < K_REG; k++) tm = fmaxf(tm, at(k));
-            const float nm = fmaxf(mj, tm);
-            if (nm > -INFINITY) {
-#pragma unroll 1
-                for (int k = 0; k < K_REG; k++) s += exp_neg_fast(at(k) - nm);
-                lj = lj * exp_neg(mj - nm) + s;
-                mj = nm;
-            }
-#pragma unroll 1
-            for (int k0 = K_REG; k0 < g.K; k0 += CR_SUB) {
-                float x4[CR_SUB];
+                for (int k0 = kbeg; k0 < kend; k0 += CR_SUB) {
+                    float x4[CR_SUB];
 #pragma unroll
-                for (int u = 0; u < CR_SUB; u++) x4[u] = at(k0 + u);
-                online_update<CR_SUB>(mj, lj, x4);
-            }
+                    for (int u = 0; u < CR_SUB; u++) {
+                        const int k = k0 + u;
+                        x4[u] = (k < kend && rs * k < lim) ? base[k * step + loff + j] : -INFINITY;
+                    }
+                    online_update<CR_SUB>(mj, lj, x4);
+                }
+            };
+            part(0, kR);
+            part(kR, kR + K_REG);
             m[j] = mj;
             l[j] = lj;
             __builtin_amdgcn_sched_barrier(0);
@@ -497,34 +536,34 @@ __device__ __forceinline__ void cr_member_partial(const CrGeo &g, int strip, int
         for (int j = 0; j < 4; j++) { wm[wave][lc * 4 + j] = m[j]; wl[wave][lc * 4 + j] = l[j]; }
     }
     __syncthreads();
-    if (threadIdx.x < CR_W) {
-        float M = wm[0][threadIdx.x], L = wl[0][threadIdx.x];
-#pragma unroll
-        for (int w = 1; w < CR_NW; w++) merge_pair(M, L, wm[w][threadIdx.x], wl[w][threadIdx.x]);
-        Mout = M;
-        Lout = L;
-    }
+    if (threadIdx.x < CR_W) cr_merge16(wm, wl, threadIdx.x, Mout, Lout);
     __syncthreads();
 }
 
-// The members' partials in tot[p][0 = max, 1 = sum][column] -> the strip's column maxima and sums, merged in a
-// fixed order (sixteen groups of members, then the groups); valid in threads 0..63 on return.
-__device__ __forceinline__ void cr_merge_members(int csplit, const float (*tot)[2][CR_W], float (*wm)[CR_W], float (*wl)[CR_W],
-                                                 float &Mout, float &Lout) {
+constexpr int CR_MPG = CR_MAX_SPLIT / CR_NW;     // members per group of 64 threads (thread = group, column)
+
+// The members' partials, four members per thread (pm, pl: member grp * mpg + q of column c) -> the strip's column
+// maxima and sums: the maximum first, then every member's sum rescaled to it and added in a fixed order (within the
+// sixteen groups, then the groups); valid in threads 0..63 on return.
+__device__ __forceinline__ void cr_merge_members(const float (&pm)[CR_MPG], const float (&pl)[CR_MPG], float (*wm)[CR_W],
+                                                 float (*wl)[CR_W], float &Mout, float &Lout) {
     const int c = threadIdx.x & 63, grp = threadIdx.x >> 6;
-    const int mpg = (csplit + CR_NW - 1) / CR_NW;
-    float M = -INFINITY, L = 0.f;
-    for (int q = 0; q < mpg; q++) {
-        const int p = grp * mpg + q;
-        if (p < csplit) merge_pair(M, L, tot[p][0][c], tot[p][1][c]);
-    }
+    float M = pm[0];
+#pragma unroll
+    for (int q = 1; q < CR_MPG; q++) M = fmaxf(M, pm[q]);
     wm[grp][c] = M;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < CR_NW; w++) M = fmaxf(M, wm[w][c]);
+    float L = 0.f;
+#pragma unroll
+    for (int q = 0; q < CR_MPG; q++) L += pl[q] * exp_neg(pm[q] - M);      // a member that is absent has sum 0
     wl[grp][c] = L;
     __syncthreads();
     if (threadIdx.x < CR_W) {
-        M = wm[0][threadIdx.x]; L = wl[0][threadIdx.x];
+        L = wl[0][threadIdx.x];
 #pragma unroll
-        for (int w = 1; w < CR_NW; w++) merge_pair(M, L, wm[w][threadIdx.x], wl[w][threadIdx.x]);
+        for (int w = 1; w < CR_NW; w++) L += wl[w][threadIdx.x];
         Mout = M;
         Lout = L;
     }
@@ -556,7 +595,7 @@ __device__ __forceinline__ bool cr_wait_slot(const unsigned long long *sp, unsig
 
 // grid: strips * csplit workgroups, all resident at once (one per compute unit).  Workgroup b: strip b % strips,
 // member b / strips, so that the workgroups that read the pieces of one row are neighbours in time.
-template <int K_REG, int K_LDS>
+template <int K_REG, int K_LDS, bool NT>
 __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restrict__ dlogits, const float *__restrict__ logits,
                                                                  const int32_t *__restrict__ targets, int V, int S,
                                                                  int strips, int csplit, int Rm, int K, float invS,
@@ -564,24 +603,33 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
                                                                  int spin_ticks) {
     __shared__ v4f lrow[K_LDS][CR_THREADS];
     __shared__ float wm[CR_NW][CR_W], wl[CR_NW][CR_W];
-    __shared__ float tot[CR_MAX_SPLIT][2][CR_W];
+    __shared__ float fb[2][CR_W];                  // one member's partial on its way to the threads that hold it
     __shared__ float fM[CR_W], fInv[CR_W];
     __shared__ float strip_loss[CR_MAX_STRIPS];
     __shared__ unsigned want[CR_MAX_SPLIT], want_leader[CR_MAX_STRIPS];
     __shared__ int failed[CR_MAX_SPLIT];
+    __shared__ int any_failed;
     const int tid = threadIdx.x;
-    const int b = blockIdx.x;
-    const int strip = b % strips, me = b / strips;
+    // Workgroups are dealt to the eight XCDs in turn.  The workgroups that read the pieces of one row run at the
+    // same time and, where the split allows, on one XCD, so that each L2 sees whole rows.
+    int strip = blockIdx.x % strips, me = blockIdx.x / strips;
+    if (csplit % 8 == 0) {
+        const int xcd = blockIdx.x % 8, q = blockIdx.x / 8;
+        strip = q % strips;
+        me = xcd + 8 * (q / strips);
+    }
+    const int b = me * strips + strip;           // the workgroup number that owns slots and counter
     const CrGeo g = {logits, V, S, strips, csplit, Rm, K};
     if (tid < csplit) { want[tid] = ws.cnt[tid * strips + strip] + 1u; failed[tid] = 0; }
     if (tid < strips) want_leader[tid] = ws.cnt[tid] + 1u;          // member 0 of strip s is workgroup s
+    if (tid == 0) any_failed = 0;
     const unsigned my_tag = ws.cnt[b] + 1u;
     __syncthreads();
 
     // ---- pass 1: this member's rows, kept; its partial published
     v4f xr[K_REG];
     float Mp = -INFINITY, Lp = 0.f;
-    cr_member_partial<K_REG, K_LDS, true>(g, strip, me, xr, lrow, wm, wl, Mp, Lp);
+    cr_member_partial<K_REG, K_LDS, true, NT>(g, strip, me, xr, lrow, wm, wl, Mp, Lp);
     if (tid < CR_W) {
         unsigned long long *mine = ws.slots + (size_t)b * CR_STRIDE;
         __hip_atomic_store(mine + tid, ((unsigned long long)my_tag << 32) | __float_as_uint(Mp), __ATOMIC_RELAXED,
@@ -589,26 +637,69 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
         __hip_atomic_store(mine + CR_W + tid, ((unsigned long long)my_tag << 32) | __float_as_uint(Lp), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     }
-    // ---- every member's partial: 128 slots each
-    for (int i = tid; i < csplit * 2 * CR_W; i += CR_THREADS) {
-        const int p = i >> 7, r = i & 127;
-        float val = 0.f;
-        if (!cr_wait_slot(ws.slots + (size_t)(p * strips + strip) * CR_STRIDE + r, want[p], spin_ticks, val)) failed[p] = 1;
-        tot[p][r >> 6][r & 63] = val;
-    }
-    __syncthreads();
-    bool counted = false;
-    for (int p = 0; p < csplit; p++) {
-        if (failed[p]) {                                             // the same for every thread: read after the barrier
-            if (tid == 0 && !counted) { atomicAdd(ws.fallbacks, 1); counted = true; }
-            float M2 = -INFINITY, L2 = 0.f;
-            cr_member_partial<K_REG, K_LDS, false>(g, strip, p, xr, lrow, wm, wl, M2, L2);
-            if (tid < CR_W) { tot[p][0][tid] = M2; tot[p][1][tid] = L2; }
+    // ---- every member's partial.  Thread (group, column) fetches the (max, sum) slots of the group's members for
+    // its column: eight slots.  The loads of a round go out together, so a round costs one trip to the memory side
+    // however many of the eight are still missing.
+    const int mc = tid & 63, mgrp = tid >> 6;
+    const int mpg = (csplit + CR_NW - 1) / CR_NW;                      // members per group, at most CR_MPG
+    float pm[CR_MPG], pl[CR_MPG];
+    {
+        unsigned pend = 0;
+#pragma unroll
+        for (int q = 0; q < CR_MPG; q++) {
+            pm[q] = -INFINITY;
+            pl[q] = 0.f;
+            if (q < mpg && mgrp * mpg + q < csplit) pend |= 3u << (2 * q);
+        }
+        const long long t0 = wall_clock64();
+        while (pend) {
+            unsigned long long pk[2 * CR_MPG];
+#pragma unroll
+            for (int f = 0; f < 2 * CR_MPG; f++) {
+                const int p = mgrp * mpg + (f >> 1);
+                if ((pend >> f) & 1u)
+                    pk[f] = __hip_atomic_load(ws.slots + (size_t)(p * strips + strip) * CR_STRIDE + (f & 1) * CR_W + mc,
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int f = 0; f < 2 * CR_MPG; f++) {
+                const int p = mgrp * mpg + (f >> 1);
+                if (((pend >> f) & 1u) && (unsigned)(pk[f] >> 32) == want[p]) {
+                    if (f & 1) pl[f >> 1] = __uint_as_float((unsigned)pk[f]);
+                    else pm[f >> 1] = __uint_as_float((unsigned)pk[f]);
+                    pend &= ~(1u << f);
+                }
+            }
+            if (pend) {
+                if (wall_clock64() - t0 >= (long long)spin_ticks) {
+#pragma unroll
+                    for (int f = 0; f < 2 * CR_MPG; f++)
+                        if ((pend >> f) & 1u) failed[mgrp * mpg + (f >> 1)] = 1;
+                    any_failed = 1;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
         }
     }
     __syncthreads();
+    if (any_failed) {                                                // the same for every thread: read after the barrier
+        if (tid == 0) atomicAdd(ws.fallbacks, 1);
+        for (int p = 0; p < csplit; p++) {
+            if (failed[p]) {
+                float M2 = -INFINITY, L2 = 0.f;
+                cr_member_partial<K_REG, K_LDS, false>(g, strip, p, xr, lrow, wm, wl, M2, L2);
+                if (tid < CR_W) { fb[0][tid] = M2; fb[1][tid] = L2; }
+                __syncthreads();
+#pragma unroll
+                for (int q = 0; q < CR_MPG; q++)
+                    if (q < mpg && mgrp * mpg + q == p) { pm[q] = fb[0][mc]; pl[q] = fb[1][mc]; }
+                __syncthreads();
+            }
+        }
+    }
     float Mc = 0.f, Lc = 1.f;
-    cr_merge_members(csplit, tot, wm, wl, Mc, Lc);
+    cr_merge_members(pm, pl, wm, wl, Mc, Lc);
     if (tid < CR_W) {
         const float inv = 1.0f / Lc;
         fM[tid] = Mc;
@@ -625,17 +716,19 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
     }
     __syncthreads();
 
-    // ---- pass 2: dlogits = (exp(l - M) / L - onehot) / S * grad_scale; the rows read last come first
+    // ---- pass 2: dlogits = (exp(l - M) / L - onehot) / S * grad_scale
     {
         const int lc = tid & 15;
         int row0 = tid >> 4;
         asm volatile("" : "+v"(row0));     // the row masks are formed again here instead of being kept from pass 1
         const int v_lo = me * Rm;
-        const int lim = min(V, v_lo + Rm) - v_lo - row0;           // this lane's rows row0 + 64k exist while 64k < lim
+        constexpr int rs = CR_RPS;
+        const int lim = min(V, v_lo + Rm) - v_lo - row0;           // this lane's rows row0 + rs*k exist while rs*k < lim
+        const int kR = max(0, K - K_REG), kL = max(0, kR - K_LDS);
         const float *src = logits + ((size_t)v_lo * S + (size_t)strip * CR_W);
         float *dst = dlogits + ((size_t)v_lo * S + (size_t)strip * CR_W);
         const unsigned loff = (unsigned)row0 * (unsigned)S + (unsigned)lc * 4u;
-        const size_t step = (size_t)CR_RPS * S;
+        const size_t step = (size_t)rs * S;
         float M[4], inv[4], sc[4];
         int tk[4];                         // the target's row is this lane's row 64k when tk == 64k
 #pragma unroll
@@ -652,31 +745,49 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 float pj = exp_neg(x[j] - M[j]) * inv[j];
-                if (tk[j] == CR_RPS * k) pj -= 1.0f;
+                if (tk[j] == rs * k) pj -= 1.0f;
                 pj = pj * sc[j];
                 if (grad_scale != 1.0f) pj = pj * grad_scale;
                 o[j] = pj;
             }
             st4_nt(dst + k * step + loff, o);
         };
-        for (int k0 = K_REG + K_LDS; k0 < K; k0 += CR_SUB) {
-            v4f t[CR_SUB];
+        // the rows read a second time run up to sixteen ahead of their use, in the registers that the register
+        // rows leave as they are written out
+        auto loadg = [&](v4f (&t)[CR_SUB], int k0) {
 #pragma unroll
             for (int u = 0; u < CR_SUB; u++)
-                if (CR_RPS * (k0 + u) < lim) t[u] = ld4_nt(src + (k0 + u) * step + loff);
+                if (k0 + u < kL && rs * (k0 + u) < lim) t[u] = ld4_nt(src + (k0 + u) * step + loff);
+        };
+        auto emitg = [&](const v4f (&t)[CR_SUB], int k0) {
 #pragma unroll
             for (int u = 0; u < CR_SUB; u++)
-                if (CR_RPS * (k0 + u) < lim) emit(k0 + u, t[u]);
-        }
+                if (k0 + u < kL && rs * (k0 + u) < lim) emit(k0 + u, t[u]);
+        };
+        v4f t0[CR_SUB], t1[CR_SUB], t2[CR_SUB], t3[CR_SUB];
+        loadg(t0, 0);
 #pragma unroll
-        for (int k = 0; k < K_LDS; k++) {
-            if (CR_RPS * (K_REG + k) < lim) emit(K_REG + k, lrow[k][tid]);
+        for (int i = 0; i < K_REG; i++) {
+            if (rs * (kR + i) < lim) emit(kR + i, xr[i]);
             __builtin_amdgcn_sched_barrier(0);       // one row at a time: the scheduler would otherwise hold them all
         }
+        loadg(t1, CR_SUB);
+        loadg(t2, 2 * CR_SUB);
+        loadg(t3, 3 * CR_SUB);
 #pragma unroll
-        for (int k = 0; k < K_REG; k++) {
-            if (CR_RPS * k < lim) emit(k, xr[k]);
+        for (int i = 0; i < K_LDS; i++) {
+            if (kL + i < kR && rs * (kL + i) < lim) emit(kL + i, lrow[i][tid]);
             __builtin_amdgcn_sched_barrier(0);
+        }
+        for (int k0 = 0; k0 < kL; k0 += 4 * CR_SUB) {
+            emitg(t0, k0);
+            loadg(t0, k0 + 4 * CR_SUB);
+            emitg(t1, k0 + CR_SUB);
+            loadg(t1, k0 + 5 * CR_SUB);
+            emitg(t2, k0 + 2 * CR_SUB);
+            loadg(t2, k0 + 6 * CR_SUB);
+            emitg(t3, k0 + 3 * CR_SUB);
+            loadg(t3, k0 + 7 * CR_SUB);
         }
     }
 
@@ -693,14 +804,21 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
         __syncthreads();
         for (int s2 = 1; s2 < strips; s2++) {
             if (failed[s2]) {                                        // that strip's loss term from memory, the same way
+                float qm[CR_MPG], ql[CR_MPG];
+#pragma unroll
+                for (int q = 0; q < CR_MPG; q++) { qm[q] = -INFINITY; ql[q] = 0.f; }
                 for (int p = 0; p < csplit; p++) {
                     float M2 = -INFINITY, L2 = 0.f;
                     cr_member_partial<K_REG, K_LDS, false>(g, s2, p, xr, lrow, wm, wl, M2, L2);
-                    if (tid < CR_W) { tot[p][0][tid] = M2; tot[p][1][tid] = L2; }
+                    if (tid < CR_W) { fb[0][tid] = M2; fb[1][tid] = L2; }
+                    __syncthreads();
+#pragma unroll
+                    for (int q = 0; q < CR_MPG; q++)
+                        if (q < mpg && mgrp * mpg + q == p) { qm[q] = fb[0][mc]; ql[q] = fb[1][mc]; }
+                    __syncthreads();
                 }
-                __syncthreads();
                 float M3 = 0.f, L3 = 1.f;
-                cr_merge_members(csplit, tot, wm, wl, M3, L3);
+                cr_merge_members(qm, ql, wm, wl, M3, L3);
                 if (tid < CR_W) {
                     const float ls = cr_strip_loss(g, s2, targets, M3, 1.0f / L3);
                     if (tid == 0) strip_loss[s2] = ls;
@@ -772,9 +890,10 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
                 xch.slots = (unsigned long long *)(base + CE_SCRATCH_BYTES);
                 xch.cnt = (unsigned *)(base + CE_SCRATCH_BYTES + (size_t)CR_MAX_WG * CR_STRIDE * 8);
                 xch.fallbacks = (int *)(base + CE_SCRATCH_BYTES + (size_t)CR_MAX_WG * CR_STRIDE * 8 + (size_t)CR_MAX_WG * 4);
-                hipLaunchKernelGGL((ce_resident_kernel<CR_K_REG, CR_K_LDS>), dim3((unsigned)(csplit * strips_r)), dim3(CR_THREADS), 0,
-                                   g_ctx.stream, (float *)dlogits, (const float *)logits, targets, V, S, strips_r, csplit, Rm, K,
-                                   1.0f / (float)S, grad_scale, loss_dev, xch, mi355_exchange_spin_ticks());
+                hipLaunchKernelGGL((ce_resident_kernel<CR_K_REG, CR_K_LDS, true>), dim3((unsigned)(csplit * strips_r)),
+                                   dim3(CR_THREADS), 0, g_ctx.stream, (float *)dlogits, (const float *)logits, targets, V, S,
+                                   strips_r, csplit, Rm, K, 1.0f / (float)S, grad_scale, loss_dev, xch,
+                                   mi355_exchange_spin_ticks());
                 LAUNCH_OK("softmax_ce (one launch)");
                 return 0;
             }

@@ -327,7 +327,7 @@ def per_op_table(br, wl, reps):
                     ("int8_quant", lambda: wl.int8(("quant",))), ("int8_dequant", lambda: wl.int8(("dequant",))),
                     ("int8_quantize_dynamic", lambda: wl.int8(("dynamic",)))):
         fn()
-        ms = time_region(br, fn, max(reps, 3))
+        ms = time_region(br, fn, max(reps, 10))
         table.append(dict(op=key, ms=ms, alg_mb=ab[key] / 1e6, gbs=ab[key] / ms / 1e6, frac=ab[key] / ms / 1e6 / PEAK_HBM_GBS))
     return table
 
