@@ -253,17 +253,25 @@ int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, 
  * pass at training/training_dynamic/train.m:497 (grad_scale; 1.0f = none).
  * dlogits = (softmax - onehot) * (1/S) * grad_scale; *loss_dev = mean_t -logf(p[tgt]+1e-10f).
  * A target outside [0,V) contributes no loss and leaves its column as the unscaled softmax
- * (stories_cpu_ops.h:98).  dlogits may alias logits. */
+ * (stories_cpu_ops.h:98).  dlogits may alias logits.
+ * fp32 logits with S a multiple of 64 (at most 1024), V >= 4096, 16-byte aligned and not in place run as ONE launch
+ * that keeps the logits in registers and LDS between the two passes (one workgroup per compute unit; partial
+ * sums exchanged inside the launch through a device array of the library, bounded wait as for the RMSNorm); every
+ * other call runs as three launches that read the logits twice.  Both forms are deterministic; they sum in
+ * different orders, so their results differ in the last bits.  Tuning knob "ce_resident": 0 = as described,
+ * 1 = the one-launch form for any V, -1 = never. */
 int mi355_softmax_ce_dev(float *dlogits, float *loss_dev, const float *logits,
                          const int32_t *targets, int V, int S, float grad_scale);
 
 /* mi355_softmax_ce_dev for callers that may not allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and the same
- * bits out, but the scratch (first-pass partials, per-column max / sum / loss) lives in a fixed 2 MiB device array
- * of the library, located once by mi355_init: the call performs no hipMalloc, no hipFree and no workspace growth.
- * Limit: 2 * ceil(V / rows per workgroup) * S * 4 + 3 * S * 4 bytes (rounded up to 256 each) must fit 2 MiB —
- * [151936, 256] needs 0.93 MiB — otherwise the call fails with a message and launches nothing.  Every call on a
- * GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race. */
+ * bits out, but the scratch lives in a fixed 3 MiB device array of the library, located once by mi355_init (call
+ * it first): the call performs no hipMalloc, no hipFree and no workspace growth.  The array holds the exchange
+ * slots of the one-launch form (which mi355_softmax_ce_dev uses from there as well) and 2 MiB for the three-launch
+ * form's first-pass partials and per-column max / sum / loss.
+ * Limit, for calls that take the three-launch form: 2 * ceil(V / rows per workgroup) * S * 4 + 3 * S * 4 bytes
+ * (rounded up to 256 each) must fit 2 MiB, otherwise the call fails with a message and launches nothing.  Every
+ * call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race. */
 int mi355_softmax_ce_noalloc_dev(float *dlogits, float *loss_dev, const float *logits, const int32_t *targets,
                                  int V, int S, float grad_scale);
 
