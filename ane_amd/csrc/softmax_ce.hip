@@ -14,6 +14,7 @@
 //           in the reverse order of pass 1 so the most recently read rows are re-read first
 //           (they are the most likely to still sit in the last-level cache).
 #include "common.h"
+#include "tile.h"
 
 #include <math.h>
 #include <type_traits>
@@ -48,12 +49,8 @@ __device__ __forceinline__ void ld_cols_nt(float (&r)[VEC], const float *p) {
 // bfloat16 logits (the optional bf16-storage variant): four columns = one 64-bit access; widened to fp32 here,
 // so everything below is the same arithmetic for both storage types.
 typedef unsigned int v2u __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ float bf_widen(unsigned bits16) { return __uint_as_float(bits16 << 16); }
-__device__ __forceinline__ unsigned bf_narrow(float f) {       // round to nearest even; NaN stays NaN
-    const unsigned u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
+__device__ __forceinline__ float bf_widen(unsigned bits16) { return bf_to_f(bits16); }
+__device__ __forceinline__ unsigned bf_narrow(float f) { return f_to_bf(f); }      // round to nearest even; NaN stays NaN
 template <int VEC>
 __device__ __forceinline__ void ld_cols(float (&r)[VEC], const uint16_t *p) {
     if constexpr (VEC == 4) {
