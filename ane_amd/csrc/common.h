@@ -31,6 +31,7 @@ struct Mi355Ctx {
     int rms_cluster;           // channel split of the clustered RMSNorm: 0 = per shape, -1 = never, 2/4/8 = forced
     int ce_resident;           // one-launch softmax-CE: 0 = where it pays, 1 = whenever the shape allows, -1 = never
     int rms_cluster_spin;      // its bounded wait in ticks of the 100 MHz clock: 0 = 2 ms, negative = do not wait at all
+                               // (-2: the one-launch cross-entropy also takes no partner's value, present or not: a test mode)
 };
 extern Mi355Ctx g_ctx;
 

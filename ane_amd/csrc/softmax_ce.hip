@@ -597,7 +597,7 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
                                                                  const int32_t *__restrict__ targets, int V, int S,
                                                                  int strips, int csplit, int Rm, int K, float invS,
                                                                  float grad_scale, float *__restrict__ loss_out, CeXch ws,
-                                                                 int spin_ticks) {
+                                                                 int spin_ticks, int take_nothing) {
     __shared__ v4f lrow[K_LDS][CR_THREADS];
     __shared__ float wm[CR_NW][CR_W], wl[CR_NW][CR_W];
     __shared__ float fb[2][CR_W];                  // one member's partial on its way to the threads that hold it
@@ -649,6 +649,13 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
             if (q < mpg && mgrp * mpg + q < csplit) pend |= 3u << (2 * q);
         }
         const long long t0 = wall_clock64();
+        if (take_nothing) {                    // test mode: every partner counts as late, whatever its slots hold
+#pragma unroll
+            for (int f = 0; f < 2 * CR_MPG; f++)
+                if ((pend >> f) & 1u) failed[mgrp * mpg + (f >> 1)] = 1;
+            any_failed = 1;
+            pend = 0;
+        }
         while (pend) {
             unsigned long long pk[2 * CR_MPG];
 #pragma unroll
@@ -795,7 +802,8 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
         __syncthreads();
         if (tid > 0 && tid < strips) {
             float val = 0.f;
-            if (!cr_wait_slot(ws.slots + (size_t)tid * CR_STRIDE + CR_LOSS_SLOT, want_leader[tid], spin_ticks, val)) failed[tid] = 1;
+            if (take_nothing || !cr_wait_slot(ws.slots + (size_t)tid * CR_STRIDE + CR_LOSS_SLOT, want_leader[tid], spin_ticks, val))
+                failed[tid] = 1;
             strip_loss[tid] = val;
         }
         __syncthreads();
@@ -890,7 +898,7 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
                 hipLaunchKernelGGL((ce_resident_kernel<CR_K_REG, CR_K_LDS, true>), dim3((unsigned)(csplit * strips_r)),
                                    dim3(CR_THREADS), 0, g_ctx.stream, (float *)dlogits, (const float *)logits, targets, V, S,
                                    strips_r, csplit, Rm, K, 1.0f / (float)S, grad_scale, loss_dev, xch,
-                                   mi355_exchange_spin_ticks());
+                                   mi355_exchange_spin_ticks(), g_ctx.rms_cluster_spin <= -2 ? 1 : 0);
                 LAUNCH_OK("softmax_ce (one launch)");
                 return 0;
             }

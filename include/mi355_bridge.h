@@ -60,7 +60,12 @@ size_t mi355_workspace_size(void);
  * "scatter_tree" (1: mi355_embed_scatter_add_dev sums long segments by a fixed tree instead of the reference's
  * sequential order: still deterministic and within 1e-5 of each row's scale, faster, no longer bit-identical to
  * the CPU loop), "buf_phase" (where mi355_buf_alloc starts buffers of 1 MiB and more within a 1 KiB group:
- * 0 = a multiple of 128 bytes that rotates from one allocation to the next, 1..8 = always (value-1)*128). */
+ * 0 = a multiple of 128 bytes that rotates from one allocation to the next, 1..8 = always (value-1)*128),
+ * "rms_cluster" (channel split of the RMSNorm over cooperating workgroups: -1 = never, 2/4/8 = forced),
+ * "ce_resident" (one-launch softmax-CE: 1 = for any V, -1 = never), "rms_cluster_spin" (how long a workgroup of those
+ * kernels and of mi355_int8_scale_dev waits for a partner's partial result before it computes it itself, in ticks
+ * of 10 ns: 0 = 2 ms; -1 = do not wait; -2 = -1, and the one-launch softmax-CE takes no partner's value at all:
+ * both are for tests, the results are the same to the bit). */
 int mi355_tune_set(const char *key, int value);
 
 /* ------------------------------------------------------------------------------------------

@@ -734,6 +734,10 @@ def test_softmax_ce_one_launch_and_its_expired_wait(br, V, S):
         br.tune("rms_cluster_spin", -1)                                  # the wait expires before it starts
         loss3, dl3 = run(1.0)
         assert loss.tobytes() == loss3.tobytes() and dl.tobytes() == dl3.tobytes()
+        if V <= 70000:
+            br.tune("rms_cluster_spin", -2)                              # and no partner's value is taken at all: every
+            loss5, dl5 = run(1.0)                                        # workgroup recomputes its whole strip, workgroup 0
+            assert loss.tobytes() == loss5.tobytes() and dl.tobytes() == dl5.tobytes()      # the other strips' loss terms
         br.tune("rms_cluster_spin", 0)
         br.tune("ce_resident", -1)                                       # the three-launch form
         loss4, dl4 = run(1.0)
