@@ -353,8 +353,9 @@ __global__ __launch_bounds__(256) void nll_grad_kernel(float *dlogits, const flo
 // ([151936][256] fp32 = 156 MB; 256 compute units x (512 KB of registers + 160 KB of LDS) = 172 MB), so one launch
 // with ONE workgroup of 1024 threads per compute unit can read most rows once: a workgroup owns a block of rows of
 // one 64-column strip (256-byte row pieces), keeps its last 16 row steps in registers and the 9 before them in LDS
-// (25 of the 38 steps of the Qwen3 vocabulary; all of them for 32000 rows), and reads only the remainder a second
-// time.  Measured at [151936][256]: 69 us against 84 us for the three launches.  The (max, sum exp) partials of the workgroups of a strip (its members)
+// (25 of the 38 steps of the Qwen3 vocabulary; all of them for 32000 rows, and for bfloat16 storage, whose rows take
+// half the space), and reads only the remainder a second time.  Measured at [151936][256]: 69 us against 84 us for
+// the three launches (bfloat16: 61 against 99).  The (max, sum exp) partials of the workgroups of a strip (its members)
 // are exchanged through tagged 8-byte slots as in the clustered RMSNorm (norm_cluster.h): one relaxed agent-scope
 // atomic {fp32 value, launch tag} per slot, a launch counter per workgroup number, nothing to clear, a bounded
 // wait.  A member whose wait for a partner expires recomputes that partner's partial from memory with the same
@@ -369,7 +370,6 @@ constexpr int CR_LOSS_SLOT = 2 * CR_W;       // after the 64 maxima and 64 sums
 constexpr int CR_STRIDE = 136;               // slots per workgroup number
 constexpr int CR_MAX_WG = 512;
 constexpr int CR_SUB = 4;                    // rows per lane and online step beyond the register rows
-constexpr int CR_K_REG = 16, CR_K_LDS = 9;   // row steps kept in registers (64 of a lane's 128) and in LDS (144 KB)
 constexpr int CR_MAX_STEPS = 64;             // beyond that most rows would be read twice anyway
 constexpr size_t CR_XCH_BYTES = (size_t)CR_MAX_WG * CR_STRIDE * 8 + (size_t)CR_MAX_WG * 4 + 256;
 
@@ -378,8 +378,43 @@ struct CeXch {
     unsigned *cnt;                 // [CR_MAX_WG] launches completed by each workgroup number
     int *fallbacks;                // workgroups whose bounded wait expired, ever (diagnostic)
 };
+// Storage of the logits: element type, the register form of a lane's four columns of one row (fp32: 16 bytes;
+// bfloat16: two packed words, widened at each use), loads, the store that rounds, and how many row steps a
+// workgroup keeps in registers (64 of a lane's 128 in both cases) and in LDS (144 KB in both cases).
+struct CrF32 {
+    typedef float T;
+    typedef v4f Raw;
+    static constexpr int K_REG = 16, K_LDS = 9;
+    static __device__ __forceinline__ Raw ld(const T *p) { return ld4(p); }
+    static __device__ __forceinline__ Raw ld_nt(const T *p) { return ld4_nt(p); }
+    static __device__ __forceinline__ Raw ninf() { Raw r = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}; return r; }
+    static __device__ __forceinline__ float at(const Raw &r, int j) { return r[j]; }
+    static __device__ __forceinline__ void st_nt(T *p, const float (&o)[4]) { Raw r = {o[0], o[1], o[2], o[3]}; st4_nt(p, r); }
+    static __device__ __forceinline__ void forget(Raw &) {}
+};
+struct CrBf16 {
+    typedef uint16_t T;
+    typedef v2u Raw;
+    static constexpr int K_REG = 32, K_LDS = 18;
+    static __device__ __forceinline__ Raw ld(const T *p) { return *reinterpret_cast<const v2u *>(p); }
+    static __device__ __forceinline__ Raw ld_nt(const T *p) { return __builtin_nontemporal_load(reinterpret_cast<const v2u *>(p)); }
+    static __device__ __forceinline__ Raw ninf() { Raw r = {0xff80ff80u, 0xff80ff80u}; return r; }
+    static __device__ __forceinline__ float at(const Raw &r, int j) { return bf_to_f((j & 1) ? r[j >> 1] >> 16 : r[j >> 1] & 0xffffu); }
+    static __device__ __forceinline__ void st_nt(T *p, const float (&o)[4]) {
+        Raw r = {f_to_bf(o[0]) | (f_to_bf(o[1]) << 16), f_to_bf(o[2]) | (f_to_bf(o[3]) << 16)};
+        __builtin_nontemporal_store(r, reinterpret_cast<v2u *>(p));
+    }
+    // Tells the compiler nothing about the words' contents from here on, so that the widened copies made for the
+    // first pass are dropped instead of being kept alive for the second (they would double the register rows).
+    static __device__ __forceinline__ void forget(Raw &r) {
+        unsigned a = r[0], b = r[1];
+        asm volatile("" : "+v"(a), "+v"(b));
+        r[0] = a; r[1] = b;
+    }
+};
+template <typename T>
 struct CrGeo {
-    const float *logits;
+    const T *logits;
     int V, S, strips, csplit, Rm, K;   // Rm rows per member, K = ceil(Rm / CR_RPS) row steps
 };
 
@@ -428,9 +463,12 @@ __device__ __forceinline__ void cr_merge16(const float (*wm)[CR_W], const float 
 // Otherwise nothing is kept: one column and one
 // group of four rows at a time, the same operations on the same values in the same order (same bits) in a handful
 // of registers, because the caller's own rows stay live in theirs.
-template <int K_REG, int K_LDS, bool KEEP, bool NT = false>
-__device__ __forceinline__ void cr_member_partial(const CrGeo &g, int strip, int p, v4f (&xr)[K_REG], v4f (*lrow)[CR_THREADS],
+template <typename ST, bool KEEP, bool NT = false>
+__device__ __forceinline__ void cr_member_partial(const CrGeo<typename ST::T> &g, int strip, int p, typename ST::Raw (&xr)[ST::K_REG],
+                                                  typename ST::Raw (*lrow)[CR_THREADS],
                                                   float (*wm)[CR_W], float (*wl)[CR_W], float &Mout, float &Lout) {
+    typedef typename ST::Raw Raw;
+    constexpr int K_REG = ST::K_REG, K_LDS = ST::K_LDS;
     static_assert(K_REG % CR_SUB == 0, "the register rows fold four at a time");
     const int lc = threadIdx.x & 15, row0 = threadIdx.x >> 4, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int v_lo = p * g.Rm;
@@ -439,33 +477,33 @@ __device__ __forceinline__ void cr_member_partial(const CrGeo &g, int strip, int
     const int lim = min(g.V, v_lo + g.Rm) - v_lo - row0;
     const int kR = max(0, g.K - K_REG), kL = max(0, kR - K_LDS);
     // a row piece = (uniform address of row v_lo + rs*k of the strip) + (this lane's fixed 32-bit offset)
-    const float *base = g.logits + ((size_t)v_lo * g.S + (size_t)strip * CR_W);
+    const typename ST::T *base = g.logits + ((size_t)v_lo * g.S + (size_t)strip * CR_W);
     const unsigned loff = (unsigned)row0 * (unsigned)g.S + (unsigned)lc * 4u;
     const size_t step = (size_t)rs * g.S;
-    const v4f ninf = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    const Raw ninf = ST::ninf();
     float m[4], l[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) { m[j] = -INFINITY; l[j] = 0.f; }
     if constexpr (KEEP) {
         // rows that stay on the chip may be read past the cache (they are not read again); the others stay cached
-        auto loadg = [&](v4f (&t)[CR_SUB], int k0) {
+        auto loadg = [&](Raw (&t)[CR_SUB], int k0) {
 #pragma unroll
             for (int u = 0; u < CR_SUB; u++) {
                 const int k = k0 + u;
-                if (k < kR && rs * k < lim) t[u] = (NT && k >= kL) ? ld4_nt(base + k * step + loff) : ld4(base + k * step + loff);
+                if (k < kR && rs * k < lim) t[u] = (NT && k >= kL) ? ST::ld_nt(base + k * step + loff) : ST::ld(base + k * step + loff);
                 else t[u] = ninf;
             }
         };
-        auto foldg = [&](const v4f (&t)[CR_SUB]) {
+        auto foldg = [&](const Raw (&t)[CR_SUB]) {
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 float x4[CR_SUB];
 #pragma unroll
-                for (int u = 0; u < CR_SUB; u++) x4[u] = t[u][j];
+                for (int u = 0; u < CR_SUB; u++) x4[u] = ST::at(t[u], j);
                 online_update<CR_SUB>(m[j], l[j], x4);
             }
         };
-        auto keepg = [&](const v4f (&t)[CR_SUB], int k0) {
+        auto keepg = [&](const Raw (&t)[CR_SUB], int k0) {
 #pragma unroll
             for (int u = 0; u < CR_SUB; u++)
                 if (k0 + u >= kL && k0 + u < kR) lrow[k0 + u - kL][threadIdx.x] = t[u];
@@ -475,10 +513,10 @@ __device__ __forceinline__ void cr_member_partial(const CrGeo &g, int strip, int
 #pragma unroll
         for (int i = 0; i < K_REG; i++) {
             const int k = kR + i;
-            xr[i] = rs * k < lim ? (NT ? ld4_nt(base + k * step + loff) : ld4(base + k * step + loff)) : ninf;
+            xr[i] = rs * k < lim ? (NT ? ST::ld_nt(base + k * step + loff) : ST::ld(base + k * step + loff)) : ninf;
         }
         {
-            v4f ta[CR_SUB], tb[CR_SUB];
+            Raw ta[CR_SUB], tb[CR_SUB];
             loadg(ta, 0);
             loadg(tb, CR_SUB);
             for (int k0 = 0; k0 < kR; k0 += 2 * CR_SUB) {
@@ -494,11 +532,13 @@ __device__ __forceinline__ void cr_member_partial(const CrGeo &g, int strip, int
         }
 #pragma unroll
         for (int c = 0; c < K_REG / CR_SUB; c++) {
-            v4f t[CR_SUB];
+            Raw t[CR_SUB];
 #pragma unroll
             for (int u = 0; u < CR_SUB; u++) t[u] = xr[c * CR_SUB + u];
             foldg(t);
         }
+#pragma unroll
+        for (int i = 0; i < K_REG; i++) ST::forget(xr[i]);
     } else {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -510,7 +550,7 @@ __device__ __forceinline__ void cr_member_partial(const CrGeo &g, int strip, int
 #pragma unroll
                     for (int u = 0; u < CR_SUB; u++) {
                         const int k = k0 + u;
-                        x4[u] = (k < kend && rs * k < lim) ? base[k * step + loff + j] : -INFINITY;
+                        x4[u] = (k < kend && rs * k < lim) ? ld_one(base + k * step + loff + j) : -INFINITY;
                     }
                     online_update<CR_SUB>(mj, lj, x4);
                 }
@@ -568,12 +608,13 @@ __device__ __forceinline__ void cr_merge_members(const float (&pm)[CR_MPG], cons
 }
 
 // Sum over the strip's columns of -log(p[target] + 1e-10), by wave 0 (every lane of it ends with the sum).
-__device__ __forceinline__ float cr_strip_loss(const CrGeo &g, int strip, const int32_t *targets, float M, float inv) {
+template <typename T>
+__device__ __forceinline__ float cr_strip_loss(const CrGeo<T> &g, int strip, const int32_t *targets, float M, float inv) {
     const int t = strip * CR_W + threadIdx.x;
     const int tg = targets[t];
     float loss = 0.f;
     if (tg >= 0 && tg < g.V) {
-        const float p = exp_neg(g.logits[(size_t)tg * g.S + t] - M) * inv;
+        const float p = exp_neg(ld_one(g.logits + (size_t)tg * g.S + t) - M) * inv;
         loss = -logf(p + 1e-10f);
     }
     return wave_sum_far_first(loss);
@@ -592,13 +633,16 @@ __device__ __forceinline__ bool cr_wait_slot(const unsigned long long *sp, unsig
 
 // grid: strips * csplit workgroups, all resident at once (one per compute unit).  Workgroup b: strip b % strips,
 // member b / strips, so that the workgroups that read the pieces of one row are neighbours in time.
-template <int K_REG, int K_LDS, bool NT>
-__global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restrict__ dlogits, const float *__restrict__ logits,
+template <typename ST, bool NT>
+__global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(typename ST::T *__restrict__ dlogits,
+                                                                 const typename ST::T *__restrict__ logits,
                                                                  const int32_t *__restrict__ targets, int V, int S,
                                                                  int strips, int csplit, int Rm, int K, float invS,
                                                                  float grad_scale, float *__restrict__ loss_out, CeXch ws,
                                                                  int spin_ticks, int take_nothing) {
-    __shared__ v4f lrow[K_LDS][CR_THREADS];
+    typedef typename ST::Raw Raw;
+    constexpr int K_REG = ST::K_REG, K_LDS = ST::K_LDS;
+    __shared__ Raw lrow[K_LDS][CR_THREADS];
     __shared__ float wm[CR_NW][CR_W], wl[CR_NW][CR_W];
     __shared__ float fb[2][CR_W];                  // one member's partial on its way to the threads that hold it
     __shared__ float fM[CR_W], fInv[CR_W];
@@ -616,7 +660,7 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
         me = xcd + 8 * (q / strips);
     }
     const int b = me * strips + strip;           // the workgroup number that owns slots and counter
-    const CrGeo g = {logits, V, S, strips, csplit, Rm, K};
+    const CrGeo<typename ST::T> g = {logits, V, S, strips, csplit, Rm, K};
     if (tid < csplit) { want[tid] = ws.cnt[tid * strips + strip] + 1u; failed[tid] = 0; }
     if (tid < strips) want_leader[tid] = ws.cnt[tid] + 1u;          // member 0 of strip s is workgroup s
     if (tid == 0) any_failed = 0;
@@ -624,9 +668,9 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
     __syncthreads();
 
     // ---- pass 1: this member's rows, kept; its partial published
-    v4f xr[K_REG];
+    Raw xr[K_REG];
     float Mp = -INFINITY, Lp = 0.f;
-    cr_member_partial<K_REG, K_LDS, true, NT>(g, strip, me, xr, lrow, wm, wl, Mp, Lp);
+    cr_member_partial<ST, true, NT>(g, strip, me, xr, lrow, wm, wl, Mp, Lp);
     if (tid < CR_W) {
         unsigned long long *mine = ws.slots + (size_t)b * CR_STRIDE;
         __hip_atomic_store(mine + tid, ((unsigned long long)my_tag << 32) | __float_as_uint(Mp), __ATOMIC_RELAXED,
@@ -692,7 +736,7 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
         for (int p = 0; p < csplit; p++) {
             if (failed[p]) {
                 float M2 = -INFINITY, L2 = 0.f;
-                cr_member_partial<K_REG, K_LDS, false>(g, strip, p, xr, lrow, wm, wl, M2, L2);
+                cr_member_partial<ST, false>(g, strip, p, xr, lrow, wm, wl, M2, L2);
                 if (tid < CR_W) { fb[0][tid] = M2; fb[1][tid] = L2; }
                 __syncthreads();
 #pragma unroll
@@ -729,8 +773,8 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
         constexpr int rs = CR_RPS;
         const int lim = min(V, v_lo + Rm) - v_lo - row0;           // this lane's rows row0 + rs*k exist while rs*k < lim
         const int kR = max(0, K - K_REG), kL = max(0, kR - K_LDS);
-        const float *src = logits + ((size_t)v_lo * S + (size_t)strip * CR_W);
-        float *dst = dlogits + ((size_t)v_lo * S + (size_t)strip * CR_W);
+        const typename ST::T *src = logits + ((size_t)v_lo * S + (size_t)strip * CR_W);
+        typename ST::T *dst = dlogits + ((size_t)v_lo * S + (size_t)strip * CR_W);
         const unsigned loff = (unsigned)row0 * (unsigned)S + (unsigned)lc * 4u;
         const size_t step = (size_t)rs * S;
         float M[4], inv[4], sc[4];
@@ -744,31 +788,31 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
             tk[j] = ok ? tg - v_lo - row0 : -1;
             sc[j] = ok ? invS : 1.0f;      // an out-of-range target leaves the column unscaled (stories_cpu_ops.h:98)
         }
-        auto emit = [&](int k, const v4f &x) {
-            v4f o;
+        auto emit = [&](int k, const Raw &x) {
+            float o[4];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                float pj = exp_neg(x[j] - M[j]) * inv[j];
+                float pj = exp_neg(ST::at(x, j) - M[j]) * inv[j];
                 if (tk[j] == rs * k) pj -= 1.0f;
                 pj = pj * sc[j];
                 if (grad_scale != 1.0f) pj = pj * grad_scale;
                 o[j] = pj;
             }
-            st4_nt(dst + k * step + loff, o);
+            ST::st_nt(dst + k * step + loff, o);
         };
         // the rows read a second time run up to sixteen ahead of their use, in the registers that the register
         // rows leave as they are written out
-        auto loadg = [&](v4f (&t)[CR_SUB], int k0) {
+        auto loadg = [&](Raw (&t)[CR_SUB], int k0) {
 #pragma unroll
             for (int u = 0; u < CR_SUB; u++)
-                if (k0 + u < kL && rs * (k0 + u) < lim) t[u] = ld4_nt(src + (k0 + u) * step + loff);
+                if (k0 + u < kL && rs * (k0 + u) < lim) t[u] = ST::ld_nt(src + (k0 + u) * step + loff);
         };
-        auto emitg = [&](const v4f (&t)[CR_SUB], int k0) {
+        auto emitg = [&](const Raw (&t)[CR_SUB], int k0) {
 #pragma unroll
             for (int u = 0; u < CR_SUB; u++)
                 if (k0 + u < kL && rs * (k0 + u) < lim) emit(k0 + u, t[u]);
         };
-        v4f t0[CR_SUB], t1[CR_SUB], t2[CR_SUB], t3[CR_SUB];
+        Raw t0[CR_SUB], t1[CR_SUB], t2[CR_SUB], t3[CR_SUB];
         loadg(t0, 0);
 #pragma unroll
         for (int i = 0; i < K_REG; i++) {
@@ -814,7 +858,7 @@ __global__ __launch_bounds__(CR_THREADS) void ce_resident_kernel(float *__restri
                 for (int q = 0; q < CR_MPG; q++) { qm[q] = -INFINITY; ql[q] = 0.f; }
                 for (int p = 0; p < csplit; p++) {
                     float M2 = -INFINITY, L2 = 0.f;
-                    cr_member_partial<K_REG, K_LDS, false>(g, s2, p, xr, lrow, wm, wl, M2, L2);
+                    cr_member_partial<ST, false>(g, s2, p, xr, lrow, wm, wl, M2, L2);
                     if (tid < CR_W) { fb[0][tid] = M2; fb[1][tid] = L2; }
                     __syncthreads();
 #pragma unroll
@@ -878,15 +922,18 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
     // compute units evenly (at least 1.75 per unit, and the last round of them as full as possible); ties go to
     // the larger block, which leaves fewer partials to merge.  At V = 151936 on 256 units: 320 rows, 475
     // workgroups (87 us for the op; 256 rows and 594 workgroups: 91 us; 384 rows and 396: 97 us).
-    if constexpr (std::is_same<T, float>::value) {
-        // The one-launch form: fp32, whole 64-column strips, out of place (a member that recomputes a partner's
-        // partial reads the partner's logits), and a vocabulary for which it pays (ce_resident: 0 = V >= 4096,
-        // 1 = any V, -1 = never).  One workgroup per compute unit at most, so that all of them are resident at once.
+    {
+        // The one-launch form: whole 64-column strips, a lane's four columns in one aligned access, out of place (a
+        // member that recomputes a partner's partial reads the partner's logits), and a vocabulary for which it
+        // pays (ce_resident: 0 = V >= 4096, 1 = any V, -1 = never).  One workgroup per compute unit at most, so that
+        // all of them are resident at once.
+        typedef typename std::conditional<std::is_same<T, float>::value, CrF32, CrBf16>::type ST;
         const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
         const int strips_r = S / CR_W;
+        const uintptr_t amask = 4 * sizeof(T) - 1;
         unsigned char *base = (g_ctx.device >= 0 && g_ctx.device < CE_MAX_DEVICES) ? g_scratch_ptr[g_ctx.device] : nullptr;
         if (g_ctx.ce_resident >= 0 && base && S % CR_W == 0 && strips_r <= CR_MAX_STRIPS && (const void *)dlogits != (const void *)logits &&
-            aligned16(logits) && aligned16(dlogits) && (V >= 4096 || g_ctx.ce_resident > 0)) {
+            (((uintptr_t)logits | (uintptr_t)dlogits) & amask) == 0 && (V >= 4096 || g_ctx.ce_resident > 0)) {
             const int csplit = cu / strips_r < CR_MAX_SPLIT ? cu / strips_r : CR_MAX_SPLIT;
             const int Rm = csplit > 0 ? (int)ceil_div((size_t)V, (size_t)csplit) : 0;
             const int K = (int)ceil_div((size_t)Rm, (size_t)CR_RPS);
@@ -895,10 +942,10 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
                 xch.slots = (unsigned long long *)(base + CE_SCRATCH_BYTES);
                 xch.cnt = (unsigned *)(base + CE_SCRATCH_BYTES + (size_t)CR_MAX_WG * CR_STRIDE * 8);
                 xch.fallbacks = (int *)(base + CE_SCRATCH_BYTES + (size_t)CR_MAX_WG * CR_STRIDE * 8 + (size_t)CR_MAX_WG * 4);
-                hipLaunchKernelGGL((ce_resident_kernel<CR_K_REG, CR_K_LDS, true>), dim3((unsigned)(csplit * strips_r)),
-                                   dim3(CR_THREADS), 0, g_ctx.stream, (float *)dlogits, (const float *)logits, targets, V, S,
-                                   strips_r, csplit, Rm, K, 1.0f / (float)S, grad_scale, loss_dev, xch,
-                                   mi355_exchange_spin_ticks(), g_ctx.rms_cluster_spin <= -2 ? 1 : 0);
+                hipLaunchKernelGGL((ce_resident_kernel<ST, true>), dim3((unsigned)(csplit * strips_r)), dim3(CR_THREADS), 0,
+                                   g_ctx.stream, dlogits, logits, targets, V, S, strips_r, csplit, Rm, K, 1.0f / (float)S,
+                                   grad_scale, loss_dev, xch, mi355_exchange_spin_ticks(),
+                                   g_ctx.rms_cluster_spin <= -2 ? 1 : 0);
                 LAUNCH_OK("softmax_ce (one launch)");
                 return 0;
             }

@@ -259,7 +259,7 @@ int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, 
  * dlogits = (softmax - onehot) * (1/S) * grad_scale; *loss_dev = mean_t -logf(p[tgt]+1e-10f).
  * A target outside [0,V) contributes no loss and leaves its column as the unscaled softmax
  * (stories_cpu_ops.h:98).  dlogits may alias logits.
- * fp32 logits with S a multiple of 64 (at most 1024), V >= 4096, 16-byte aligned and not in place run as ONE launch
+ * Logits with S a multiple of 64 (at most 1024), V >= 4096, 16-byte aligned and not in place run as ONE launch
  * that keeps the logits in registers and LDS between the two passes (one workgroup per compute unit; partial
  * sums exchanged inside the launch through a device array of the library, bounded wait as for the RMSNorm); every
  * other call runs as three launches that read the logits twice.  Both forms are deterministic; they sum in

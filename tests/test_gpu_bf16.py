@@ -126,6 +126,42 @@ def test_rmsnorm_bf16_clustered_every_split_and_the_expired_wait(br, B, C, S):
     assert H.rel_err(back(dy2), rdx) <= TOL16
 
 
+@pytest.mark.parametrize("V,S", [(4099, 64), (32000, 256), (151936, 256), (700, 128), (9000, 1024), (5000, 192)])
+def test_softmax_ce_bf16_one_launch_and_its_expired_wait(br, V, S):
+    """The bf16 instance of the kernel that keeps the logits on the chip between the passes (every row of
+    [151936,256] fits): against the oracle, the same bits run to run, with the bounded wait expired at once and with
+    no partner's value taken at all; close to the three-launch form."""
+    print("[case] bf16 softmax_ce one launch V=%d S=%d" % (V, S), flush=True)
+    lb, logits = bf(H.normal(250, (V, S), 0, 2.0))
+    tgt = np.random.default_rng(251).integers(0, V, S).astype(np.int32)
+    tgt[1] = V; tgt[S - 2] = -1
+    ld, td = dev(br, lb), dev(br, tgt)
+
+    def run():
+        dl, lossd = br.DevArray((V, S), np.uint16), br.DevArray(1)
+        br.check(br.lib.mi355_softmax_ce_bf16_dev(dl.ptr, lossd.ptr, ld.ptr, td.ptr, V, S, 1.0))
+        return lossd.numpy().copy(), dl.numpy()
+
+    try:
+        br.tune("ce_resident", 1); br.tune("rms_cluster_spin", 0)
+        loss, dl = run()
+        rl, rd = O.cross_entropy(logits, tgt)
+        assert abs(float(loss[0]) - rl) <= 1e-5 * abs(rl) and H.rel_err(O.cvt_bf16_f32(dl), rd) <= TOL16
+        loss2, dl2 = run()
+        assert loss.tobytes() == loss2.tobytes() and dl.tobytes() == dl2.tobytes()
+        for spin in ((-1, -2) if V <= 70000 else (-1,)):
+            br.tune("rms_cluster_spin", spin)
+            loss3, dl3 = run()
+            assert loss.tobytes() == loss3.tobytes() and dl.tobytes() == dl3.tobytes(), spin
+        br.tune("rms_cluster_spin", 0)
+        br.tune("ce_resident", -1)                                       # the three-launch form
+        loss4, dl4 = run()
+        assert abs(float(loss4[0]) - float(loss[0])) <= 2e-6 * abs(float(loss[0]))
+        assert H.rel_err(O.cvt_bf16_f32(dl4), O.cvt_bf16_f32(dl)) <= TOL16
+    finally:
+        br.tune("ce_resident", 0); br.tune("rms_cluster_spin", 0)
+
+
 def test_bf16_bad_arguments(br):
     a = br.DevArray(64, np.uint16); w = br.DevArray(8)
     assert br.lib.mi355_rmsnorm_fwd_bf16_dev(a.ptr, a.ptr, None, 8, 8, 1, 1e-5) == -1
