@@ -105,6 +105,34 @@ def test_softmax_ce_random_shapes(br, V, S):
     assert abs(float(lossd.numpy()[0]) - rl) <= TOL * max(abs(rl), 1e-3) and H.err_std(dl.numpy(), rd) <= TOL
 
 
+def _ce_one_launch_shapes():
+    rng = np.random.default_rng(6)
+    return [(int(rng.integers(1, 30000)), 64 * int(rng.integers(1, 17))) for _ in range(10)] + [(3, 64), (130, 256), (65, 1024)]
+
+
+@pytest.mark.parametrize("V,S", _ce_one_launch_shapes())
+def test_softmax_ce_one_launch_random_shapes(br, V, S):
+    """The one-launch form on every shape it accepts (any V, S = 64 .. 1024): members with ragged, single and no
+    rows, 1 to 16 strips; against the oracle and, to the bit, against itself with every partner's value refused."""
+    print("[case] softmax_ce one launch V=%d S=%d" % (V, S), flush=True)
+    logits = H.normal(22, (V, S), 0, 2.0)
+    tgt = np.random.default_rng(23).integers(-1, V + 1, S).astype(np.int32)
+    ld, td = dev(br, logits), dev(br, tgt)
+    rl, rd = O.cross_entropy(logits, tgt)
+    try:
+        br.tune("ce_resident", 1)
+        out = []
+        for spin in (0, -2):
+            br.tune("rms_cluster_spin", spin)
+            dl, lossd = br.DevArray(logits.shape), br.DevArray(1)
+            br.check(br.lib.mi355_softmax_ce_dev(dl.ptr, lossd.ptr, ld.ptr, td.ptr, V, S, 1.0))
+            out.append((lossd.numpy().tobytes(), dl.numpy().tobytes()))
+            assert abs(float(lossd.numpy()[0]) - rl) <= TOL * max(abs(rl), 1e-3) and H.err_std(dl.numpy(), rd) <= TOL
+        assert out[0] == out[1]
+    finally:
+        br.tune("ce_resident", 0); br.tune("rms_cluster_spin", 0)
+
+
 def _embed_cases():
     """Seeded random shapes and id distributions for the gather and the ordered scatter-add: uniform ids, Zipf ids,
     two or three hot tokens, ids of which a third are out of range, one token only; sequence lengths that are not
