@@ -31,9 +31,9 @@ PEAK_HBM_GBS = 8000.0      # MI355X published HBM3E peak
 # runs summarised in profiles/qwen3_sweep_pmc_fetch_write.md (FETCH_SIZE x 1.9992 + WRITE_SIZE x 0.9992, the
 # factors the same counters need to read 50.33 MB for a plain 50.33 MB copy).  Not measured live.
 MEASURED_TRAFFIC_BYTES = {"swiglu_bwd": 251.60e6}
-# the same for the one launch of softmax-CE on [151936,256] (fetch 208.34 + write 155.89 MB: 13 of a workgroup's 38
+# the same for the one launch of softmax-CE on [151936,256] (fetch 208.10 + write 155.81 MB: 13 of a workgroup's 38
 # row steps do not fit its registers and LDS and are read a second time), and per op of the sweep (same profile)
-CE_TRAFFIC_BYTES = 364.23e6
+CE_TRAFFIC_BYTES = 363.91e6
 OP_TRAFFIC_BYTES = {"rmsnorm_fwd": 34.04e6, "rmsnorm_bwd": 51.43e6 + 1.62e6 / 2, "qknorm_rope_fwd": 100.99e6,
                     "qknorm_rope_bwd": 152.08e6, "swiglu_fwd": 150.97e6, "swiglu_bwd": 251.60e6, "residual": 50.33e6,
                     "residual_rmsnorm_fwd": 67.64e6, "rmsnorm_bwd_residual": 85.04e6, "scale_copy": 100.66e6,
