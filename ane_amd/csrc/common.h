@@ -28,6 +28,8 @@ struct Mi355Ctx {
     size_t ws_bytes;
     // tuning knobs (0 = pick per shape)
     int rms_lpr, rms_threads, ew_unroll, ce_rows, ce_rows2, qk_lpr, qk_threads, gemm_splitk, scatter_tree, buf_phase;
+    int scatter_cols;          // ordered scatter-add with the columns of dE dealt out to the workgroups: 0 = where it pays,
+                               // 1 = whenever the shape allows, -1 = never
     int rms_cluster;           // channel split of the clustered RMSNorm: 0 = per shape, -1 = never, 2/4/8 = forced
     int ce_resident;           // one-launch softmax-CE: 0 = where it pays, 1 = whenever the shape allows, -1 = never
     int rms_cluster_spin;      // its bounded wait in ticks of the 100 MHz clock: 0 = 2 ms, negative = do not wait at all

@@ -176,7 +176,7 @@ MI355_API int mi355_tune_set(const char *key, int value) {
         {"rms_lpr", &g_ctx.rms_lpr}, {"rms_threads", &g_ctx.rms_threads},
         {"ew_unroll", &g_ctx.ew_unroll},
         {"ce_rows", &g_ctx.ce_rows}, {"ce_rows2", &g_ctx.ce_rows2}, {"buf_phase", &g_ctx.buf_phase}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
-        {"gemm_splitk", &g_ctx.gemm_splitk}, {"scatter_tree", &g_ctx.scatter_tree},
+        {"gemm_splitk", &g_ctx.gemm_splitk}, {"scatter_tree", &g_ctx.scatter_tree}, {"scatter_cols", &g_ctx.scatter_cols},
         {"rms_cluster", &g_ctx.rms_cluster}, {"rms_cluster_spin", &g_ctx.rms_cluster_spin},
         {"ce_resident", &g_ctx.ce_resident},
     };

@@ -812,6 +812,8 @@ int rows_by_index(const char *who, float *dst, const float *src, const int32_t *
     return 0;
 }
 
+#include "embed_cols.h"
+
 int key_bits(int V) {
     int bits = 1;
     while (bits < 31 && (1L << bits) <= (long)V) bits++;   // keys range over [0, V]
@@ -844,6 +846,14 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     if ((size_t)batch * S > (size_t)1 << 30) return mi355_fail("embed_scatter_add: more than 2^30 positions");
     if (!aligned16(dx) || !aligned16(dE)) return mi355_fail("embed_scatter_add: pointers must be 16-byte aligned");
     const int N = batch * S;
+    // Two forms with the same bits (embed_cols.h says what each costs).  Columns of dE owned by workgroups: dx is
+    // read where it lies, nothing is copied; chosen where one round of workgroups covers D and the positions are few
+    // enough that the small accesses to dE (one per token and workgroup) do not outweigh the copy.
+    if (!g_ctx.scatter_tree && g_ctx.scatter_cols >= 0 && S % 4 == 0 && V < (1 << (32 - CB_BITS))) {
+        const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
+        if (g_ctx.scatter_cols > 0 || (N <= SMALL_N && (int)ceil_div((size_t)D, cols_per_workgroup(D)) <= cu))
+            return scatter_add_cols(dE, dx, ids, V, D, S, N);
+    }
     const int bits = key_bits(V);
     const bool small = N <= SMALL_N && bits + POS_BITS <= 32;
     if (!small &&

@@ -59,7 +59,9 @@ size_t mi355_workspace_size(void);
  * "gemm_splitk" (K slices of mi355_sgemm_dev; 1 = never split),
  * "scatter_tree" (1: mi355_embed_scatter_add_dev sums long segments by a fixed tree instead of the reference's
  * sequential order: still deterministic and within 1e-5 of each row's scale, faster, no longer bit-identical to
- * the CPU loop), "buf_phase" (where mi355_buf_alloc starts buffers of 1 MiB and more within a 1 KiB group:
+ * the CPU loop), "scatter_cols" (the form of mi355_embed_scatter_add_dev in which every workgroup owns a few columns
+ * of the gradient table and reads its rows of dx in place: 1 = for any number of positions, -1 = never),
+ * "buf_phase" (where mi355_buf_alloc starts buffers of 1 MiB and more within a 1 KiB group:
  * 0 = a multiple of 128 bytes that rotates from one allocation to the next, 1..8 = always (value-1)*128),
  * "rms_cluster" (channel split of the RMSNorm over cooperating workgroups: -1 = never, 2/4/8 = forced),
  * "ce_resident" (one-launch softmax-CE: 1 = for any V, -1 = never), "rms_cluster_spin" (how long a workgroup of those

@@ -112,12 +112,12 @@ def test_graph_capture_refuses_ops_that_allocate(br):
     L = br.lib
     dE = br.DevArray((50, 16)); dx = br.DevArray.from_numpy(H.normal(40, (1, 16, 8)))
     ids = br.DevArray.from_numpy(np.arange(8, dtype=np.int32))
-    br.check(L.mi355_embed_scatter_add_dev(dE.ptr, dx.ptr, ids.ptr, 1 << 18, 16, 8, 1))   # sizes the workspace
+    br.check(L.mi355_embed_scatter_add_dev(dE.ptr, dx.ptr, ids.ptr, 1 << 20, 16, 8, 1))   # sizes the workspace
     br.sync()
     a = br.DevArray(64)
     br.check(L.mi355_graph_begin())
     assert L.mi355_graph_begin() == -1
-    assert L.mi355_embed_scatter_add_dev(dE.ptr, dx.ptr, ids.ptr, 1 << 18, 16, 8, 1) == -1    # library-sort path
+    assert L.mi355_embed_scatter_add_dev(dE.ptr, dx.ptr, ids.ptr, 1 << 20, 16, 8, 1) == -1    # library-sort path
     assert L.mi355_sgemm_dev(0, 0, 4, 4, 4, 1.0, a.ptr, 4, a.ptr, 4, 0.0, a.ptr, 4) == -1
     assert "captured" in br.last_error()
     br.check(L.mi355_axpby_dev(a.ptr, a.ptr, None, 2.0, 64, 1))

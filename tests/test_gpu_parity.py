@@ -518,6 +518,9 @@ def test_embed_gather_bit_exact(br, V, D, B, S, oob):
     (50, 3, 1, 257, 5),
     (20, 12001, 1, 130, 2),       # wide rows: more column chunks than compute units
     (7, 8192, 1, 600, 0),
+    (524287, 6, 3, 3000, 2),      # the largest vocabulary of the column form; a partial second block of positions
+    (2000, 770, 5, 4096, 0),      # 20480 positions, 257 workgroups of three columns, the last with two
+    (40, 515, 1, 8192, 0),        # exactly one block; one column left over for the last workgroup
 ])
 def test_embed_scatter_add_bit_exact_and_deterministic(br, V, D, B, S, oob):
     say("scatter_add V=%d D=%d B=%d S=%d" % (V, D, B, S))
@@ -525,14 +528,21 @@ def test_embed_scatter_add_bit_exact_and_deterministic(br, V, D, B, S, oob):
     dx = H.normal(63, (B, D, S))
     dE0 = H.normal(64, (V, D), 0, 0.5)
     idd, dxd = dev(br, ids), dev(br, dx)
-    outs = []
-    for _ in range(2):
-        dEd = dev(br, dE0)
-        br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, idd.ptr, V, D, S, B))
-        outs.append(dEd.numpy())
-    assert outs[0].tobytes() == outs[1].tobytes()                      # run-to-run deterministic
     ref = O.embed_backward(dE0, dx, ids)
-    assert outs[0].tobytes() == ref.tobytes()                          # the ordered fp32 sum of the reference loop
+    # the form chosen for the shape, then the two forms by name: a token-major copy of dx summed row by row (-1),
+    # columns of dE owned by workgroups (1; shapes it does not take fall back to the other)
+    for form in (0, -1, 1):
+        br.tune("scatter_cols", form)
+        try:
+            outs = []
+            for _ in range(2):
+                dEd = dev(br, dE0)
+                br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, idd.ptr, V, D, S, B))
+                outs.append(dEd.numpy())
+        finally:
+            br.tune("scatter_cols", 0)
+        assert outs[0].tobytes() == outs[1].tobytes(), form            # run-to-run deterministic
+        assert outs[0].tobytes() == ref.tobytes(), form                # the ordered fp32 sum of the reference loop
 
 
 def test_embed_scatter_add_tree_order_is_deterministic_and_close(br):
@@ -543,7 +553,7 @@ def test_embed_scatter_add_tree_order_is_deterministic_and_close(br):
     dx = H.normal(63, (B, D, S)); dE0 = H.normal(64, (V, D), 0, 0.5)
     idd, dxd = dev(br, ids), dev(br, dx)
     ref = O.embed_backward(dE0, dx, ids)
-    br.tune("scatter_tree", 1)
+    br.tune("scatter_tree", 1)                  # (selects the token-major form: the tree is an order of its long segments)
     try:
         outs = []
         for _ in range(2):
@@ -577,13 +587,48 @@ def test_embed_scatter_add_no_valid_id(br):
     assert dEd.numpy().tobytes() == dE0.tobytes()
 
 
-def test_embed_scatter_add_single_hot_token(br):
-    V, D, B, S = 10, 192, 4, 256
+@pytest.mark.parametrize("form", [-1, 1])
+@pytest.mark.parametrize("B", [4, 80])
+def test_embed_scatter_add_single_hot_token(br, form, B):
+    """One token at every position: one chain of B*256 dependent adds per column; with 80 sequences it runs through
+    three blocks of positions of the column form, carried from block to block on the chip."""
+    V, D, S = 10, 192, 256
     ids = np.full((B, S), 7, np.int32)
     dx = H.normal(65, (B, D, S)) * np.float32(100)
     dE0 = np.zeros((V, D), np.float32)
     idd, dxd, dEd = dev(br, ids), dev(br, dx), dev(br, dE0)
-    br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, idd.ptr, V, D, S, B))
+    br.tune("scatter_cols", form)
+    try:
+        br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, idd.ptr, V, D, S, B))
+    finally:
+        br.tune("scatter_cols", 0)
+    assert dEd.numpy().tobytes() == O.embed_backward(dE0, dx, ids).tobytes()
+
+
+def test_embed_scatter_add_column_form_runs_that_change_length(br):
+    """Tokens whose runs are long in one block of positions and short or absent in the next, in every order: the
+    sums carried on the chip from block to block and the ones re-read from dE must agree with the reference loop."""
+    V, D, S, B = 600, 9, 256, 128                      # 32768 positions: four blocks of 8192
+    rng = np.random.default_rng(77)
+    N = B * S
+    ids = rng.integers(300, V, N).astype(np.int32)     # background: tokens that occur a few times per block
+    blk = np.arange(N) // 8192
+    for tok, pattern in enumerate([(40, 0, 40, 40), (0, 40, 3, 40), (40, 3, 0, 1), (1, 40, 40, 0), (16, 15, 16, 15),
+                                   (2000, 2000, 1, 2000), (3, 2, 1, 0)]):
+        for b, n in enumerate(pattern):
+            pos = rng.choice(np.flatnonzero(blk == b), n, replace=False)
+            ids[pos] = tok
+    # tokens 256 apart share an entry of the table that carries sums between blocks
+    ids[rng.choice(N, 3000, replace=False)] = 256
+    ids[rng.choice(N, 3000, replace=False)] = 0
+    ids = ids.reshape(B, S)
+    dx = H.normal(68, (B, D, S)); dE0 = H.normal(69, (V, D))
+    idd, dxd, dEd = dev(br, ids), dev(br, dx), dev(br, dE0)
+    br.tune("scatter_cols", 1)
+    try:
+        br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, idd.ptr, V, D, S, B))
+    finally:
+        br.tune("scatter_cols", 0)
     assert dEd.numpy().tobytes() == O.embed_backward(dE0, dx, ids).tobytes()
 
 

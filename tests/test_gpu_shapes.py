@@ -180,10 +180,12 @@ def test_embed_gather_scatter_random_shapes(br, case, kind, V, D, B, S, seed):
     dxd, dEd = dev(br, dx), dev(br, dE0)
     tree = case % 7 == 6
     br.tune("scatter_tree", int(tree))
+    br.tune("scatter_cols", (0, -1, 1)[case % 3])       # the form chosen for the shape / token-major rows / columns of dE
     try:
         br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, idd.ptr, V, D, S, B))
     finally:
         br.tune("scatter_tree", 0)
+        br.tune("scatter_cols", 0)
     got, ref = dEd.numpy(), O.embed_backward(dE0, dx, ids)
     if not tree:
         assert got.tobytes() == ref.tobytes()
