@@ -39,8 +39,10 @@ OP_TRAFFIC_BYTES = {"rmsnorm_fwd": 34.04e6, "rmsnorm_bwd": 51.43e6 + 1.62e6 / 2,
                     "residual_rmsnorm_fwd": 67.64e6, "rmsnorm_bwd_residual": 85.04e6, "scale_copy": 100.66e6,
                     "softmax_ce": CE_TRAFFIC_BYTES, "int8_scale": 16.91e6, "int8_quant": 20.99e6, "int8_dequant": 20.99e6}
 # the same for BASELINE.json config 2 (profiles/embed_config2_pmc_fetch_write.md): the three launches of the ordered
-# scatter-add (chunk sort 0.16 + ranks and transpose 101.70 + segment sums 74.32 MB) and the gather
-SCATTER_TRAFFIC_BYTES = 176.18e6
+# scatter-add in its column form (chunk sort 0.15 + ranks 0.74 + column sums 75.65 MB), in its row form (chunk sort
+# 0.16 + ranks and transpose 101.68 + segment sums 74.32 MB), and the gather
+SCATTER_TRAFFIC_BYTES = 76.54e6
+SCATTER_ROWS_TRAFFIC_BYTES = 176.16e6
 GATHER_TRAFFIC_BYTES = 70.14e6
 
 # Qwen3-0.6B (training/training_dynamic/models/qwen3_06b.h:6-16), batch 16
@@ -443,10 +445,14 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
         gather(); scatter()
     t_g = time_region(br, gather, steps) / nbuf
     t_s = time_region(br, scatter, steps) / nbuf
-    br.tune("scatter_tree", 1)          # the opt-in fixed-tree order for long segments (deterministic, not bit-identical)
+    br.tune("scatter_cols", -1)         # the other form of the same sums: a token-major copy of dx, summed row by row
+    scatter()
+    t_s_rows = time_region(br, scatter, steps) / nbuf
+    br.tune("scatter_tree", 1)          # ... and its opt-in fixed-tree order for long segments (deterministic, not bit-identical)
     scatter()
     t_s_tree = time_region(br, scatter, steps) / nbuf
     br.tune("scatter_tree", 0)
+    br.tune("scatter_cols", 0)
 
     def copy():                         # y = 1.0*a over one activation slab: the streaming rate next to the two ops, and
         for x, g in zip(xs, gs):        # the known-size dispatch that scales the traffic counters of the profile
@@ -470,9 +476,12 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
                    row("embed_scatter_add", t_s, b_s, traffic_mb=SCATTER_TRAFFIC_BYTES / 1e6,
                        traffic_frac=SCATTER_TRAFFIC_BYTES / t_s / 1e6 / PEAK_HBM_GBS,
                        traffic_source="profiles/embed_config2_pmc_fetch_write.md"),
-                   row("embed_scatter_add (scatter_tree=1)", t_s_tree, b_s),
+                   row("embed_scatter_add (scatter_cols=-1: token-major copy, row sums)", t_s_rows, b_s,
+                       traffic_mb=SCATTER_ROWS_TRAFFIC_BYTES / 1e6,
+                       traffic_frac=SCATTER_ROWS_TRAFFIC_BYTES / t_s_rows / 1e6 / PEAK_HBM_GBS),
+                   row("embed_scatter_add (scatter_cols=-1, scatter_tree=1)", t_s_tree, b_s),
                    row("copy of one activation slab", t_c, 8 * D * N)],
-           "roofline": dict(bound="hbm", kernel="embed_scatter_add (3 launches)", achieved=b_s / t_s / 1e6, peak=PEAK_HBM_GBS,
+           "roofline": dict(bound="hbm", kernel="embed_scatter_add (3 launches: chunk sort, ranks, column sums)", achieved=b_s / t_s / 1e6, peak=PEAK_HBM_GBS,
                             unit="GB/s", frac=b_s / t_s / 1e6 / PEAK_HBM_GBS,
                             traffic=SCATTER_TRAFFIC_BYTES, traffic_source="profiles/embed_config2_pmc_fetch_write.md",
                             alg_bytes_per_launch=b_s, avg_launch_ms=t_s)}

@@ -251,7 +251,10 @@ int mi355_embed_gather_dev(float *x, const float *E, const int32_t *ids, int V, 
 /* Embedding backward.  Replaces embed_backward — training/stories_cpu_ops.h:123-131,
  * training/training_dynamic/cpu_ops.h:158-164.  dE[ids[b][t]][d] += dx[b][d][t], each (row, d) sum
  * taken in ascending (b, t) order starting from the value already in dE, so the result is
- * bit-identical to the reference loop and run-to-run deterministic.  Ids outside [0,V) are skipped. */
+ * bit-identical to the reference loop and run-to-run deterministic.  Ids outside [0,V) are skipped.
+ * Two forms give the same bits: up to 16384 positions (S a multiple of 4, V < 2^19, D within one round of workgroups)
+ * every workgroup owns a few columns of dE and reads its rows of dx in place; otherwise dx is first copied
+ * token-major and summed row by row (the "scatter_cols" knob names a form). */
 int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, int V, int D,
                                 int S, int batch);
 
