@@ -849,7 +849,7 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     // Two forms with the same bits (embed_cols.h says what each costs).  Columns of dE owned by workgroups: dx is
     // read where it lies, nothing is copied; chosen where one round of workgroups covers D and the positions are few
     // enough that the small accesses to dE (one per token and workgroup) do not outweigh the copy.
-    if (!g_ctx.scatter_tree && g_ctx.scatter_cols >= 0 && S % 4 == 0 && V < (1 << (32 - CB_BITS))) {
+    if (!g_ctx.scatter_tree && g_ctx.scatter_cols >= 0 && (S % 4 == 0 || N <= COL_SMALL) && V < (1 << (32 - CB_BITS))) {
         const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
         if (g_ctx.scatter_cols > 0 || (N <= SMALL_N && (int)ceil_div((size_t)D, cols_per_workgroup(D)) <= cu))
             return scatter_add_cols(dE, dx, ids, V, D, S, N);

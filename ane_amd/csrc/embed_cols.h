@@ -11,7 +11,7 @@
 // ranks ascending; dE = acc.  Blocks in ascending order and ranks ascending within a run are the order of the
 // reference loop, so the result is that loop's bit for bit.
 //
-// Three launches:
+// Three launches (one, col_sum_small_kernel, up to 512 positions):
 //   1. chunk_sort_blk_kernel: every 256 consecutive (token, position-in-block) words sorted by counting.
 //   2. block_rank_kernel: the sorted chunks of a block merged by rank (16 lanes per position, a binary search per
 //      chunk): rk[position] = its rank within the block, and the block's runs {token, first rank, length}, long runs
@@ -347,11 +347,110 @@ __global__ __launch_bounds__(1024) void col_sum_kernel(float *dE, const float *_
     }
 }
 
+// Up to COL_SMALL positions (one sequence of the reference's loops): plan and sums in ONE launch.  Every workgroup
+// ranks all positions itself in LDS (two threads per position count the smaller words; 1 us, redundant but without
+// a launch boundary), marks the first rank of every run in a 512-bit mask, writes its K columns of dx to LDS at their
+// ranks and sums the runs, one lane per (run, column), from dE and back to it.  Any S.
+constexpr int COL_SMALL = 512, COL_SMALL_BITS = 10;
+
+template <int K>
+__global__ __launch_bounds__(1024) void col_sum_small_kernel(float *dE, const float *__restrict__ dx,
+                                                             const int32_t *__restrict__ ids, int N, int V, int D, int S) {
+    constexpr int XP = COL_SMALL + 48;
+    __shared__ __attribute__((aligned(16))) unsigned words[COL_SMALL];
+    __shared__ unsigned sorted[COL_SMALL];
+    __shared__ unsigned short rank_of[COL_SMALL];
+    __shared__ unsigned long long heads[COL_SMALL / 64];
+    __shared__ __attribute__((aligned(16))) float xs[K][XP];
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int d0 = xcd_remap(blockIdx.x, gridDim.x) * K;
+    const int kv = min(K, D - d0);
+    // this thread's values of dx: element i = column i / N, position i % N (coalesced along the positions)
+    constexpr int XPT = (COL_SMALL * K + 1023) / 1024;
+    float xv[XPT];
+#pragma unroll
+    for (int q = 0; q < XPT; q++) {
+        const int i = t + 1024 * q, d = i / N, p = i - d * N;
+        xv[q] = 0.f;
+        if (d < kv) {
+            const int b = p / S;
+            xv[q] = dx[((size_t)b * D + d0 + d) * S + (p - b * S)];
+        }
+    }
+    if (t < COL_SMALL) {
+        unsigned key = (unsigned)V;                             // padding and out-of-range ids sort last
+        if (t < N) {
+            const int id = ids[t];
+            if (id >= 0 && id < V) key = (unsigned)id;
+        }
+        words[t] = (key << COL_SMALL_BITS) | (unsigned)t;
+    }
+    __syncthreads();
+    {
+        const int p = t >> 1, h = t & 1;
+        const unsigned w = words[p];
+        int r = 0;
+#pragma unroll 8
+        for (int j = 0; j < COL_SMALL / 2; j += 4) {
+            const v4u q = *reinterpret_cast<const v4u *>(&words[h * (COL_SMALL / 2) + j]);
+            r += (q.x < w ? 1 : 0) + (q.y < w ? 1 : 0) + (q.z < w ? 1 : 0) + (q.w < w ? 1 : 0);
+        }
+        r += __shfl_xor(r, 1, 64);
+        if (h == 0) {
+            rank_of[p] = (unsigned short)r;
+            sorted[r] = w;
+        }
+    }
+    __syncthreads();
+    if (t < COL_SMALL) {
+        // a run starts where the token changes; the first padding word starts one too, so every run ends at a mark
+        const bool head = t == 0 || (sorted[t - 1] >> COL_SMALL_BITS) != (sorted[t] >> COL_SMALL_BITS);
+        const unsigned long long m = __builtin_amdgcn_ballot_w64(head);
+        if (lane == 0) heads[wave] = m;
+    }
+#pragma unroll
+    for (int q = 0; q < XPT; q++) {
+        const int i = t + 1024 * q, d = i / N, p = i - d * N;
+        if (d < K) xs[d][rank_of[p]] = xv[q];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < XPT; q++) {
+        const int i = t + 1024 * q, d = i / COL_SMALL, r = i % COL_SMALL;
+        const unsigned tok = sorted[r] >> COL_SMALL_BITS;
+        const bool head = (heads[r >> 6] >> (r & 63)) & 1ull;
+        if (d < kv && head && tok < (unsigned)V) {
+            // the next mark after r
+            int end = COL_SMALL;
+            unsigned long long m = (r & 63) == 63 ? 0ull : (heads[r >> 6] >> ((r & 63) + 1));
+            if (m) end = r + 1 + __builtin_ctzll(m);
+            else
+                for (int wq = (r >> 6) + 1; wq < COL_SMALL / 64; wq++)
+                    if (heads[wq]) { end = wq * 64 + __builtin_ctzll(heads[wq]); break; }
+            float *dst = dE + (size_t)tok * D + d0 + d;
+            *dst = long_chain(*dst, &xs[d][0], r, end - r);
+        }
+    }
+}
+
 // Columns of dE per workgroup: three from D = 513 on (256 workgroups at D = 768).
 int cols_per_workgroup(int D) { return D > 512 ? 3 : D > 256 ? 2 : 1; }
 
-// Launches the three kernels.  The caller has checked: S a multiple of 4, V < 2^(32 - CB_BITS), dx 16-byte aligned.
+// Launches the kernels of the column form.  The caller has checked: V < 2^(32 - CB_BITS) and, beyond COL_SMALL
+// positions, S a multiple of 4 and dx 16-byte aligned.
 int scatter_add_cols(float *dE, const float *dx, const int32_t *ids, int V, int D, int S, int N) {
+    const int K = cols_per_workgroup(D);
+    const dim3 grid((unsigned)ceil_div((size_t)D, K));
+    if (N <= COL_SMALL) {
+#define COL_LAUNCH(KK)                                                                                              \
+    case KK:                                                                                                        \
+        hipLaunchKernelGGL(col_sum_small_kernel<KK>, grid, dim3(1024), 0, g_ctx.stream, dE, dx, ids, N, V, D, S);   \
+        break;
+        switch (K) { COL_LAUNCH(1) COL_LAUNCH(2) COL_LAUNCH(3) }
+#undef COL_LAUNCH
+        LAUNCH_OK("embed_scatter_add column sums");
+        return 0;
+    }
     const int nchunks = (int)ceil_div((size_t)N, CHUNK), nblk = (int)ceil_div((size_t)N, CB);
     size_t total = 0;
     auto take = [&total](size_t bytes) {
@@ -374,8 +473,6 @@ int scatter_add_cols(float *dE, const float *dx, const int32_t *ids, int V, int 
     hipLaunchKernelGGL(block_rank_kernel, dim3((unsigned)ceil_div((size_t)N, 64)), dim3(1024), 0, g_ctx.stream, rk, tasks,
                        cnt, sorted_chunks, ids, N, V, nchunks);
     LAUNCH_OK("embed_scatter_add plan");
-    const int K = cols_per_workgroup(D);
-    const dim3 grid((unsigned)ceil_div((size_t)D, K));
 #define COL_LAUNCH(KK)                                                                                              \
     case KK:                                                                                                        \
         hipLaunchKernelGGL(col_sum_kernel<KK>, grid, dim3(1024), 0, g_ctx.stream, dE, dx, tasks, cnt, rk, N, D, S, nblk); \

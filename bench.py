@@ -454,6 +454,19 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
     br.tune("scatter_tree", 0)
     br.tune("scatter_cols", 0)
 
+    # one sequence of 256 ids: the reference's own call (embed_backward once per training step, S = 256)
+    def scatter_one():
+        for g, dE in zip(gs, dEs):
+            br.check(br.lib.mi355_embed_scatter_add_dev(dE.ptr, g.ptr, idd.ptr, V, D, S, 1))
+    scatter_one()
+    t_s1 = time_region(br, scatter_one, steps) / nbuf
+    br.tune("scatter_cols", -1)
+    scatter_one()
+    t_s1_rows = time_region(br, scatter_one, steps) / nbuf
+    br.tune("scatter_cols", 0)
+    U1 = int(np.unique(ids[0]).size)
+    b_s1 = 4 * D * S + 8 * D * U1 + 4 * S
+
     def copy():                         # y = 1.0*a over one activation slab: the streaming rate next to the two ops, and
         for x, g in zip(xs, gs):        # the known-size dispatch that scales the traffic counters of the profile
             br.check(br.lib.mi355_axpby_dev(x.ptr, g.ptr, None, 1.0, g.size, 1))
@@ -480,6 +493,8 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
                        traffic_mb=SCATTER_ROWS_TRAFFIC_BYTES / 1e6,
                        traffic_frac=SCATTER_ROWS_TRAFFIC_BYTES / t_s_rows / 1e6 / PEAK_HBM_GBS),
                    row("embed_scatter_add (scatter_cols=-1, scatter_tree=1)", t_s_tree, b_s),
+                   row("embed_scatter_add, one sequence of 256 ids", t_s1, b_s1),
+                   row("embed_scatter_add, one sequence of 256 ids (scatter_cols=-1)", t_s1_rows, b_s1),
                    row("copy of one activation slab", t_c, 8 * D * N)],
            "roofline": dict(bound="hbm", kernel="embed_scatter_add (3 launches: chunk sort, ranks, column sums)", achieved=b_s / t_s / 1e6, peak=PEAK_HBM_GBS,
                             unit="GB/s", frac=b_s / t_s / 1e6 / PEAK_HBM_GBS,

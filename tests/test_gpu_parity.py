@@ -521,6 +521,10 @@ def test_embed_gather_bit_exact(br, V, D, B, S, oob):
     (524287, 6, 3, 3000, 2),      # the largest vocabulary of the column form; a partial second block of positions
     (2000, 770, 5, 4096, 0),      # 20480 positions, 257 workgroups of three columns, the last with two
     (40, 515, 1, 8192, 0),        # exactly one block; one column left over for the last workgroup
+    (100, 7, 2, 256, 0),          # 512 positions: the most the single-launch column kernel takes
+    (100, 7, 4, 129, 1),          # 516: one more (S not a multiple of 4: row form)
+    (3000, 770, 1, 511, 3),       # single launch, S odd, 257 workgroups, the last with two columns
+    (2, 1, 1, 512, 0),            # single launch: two runs of ~256, one column
 ])
 def test_embed_scatter_add_bit_exact_and_deterministic(br, V, D, B, S, oob):
     say("scatter_add V=%d D=%d B=%d S=%d" % (V, D, B, S))
