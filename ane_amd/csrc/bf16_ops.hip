@@ -444,12 +444,16 @@ __global__ __launch_bounds__(THREADS) void qknorm_rope_bwd_bf16_kernel(
         float g0[VEC], g1[VEC], c[VEC], sn[VEC];
         unpack<VEC>(g0, rg0[kk]);
         unpack<VEC>(g1, rg1[kk]);
-        if (rp < half && col_ok) {
-            ldtab<VEC>(c, cos_t + (size_t)rp * S + col);
-            ldtab<VEC>(sn, sin_t + (size_t)rp * S + col);
-        } else {
+        // (loaded from a valid address in every lane and zeroed by selects: with the loads under a branch the
+        // compiler merges the two paths through scratch memory, and a kernel with scratch is dispatched later)
+        const bool ok = rp < half && col_ok;
+        const size_t to = ok ? (size_t)rp * S + col : 0;
+        ldtab<VEC>(c, cos_t + to);
+        ldtab<VEC>(sn, sin_t + to);
 #pragma unroll
-            for (int j = 0; j < VEC; j++) c[j] = sn[j] = 0.f;
+        for (int j = 0; j < VEC; j++) {
+            c[j] = ok ? c[j] : 0.f;
+            sn[j] = ok ? sn[j] : 0.f;
         }
 #pragma unroll
         for (int j = 0; j < VEC; j++) {

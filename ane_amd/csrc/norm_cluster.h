@@ -65,7 +65,7 @@ struct StoreBf16 {
     static __device__ __forceinline__ Raw pack(const float (&v)[VEC]) {
         Raw r;
 #pragma unroll
-        for (int j = 0; j < 4; j++) r[j] = f_to_bf(v[2 * j]) | (f_to_bf(v[2 * j + 1]) << 16);
+        for (int j = 0; j < 4; j++) r[j] = f2_to_bf2(v[2 * j], v[2 * j + 1]);
         return r;
     }
     static __device__ __forceinline__ Raw zero() { return raw_zero<VEC>(); }

@@ -401,7 +401,7 @@ struct CrBf16 {
     static __device__ __forceinline__ Raw ninf() { Raw r = {0xff80ff80u, 0xff80ff80u}; return r; }
     static __device__ __forceinline__ float at(const Raw &r, int j) { return bf_to_f((j & 1) ? r[j >> 1] >> 16 : r[j >> 1] & 0xffffu); }
     static __device__ __forceinline__ void st_nt(T *p, const float (&o)[4]) {
-        Raw r = {f_to_bf(o[0]) | (f_to_bf(o[1]) << 16), f_to_bf(o[2]) | (f_to_bf(o[3]) << 16)};
+        Raw r = {f2_to_bf2(o[0], o[1]), f2_to_bf2(o[2], o[3])};
         __builtin_nontemporal_store(r, reinterpret_cast<v2u *>(p));
     }
     // Tells the compiler nothing about the words' contents from here on, so that the widened copies made for the
