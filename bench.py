@@ -26,6 +26,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBS = 8000.0      # MI355X published HBM3E peak
+STREAM_LAUNCH_MS, STREAM_RATE_BYTES_PER_MS = 0.0035, 6.97e9      # measured: one streaming launch = 3.5 us + bytes / 6.97 TB/s
 
 # HBM-side bytes per dispatch of the dominant kernel at the default workload, from the two rocprofv3 --pmc
 # runs summarised in profiles/qwen3_sweep_pmc_fetch_write.md (FETCH_SIZE x 1.9992 + WRITE_SIZE x 0.9992, the
@@ -817,6 +818,9 @@ def main():
             if tb:
                 r["traffic_mb"] = tb / 1e6
                 r["traffic_frac"] = tb / r["ms"] / 1e6 / PEAK_HBM_GBS
+                # what one launch that only streams those bytes takes on this part (cold operands): the fit of a
+                # plain out = a*b kernel at 151 and 302 MB, 3.5 us + bytes / 6.97 TB/s
+                r["stream_model_ms"] = STREAM_LAUNCH_MS + tb / STREAM_RATE_BYTES_PER_MS
     out = {
         "metric": "layer-op tokens/s at %s shape (fused-op HBM GB/s and %% of peak in `ops`)" % (
             "Qwen3-0.6B" if cfg["name"] == "qwen3-0.6b" else "Stories110M"),
