@@ -18,7 +18,7 @@
 //      listed from the front of the block's task array, short ones from its back.
 //   3. col_sum_kernel<K>: per block, every thread writes its values of dx (fetched into registers while the previous
 //      block was summed) to LDS at their ranks, so that a run is a contiguous piece of an LDS column.  Waves 0..K-1
-//      take the long runs of one column each (128-bit LDS reads one group ahead of the adds); the other waves take the
+//      take the long runs of one column each (128-bit LDS reads issued sixteen adds ahead); the other waves take the
 //      short runs, K columns to a lane.  A long run's result also stays in LDS under its token, so the run of the
 //      same token in the next block starts from there and not from a load of dE: the chain of the most frequent
 //      token, which bounds the whole operation, goes on from block to block without a trip to memory.
