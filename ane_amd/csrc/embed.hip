@@ -851,7 +851,10 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     // enough that the small accesses to dE (one per token and workgroup) do not outweigh the copy.
     if (!g_ctx.scatter_tree && g_ctx.scatter_cols >= 0 && (S % 4 == 0 || N <= COL_SMALL) && V < (1 << (32 - CB_BITS))) {
         const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
-        if (g_ctx.scatter_cols > 0 || (N <= SMALL_N && (int)ceil_div((size_t)D, cols_per_workgroup(D)) <= cu))
+        // (also while a graph is recorded, for inputs whose row form would call the library sort, which cannot be)
+        const bool rows_recordable = N <= SMALL_N && key_bits(V) + POS_BITS <= 32;
+        if (g_ctx.scatter_cols > 0 || (N <= SMALL_N && (int)ceil_div((size_t)D, cols_per_workgroup(D)) <= cu) ||
+            (g_ctx.capturing && !rows_recordable))
             return scatter_add_cols(dE, dx, ids, V, D, S, N);
     }
     const int bits = key_bits(V);

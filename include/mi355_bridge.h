@@ -254,7 +254,8 @@ int mi355_embed_gather_dev(float *x, const float *E, const int32_t *ids, int V, 
  * bit-identical to the reference loop and run-to-run deterministic.  Ids outside [0,V) are skipped.
  * Two forms give the same bits: up to 16384 positions (S a multiple of 4, V < 2^19, D within one round of workgroups)
  * every workgroup owns a few columns of dE and reads its rows of dx in place; otherwise dx is first copied
- * token-major and summed row by row (the "scatter_cols" knob names a form). */
+ * token-major and summed row by row (the "scatter_cols" knob names a form).  While a graph is recorded, inputs beyond
+ * 16384 positions take the first form too (the library sort of the second cannot be recorded). */
 int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, int V, int D,
                                 int S, int batch);
 

@@ -130,6 +130,35 @@ def test_graph_capture_refuses_ops_that_allocate(br):
     L.mi355_graph_free(None)
 
 
+def test_graph_records_a_scatter_add_beyond_16384_positions(br):
+    """Eagerly such an input takes the library sort, which cannot be recorded; during a capture the entry point takes
+    the form with the columns of dE owned by workgroups instead: same bits, replayed three times."""
+    L = br.lib
+    V, D, B, S = 3000, 24, 80, 256                            # 20480 positions
+    ids = H.zipf_ids(5, B * S, V).astype(np.int32).reshape(B, S)
+    dx = H.normal(41, (B, D, S)); dE0 = H.normal(42, (V, D))
+    idd, dxd = br.DevArray.from_numpy(ids), br.DevArray.from_numpy(dx)
+    eager = br.DevArray.from_numpy(dE0)
+    br.check(L.mi355_embed_scatter_add_dev(eager.ptr, dxd.ptr, idd.ptr, V, D, S, B))     # also sizes the workspace
+    br.sync()
+    assert eager.numpy().tobytes() == O.embed_backward(dE0, dx, ids).tobytes()
+    rec = br.DevArray.from_numpy(dE0)
+    br.check(L.mi355_graph_begin())
+    br.check(L.mi355_embed_scatter_add_dev(rec.ptr, dxd.ptr, idd.ptr, V, D, S, B))
+    g = L.mi355_graph_end()
+    assert g
+    try:
+        want = dE0
+        for rep in range(3):
+            br.check(L.mi355_graph_launch(g))
+            want = O.embed_backward(want, dx, ids)
+            assert rec.numpy().tobytes() == want.tobytes(), rep
+            br.check(L.mi355_axpby_dev(eager.ptr, eager.ptr, None, 1.0, 64, 1))          # eager work between replays
+            br.sync()
+    finally:
+        L.mi355_graph_free(g)
+
+
 def test_graph_replays_the_one_launch_cross_entropy(br):
     """The cross-entropy kernel whose workgroups exchange partials inside the launch, recorded without a warm-up
     call (it allocates nothing: its slots and launch counters live in a device array of the library that is
