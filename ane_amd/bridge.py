@@ -51,6 +51,7 @@ SIGNATURES = {
     "mi355_sync": (_i, []),
     "mi355_workspace_reserve": (_i, [_z]),
     "mi355_tune_set": (_i, [C.c_char_p, _i]),
+    "mi355_exchange_stats": (_i, [C.POINTER(C.c_longlong), C.POINTER(C.c_longlong)]),
     "mi355_buf_alloc": (_p, [_z]),
     "mi355_buf_free": (None, [_p]),
     "mi355_buf_devptr": (_p, [_p]),
@@ -179,6 +180,13 @@ def device_info():
 def tune(key, value):
     if lib.mi355_tune_set(key.encode(), int(value)) != 0:
         raise BridgeError("unknown tuning knob %r" % key)
+
+
+def exchange_fallbacks():
+    """(shared exchange area, one-launch softmax-CE): workgroups whose bounded wait for a partner expired, ever."""
+    a, c = C.c_longlong(0), C.c_longlong(0)
+    check(lib.mi355_exchange_stats(C.byref(a), C.byref(c)), "mi355_exchange_stats")
+    return a.value, c.value
 
 
 class DevArray:

@@ -751,8 +751,9 @@ MI355_API int mi355_rmsnorm_bwd_bf16_dev(uint16_t *dx, float *dw, const uint16_t
     if (!dx || !dw || !dy || !x || !w) return mi355_fail("rmsnorm_bwd_bf16: NULL pointer");
     if (C <= 0 || S <= 0 || batch <= 0) return mi355_fail("rmsnorm_bwd_bf16: bad shape C=%d S=%d batch=%d", C, S, batch);
     if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd_bf16: variant must be 0 or 1");
+    if (dx == x) return mi355_fail("rmsnorm_bwd_bf16: dx must not alias x (dx may alias dy)");      // as the fp32 op
     const bool vec_ok = S % 8 == 0 && aligned16(x) && aligned16(dy) && aligned16(dx);
-    const ClusterPlan cp = (dx == dy || dx == x) ? NO_CLUSTER : plan_cluster_bf(C, S, batch, vec_ok);
+    const ClusterPlan cp = dx == dy ? NO_CLUSTER : plan_cluster_bf(C, S, batch, vec_ok);
     if (cp.csplit) {
         if (!mi355_exchange(&g_bf_cluster_ws)) return -1;
         const int nrows = cp.nblk / cp.csplit;

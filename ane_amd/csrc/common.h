@@ -33,7 +33,8 @@ struct Mi355Ctx {
     int rms_cluster;           // channel split of the clustered RMSNorm: 0 = per shape, -1 = never, 2/4/8 = forced
     int ce_resident;           // one-launch softmax-CE: 0 = where it pays, 1 = whenever the shape allows, -1 = never
     int rms_cluster_spin;      // its bounded wait in ticks of the 100 MHz clock: 0 = 2 ms, negative = do not wait at all
-                               // (-2: the one-launch cross-entropy also takes no partner's value, present or not: a test mode)
+    int xch_take_nothing;      // test mode of those kernels: 1 = no partner's value is taken, present or not, so every
+                               // workgroup goes the way of an expired wait
 };
 extern Mi355Ctx g_ctx;
 
@@ -58,8 +59,11 @@ struct Mi355Exchange {
     int *fallbacks;                // workgroups whose bounded wait expired, ever (diagnostic)
 };
 bool mi355_exchange(Mi355Exchange *out);
-// Ticks of the 100 MHz clock that such a kernel waits for a partner before it does the partner's work itself.
+// Ticks of the 100 MHz clock that such a kernel waits for a partner before it does the partner's work itself;
+// negative: the kernel does not even look at a partner's slot (the xch_take_nothing test mode).
 int mi355_exchange_spin_ticks(void);
+// Device address of the expired-wait counter of the one-launch cross-entropy (softmax_ce.hip), NULL before init.
+int *mi355_ce_fallbacks_dev(void);
 // Runs every queued weight-gradient reduction (dw_reduce.hip).
 extern "C" int mi355_dw_flush(void);
 

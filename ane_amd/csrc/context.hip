@@ -78,7 +78,23 @@ bool mi355_exchange(Mi355Exchange *out) {
 }
 
 int mi355_exchange_spin_ticks(void) {
+    if (g_ctx.xch_take_nothing > 0) return -1;
     return g_ctx.rms_cluster_spin == 0 ? 200000 : (g_ctx.rms_cluster_spin < 0 ? 0 : g_ctx.rms_cluster_spin);
+}
+
+// How many workgroups, since the library was loaded, gave up the bounded wait for a partner's value and computed it
+// themselves.  The results are the same to the bit either way, so this count is the only sign of a device on which
+// the cooperating workgroups are not resident together (each expiry costs the wait plus the recomputation).
+MI355_API int mi355_exchange_stats(long long *shared_area, long long *softmax_ce) {
+    if (!mi355_ready("exchange_stats")) return -1;
+    if (!mi355_outside_capture("exchange_stats")) return -1;
+    int a = 0, c = 0;
+    HIP_OK(hipStreamSynchronize(g_ctx.stream));
+    if (g_xch.fallbacks) HIP_OK(hipMemcpy(&a, g_xch.fallbacks, sizeof(int), hipMemcpyDeviceToHost));
+    if (int *p = mi355_ce_fallbacks_dev()) HIP_OK(hipMemcpy(&c, p, sizeof(int), hipMemcpyDeviceToHost));
+    if (shared_area) *shared_area = a;
+    if (softmax_ce) *softmax_ce = c;
+    return 0;
 }
 
 int mi355_ce_setup(void);        // softmax_ce.hip: locates its fixed scratch array on the current device
@@ -178,7 +194,7 @@ MI355_API int mi355_tune_set(const char *key, int value) {
         {"ce_rows", &g_ctx.ce_rows}, {"ce_rows2", &g_ctx.ce_rows2}, {"buf_phase", &g_ctx.buf_phase}, {"qk_lpr", &g_ctx.qk_lpr}, {"qk_threads", &g_ctx.qk_threads},
         {"gemm_splitk", &g_ctx.gemm_splitk}, {"scatter_tree", &g_ctx.scatter_tree}, {"scatter_cols", &g_ctx.scatter_cols},
         {"rms_cluster", &g_ctx.rms_cluster}, {"rms_cluster_spin", &g_ctx.rms_cluster_spin},
-        {"ce_resident", &g_ctx.ce_resident},
+        {"ce_resident", &g_ctx.ce_resident}, {"xch_take_nothing", &g_ctx.xch_take_nothing},
     };
     for (auto &t : tab)
         if (strcmp(t.k, key) == 0) { *t.v = value; return 0; }

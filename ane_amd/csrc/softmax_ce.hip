@@ -944,8 +944,8 @@ int ce_run(const char *who, T *dlogits, float *loss_dev, const T *logits, const 
                 xch.fallbacks = (int *)(base + CE_SCRATCH_BYTES + (size_t)CR_MAX_WG * CR_STRIDE * 8 + (size_t)CR_MAX_WG * 4);
                 hipLaunchKernelGGL((ce_resident_kernel<ST, true>), dim3((unsigned)(csplit * strips_r)), dim3(CR_THREADS), 0,
                                    g_ctx.stream, dlogits, logits, targets, V, S, strips_r, csplit, Rm, K, 1.0f / (float)S,
-                                   grad_scale, loss_dev, xch, mi355_exchange_spin_ticks(),
-                                   g_ctx.rms_cluster_spin <= -2 ? 1 : 0);
+                                   grad_scale, loss_dev, xch, mi355_exchange_spin_ticks() < 0 ? 0 : mi355_exchange_spin_ticks(),
+                                   g_ctx.xch_take_nothing > 0 ? 1 : 0);
                 LAUNCH_OK("softmax_ce (one launch)");
                 return 0;
             }
@@ -1038,6 +1038,11 @@ int mi355_ce_setup(void) {
     g_scratch_ptr[dev] = ptr;
     (void)grad_blocks_per_cu<float>();
     return 0;
+}
+
+int *mi355_ce_fallbacks_dev(void) {
+    unsigned char *base = (g_ctx.ready && g_ctx.device >= 0 && g_ctx.device < CE_MAX_DEVICES) ? g_scratch_ptr[g_ctx.device] : nullptr;
+    return base ? (int *)(base + CE_SCRATCH_BYTES + (size_t)CR_MAX_WG * CR_STRIDE * 8 + (size_t)CR_MAX_WG * 4) : nullptr;
 }
 
 // The same op with its scratch in the fixed device array: no hipMalloc, no hipFree, no workspace growth.

@@ -66,9 +66,21 @@ size_t mi355_workspace_size(void);
  * "rms_cluster" (channel split of the RMSNorm over cooperating workgroups: -1 = never, 2/4/8 = forced),
  * "ce_resident" (one-launch softmax-CE: 1 = for any V, -1 = never), "rms_cluster_spin" (how long a workgroup of those
  * kernels and of mi355_int8_scale_dev waits for a partner's partial result before it computes it itself, in ticks
- * of 10 ns: 0 = 2 ms; -1 = do not wait; -2 = -1, and the one-launch softmax-CE takes no partner's value at all:
- * both are for tests, the results are the same to the bit). */
+ * of 10 ns: 0 = 2 ms; -1 = do not wait), "xch_take_nothing" (1: those kernels take no partner's value at
+ * all, present or not, so every workgroup goes the way of an expired wait).  The last two settings are for tests: the
+ * results are the same to the bit. */
 int mi355_tune_set(const char *key, int value);
+
+/* How often, since the library was loaded, a workgroup of a kernel whose workgroups hand partial results to one
+ * another inside one launch gave up its bounded wait for a partner and computed the partner's part itself:
+ * *shared_area counts the clustered RMSNorm family and mi355_int8_scale_dev, *softmax_ce the one-launch
+ * softmax-CE (either pointer may be NULL).  No counterpart in the reference, whose ops are single loops
+ * (training/stories_cpu_ops.h:6-53, bridge/ane_bridge.m:346-353).  The results are identical to the bit whichever way
+ * a value was obtained, so these counts are the only sign that the cooperating workgroups do not run together (a GPU
+ * shared with other work): every expiry costs the wait ("rms_cluster_spin") plus the recomputation.  A caller that
+ * sees them grow can switch the cooperating forms off with mi355_tune_set("rms_cluster", -1) and ("ce_resident", -1).
+ * Waits for the stream and copies two words to the host: not possible during a graph capture.  0 / -1. */
+int mi355_exchange_stats(long long *shared_area, long long *softmax_ce);
 
 /* ------------------------------------------------------------------------------------------
  * Device buffers (opaque).  Replace the IOSurface-backed tensors behind

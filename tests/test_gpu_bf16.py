@@ -107,13 +107,22 @@ def test_rmsnorm_bf16_clustered_every_split_and_the_expired_wait(br, B, C, S):
             y, dx, dwv = got
             assert H.rel_err(O.cvt_bf16_f32(y), ry) <= TOL16, split
             assert H.rel_err(O.cvt_bf16_f32(dx), rdx) <= TOL16 and H.rel_err(dwv, rdw) <= 1e-5, split
+            expired = br.exchange_fallbacks()[0]
             again = run_all()
             assert all(a.tobytes() == b.tobytes() for a, b in zip(got, again)), split
+            assert br.exchange_fallbacks()[0] == expired, split         # every column sum came from the partners
             br.tune("rms_cluster_spin", -1)                              # the wait expires before it starts
             alone = run_all()
             assert all(a.tobytes() == b.tobytes() for a, b in zip(got, alone)), split
+            br.tune("rms_cluster_spin", 0); br.tune("xch_take_nothing", 1)
+            refused = run_all()                                          # every workgroup computes its partners' sums itself
+            assert all(a.tobytes() == b.tobytes() for a, b in zip(got, refused)), split
+            moved = br.exchange_fallbacks()[0] - expired
+            if (split == 0 and (B, C, S) == (16, 1024, 256)) or (split and -(-C // split) <= 256):
+                assert moved > 0, split      # (a member holds at most 256 rows; the library splits the named shape itself)
+            br.tune("xch_take_nothing", 0)
     finally:
-        br.tune("rms_cluster", 0); br.tune("rms_cluster_spin", 0)
+        br.tune("rms_cluster", 0); br.tune("rms_cluster_spin", 0); br.tune("xch_take_nothing", 0)
     br.tune("rms_cluster", -1)                                           # never clustered: the single-workgroup tiles
     try:
         y, dx, dwv = run_all()
@@ -147,25 +156,32 @@ def test_softmax_ce_bf16_one_launch_and_its_expired_wait(br, V, S):
         loss, dl = run()
         rl, rd = O.cross_entropy(logits, tgt)
         assert abs(float(loss[0]) - rl) <= 1e-5 * abs(rl) and H.rel_err(O.cvt_bf16_f32(dl), rd) <= TOL16
+        expired = br.exchange_fallbacks()[1]
         loss2, dl2 = run()
         assert loss.tobytes() == loss2.tobytes() and dl.tobytes() == dl2.tobytes()
-        for spin in ((-1, -2) if V <= 70000 else (-1,)):
-            br.tune("rms_cluster_spin", spin)
+        assert br.exchange_fallbacks()[1] == expired                     # every partial was handed over
+        for spin, refuse in ((-1, 0), (0, 1)):
+            br.tune("rms_cluster_spin", spin); br.tune("xch_take_nothing", refuse)
             loss3, dl3 = run()
-            assert loss.tobytes() == loss3.tobytes() and dl.tobytes() == dl3.tobytes(), spin
-        br.tune("rms_cluster_spin", 0)
+            assert loss.tobytes() == loss3.tobytes() and dl.tobytes() == dl3.tobytes(), (spin, refuse)
+        assert br.exchange_fallbacks()[1] > expired
+        br.tune("rms_cluster_spin", 0); br.tune("xch_take_nothing", 0)
         br.tune("ce_resident", -1)                                       # the three-launch form
         loss4, dl4 = run()
         assert abs(float(loss4[0]) - float(loss[0])) <= 2e-6 * abs(float(loss[0]))
         assert H.rel_err(O.cvt_bf16_f32(dl4), O.cvt_bf16_f32(dl)) <= TOL16
     finally:
-        br.tune("ce_resident", 0); br.tune("rms_cluster_spin", 0)
+        br.tune("ce_resident", 0); br.tune("rms_cluster_spin", 0); br.tune("xch_take_nothing", 0)
 
 
 def test_bf16_bad_arguments(br):
     a = br.DevArray(64, np.uint16); w = br.DevArray(8)
     assert br.lib.mi355_rmsnorm_fwd_bf16_dev(a.ptr, a.ptr, None, 8, 8, 1, 1e-5) == -1
     assert br.lib.mi355_rmsnorm_bwd_bf16_dev(a.ptr, w.ptr, a.ptr, a.ptr, w.ptr, 8, 8, 1, 1e-5, 2) == -1
+    a2, a3 = br.DevArray(64, np.uint16), br.DevArray(64, np.uint16)
+    assert br.lib.mi355_rmsnorm_bwd_bf16_dev(a.ptr, w.ptr, a2.ptr, a.ptr, w.ptr, 8, 8, 1, 1e-5, 0) == -1     # dx over x
+    assert "alias" in br.last_error()
+    assert br.lib.mi355_rmsnorm_bwd_bf16_dev(a2.ptr, w.ptr, a2.ptr, a3.ptr, w.ptr, 8, 8, 1, 1e-5, 0) == 0    # dx over dy
     assert br.lib.mi355_swiglu_fwd_bf16_dev(a.ptr, a.ptr, a.ptr, 0) == -1
     assert br.lib.mi355_axpby_bf16_dev(a.ptr, a.ptr, None, 1.0, 64, 0) == -1
     assert br.lib.mi355_cvt_f32_bf16_dev(a.ptr, 4, w.ptr, 8, 1, 8) == -1

@@ -27,6 +27,21 @@ def say(msg):
     print("[case] " + msg, flush=True)
 
 
+def rms_cluster_blocks(br, op, Cc, S, B):
+    """Workgroups that a norm entry point launches as clusters for this shape under the current knobs (op 0 = forward,
+    1 = backward, 2 = backward + residual); 0 when it runs the single-workgroup tile."""
+    t = (C.c_int * 5)()
+    br.check(br.lib.mi355_rmsnorm_tile(op, Cc, S, B, 1, t))
+    return t[4] * B * ((S + 63) // 64)
+
+
+def ce_one_launch_blocks(br, V, S):
+    """Workgroups of the one-launch softmax-CE for a shape that takes it (one per compute unit at most)."""
+    cus = br.device_info()[2]
+    strips = S // 64
+    return min(cus // strips, 64) * strips
+
+
 # ---------------------------------------------------------------------------------------------
 # RMSNorm
 # ---------------------------------------------------------------------------------------------
@@ -228,6 +243,11 @@ def test_rmsnorm_clustered_every_split_and_the_expired_wait(br, B, Cc, S):
     try:
         for split in (0, 2, 4, 8):
             br.tune("rms_cluster", split); br.tune("rms_cluster_spin", 0)
+            blocks = (2 * rms_cluster_blocks(br, 0, Cc, S, B) + rms_cluster_blocks(br, 1, Cc, S, B) +
+                      rms_cluster_blocks(br, 2, Cc, S, B))               # of the four launches of run_all
+            if split == 0 and (B, Cc, S) in ((16, 1024, 256), (1, 768, 256)):
+                assert blocks > 0                                        # the shapes the library clusters by itself
+            expired = br.exchange_fallbacks()[0]
             got = run_all()
             y, dx, dwv, dx3, dxs, dw3, y2, y2n = got
             assert H.err_elem(y, ry) <= TOL, split
@@ -238,11 +258,19 @@ def test_rmsnorm_clustered_every_split_and_the_expired_wait(br, B, Cc, S):
             assert np.array_equal(y2, r2) and H.err_elem(y2n, r2n) <= TOL, split
             again = run_all()                                            # run-to-run deterministic
             assert all(a.tobytes() == b.tobytes() for a, b in zip(got, again)), split
-            br.tune("rms_cluster_spin", -1)                              # the wait expires before it starts
-            alone = run_all()
+            # these two runs took every column sum from the partners: no workgroup's wait expired
+            assert br.exchange_fallbacks()[0] == expired, split
+            br.tune("rms_cluster_spin", -1)                              # the wait expires before it starts: a partner's
+            alone = run_all()                                            # value is taken only if it is already there
             assert all(a.tobytes() == b.tobytes() for a, b in zip(got, alone)), split
+            br.tune("rms_cluster_spin", 0); br.tune("xch_take_nothing", 1)
+            expired = br.exchange_fallbacks()[0]
+            refused = run_all()                                          # every workgroup computes its partners' sums itself
+            assert all(a.tobytes() == b.tobytes() for a, b in zip(got, refused)), split
+            assert br.exchange_fallbacks()[0] - expired == blocks, split
+            br.tune("xch_take_nothing", 0)
     finally:
-        br.tune("rms_cluster", 0); br.tune("rms_cluster_spin", 0)
+        br.tune("rms_cluster", 0); br.tune("rms_cluster_spin", 0); br.tune("xch_take_nothing", 0)
     br.tune("rms_cluster", -1)                                           # never clustered: the single-workgroup tiles
     try:
         y = run_all()[0]
@@ -663,14 +691,19 @@ def test_int8_scale_single_launch_and_its_expired_wait(br, n):
     x[n // 2] = np.float32(-123.25)
     xd = dev(br, x); sd = br.DevArray(1)
     try:
-        for spin in (0, -1):
-            br.tune("rms_cluster_spin", spin)
+        for spin, refuse in ((0, 0), (-1, 0), (0, 1)):
+            br.tune("rms_cluster_spin", spin); br.tune("xch_take_nothing", refuse)
             for off in (0, 1):                       # off = 1: the address is not 16-byte aligned (scalar path)
                 sd.upload(np.zeros(1, np.float32))
-                br.check(br.lib.mi355_int8_scale_dev(sd.ptr, xd.ptr + 4 * off, n))
-                assert sd.numpy()[0] == np.float32(O.int8_scale(x[off:off + n])), (spin, off)
+                expired = br.exchange_fallbacks()[0]
+                for _ in range(3):
+                    br.check(br.lib.mi355_int8_scale_dev(sd.ptr, xd.ptr + 4 * off, n))
+                assert sd.numpy()[0] == np.float32(O.int8_scale(x[off:off + n])), (spin, refuse, off)
+                # handed over in the normal run (no wait expired); workgroup 0 alone when it refuses the others' maxima
+                if spin == 0:
+                    assert br.exchange_fallbacks()[0] - expired == 3 * refuse, (refuse, off)
     finally:
-        br.tune("rms_cluster_spin", 0)
+        br.tune("rms_cluster_spin", 0); br.tune("xch_take_nothing", 0)
     z = dev(br, np.zeros(4096, np.float32))
     br.check(br.lib.mi355_int8_scale_dev(sd.ptr, z.ptr, 4096))
     assert sd.numpy()[0] == 1.0
@@ -777,23 +810,26 @@ def test_softmax_ce_one_launch_and_its_expired_wait(br, V, S):
             rl, rd = O.cross_entropy(logits, tgt, scale)
             assert abs(float(loss[0]) - rl) <= TOL * abs(rl) + 1e-12
             assert H.err_std(dl, rd) <= TOL
+        expired = br.exchange_fallbacks()[1]
         loss, dl = run(1.0)
         loss2, dl2 = run(1.0)
         assert loss.tobytes() == loss2.tobytes() and dl.tobytes() == dl2.tobytes()
+        assert br.exchange_fallbacks()[1] == expired                     # every partial was handed over: no wait expired
         br.tune("rms_cluster_spin", -1)                                  # the wait expires before it starts
         loss3, dl3 = run(1.0)
         assert loss.tobytes() == loss3.tobytes() and dl.tobytes() == dl3.tobytes()
-        if V <= 70000:
-            br.tune("rms_cluster_spin", -2)                              # and no partner's value is taken at all: every
-            loss5, dl5 = run(1.0)                                        # workgroup recomputes its whole strip, workgroup 0
-            assert loss.tobytes() == loss5.tobytes() and dl.tobytes() == dl5.tobytes()      # the other strips' loss terms
-        br.tune("rms_cluster_spin", 0)
+        br.tune("rms_cluster_spin", 0); br.tune("xch_take_nothing", 1)   # no partner's value is taken at all: every
+        expired = br.exchange_fallbacks()[1]                             # workgroup recomputes its whole strip, workgroup 0
+        loss5, dl5 = run(1.0)                                            # the other strips' loss terms
+        assert loss.tobytes() == loss5.tobytes() and dl.tobytes() == dl5.tobytes()
+        assert br.exchange_fallbacks()[1] - expired == ce_one_launch_blocks(br, V, S)
+        br.tune("xch_take_nothing", 0)
         br.tune("ce_resident", -1)                                       # the three-launch form
         loss4, dl4 = run(1.0)
         assert abs(float(loss4[0]) - float(loss[0])) <= 2e-6 * abs(float(loss[0]))
         assert H.err_std(dl4, dl) <= 2e-6
     finally:
-        br.tune("ce_resident", 0); br.tune("rms_cluster_spin", 0)
+        br.tune("ce_resident", 0); br.tune("rms_cluster_spin", 0); br.tune("xch_take_nothing", 0)
 
 
 # ---------------------------------------------------------------------------------------------

@@ -122,15 +122,17 @@ def test_softmax_ce_one_launch_random_shapes(br, V, S):
     try:
         br.tune("ce_resident", 1)
         out = []
-        for spin in (0, -2):
-            br.tune("rms_cluster_spin", spin)
+        for refuse in (0, 1):
+            br.tune("xch_take_nothing", refuse)
+            expired = br.exchange_fallbacks()[1]
             dl, lossd = br.DevArray(logits.shape), br.DevArray(1)
             br.check(br.lib.mi355_softmax_ce_dev(dl.ptr, lossd.ptr, ld.ptr, td.ptr, V, S, 1.0))
             out.append((lossd.numpy().tobytes(), dl.numpy().tobytes()))
             assert abs(float(lossd.numpy()[0]) - rl) <= TOL * max(abs(rl), 1e-3) and H.err_std(dl.numpy(), rd) <= TOL
+            assert (br.exchange_fallbacks()[1] > expired) == bool(refuse)
         assert out[0] == out[1]
     finally:
-        br.tune("ce_resident", 0); br.tune("rms_cluster_spin", 0)
+        br.tune("ce_resident", 0); br.tune("xch_take_nothing", 0)
 
 
 def _embed_cases():
