@@ -113,6 +113,8 @@ SIGNATURES = {
     "mi355_cvt_bf16_f32_dev": (_i, [_p, _z, _p, _z, _z, _z]),
     "mi355_rmsnorm_fwd_bf16_dev": (_i, [_p, _p, _p, _i, _i, _i, _f]),
     "mi355_rmsnorm_bwd_bf16_dev": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _f, _i]),
+    "mi355_residual_rmsnorm_fwd_bf16_dev": (_i, [_p, _p, _p, _p, _f, _p, _i, _i, _i, _f]),
+    "mi355_rmsnorm_bwd_residual_bf16_dev": (_i, [_p, _p, _p, _p, _p, _p, _p, _f, _i, _i, _i, _f, _i]),
     "mi355_swiglu_fwd_bf16_dev": (_i, [_p, _p, _p, _z]),
     "mi355_swiglu_bwd_bf16_dev": (_i, [_p, _p, _p, _p, _p, _z]),
     "mi355_axpby_bf16_dev": (_i, [_p, _p, _p, _f, _z, _i]),

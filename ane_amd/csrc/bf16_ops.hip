@@ -189,7 +189,8 @@ template <int VEC, int LPR, int THREADS, int CAP>
 __global__ __launch_bounds__(THREADS) void rms_bwd_bf16_kernel(bf16_t *dx, float *__restrict__ dw_part, const bf16_t *dy,
                                                                const bf16_t *__restrict__ x,
                                                                const float *__restrict__ w, int C, int S, int strips,
-                                                               int nblk, float eps, float invC, int variant) {
+                                                               int nblk, float eps, float invC, int variant,
+                                                               const bf16_t *res, bf16_t *dx2, float alpha2) {
     constexpr int RPS = THREADS / LPR;
     constexpr int NW = THREADS / 64;
     constexpr int G = LPR < 64 ? LPR : 64;
@@ -215,7 +216,23 @@ __global__ __launch_bounds__(THREADS) void rms_bwd_bf16_kernel(bf16_t *dx, float
             else o[j] = (dyr[j] * wc) * rr[j] - (xr[j] * dotn[j]) * rr[j];
             p += (dyr[j] * xr[j]) * rr[j];
         }
-        if (col_ok) stb<VEC>(dx + base + (size_t)c * S, o);
+        if (col_ok) {
+            // res != NULL: the backward residual rides along, dx = rmsnorm_bwd + res, and dx2 = alpha2 * dx if asked
+            // for (training/training_dynamic/train.m:586-595); res is read here, by the thread that then writes the
+            // same elements of dx, so dx may lie over res
+            if (res) {
+                float rv[VEC];
+                ldb<VEC, true>(rv, res + base + (size_t)c * S);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) o[j] = o[j] + rv[j];
+            }
+            stb<VEC>(dx + base + (size_t)c * S, o);
+            if (dx2) {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) o[j] = o[j] * alpha2;
+                stb<VEC>(dx2 + base + (size_t)c * S, o);
+            }
+        }
         p = group_sum<G>(p);
         if (lc == 0) part[c] = p;
     };
@@ -772,8 +789,82 @@ MI355_API int mi355_rmsnorm_bwd_bf16_dev(uint16_t *dx, float *dw, const uint16_t
     const int nblk = strips * batch;
     float *part = mi355_dw_partials((size_t)nblk * C, dw, nullptr);
     if (!part) return -1;
-    BF_DISPATCH(rms_bwd_bf16_kernel, cfg, nblk, dx, part, dy, x, w, C, S, strips, nblk, eps, 1.0f / (float)C, variant);
+    BF_DISPATCH(rms_bwd_bf16_kernel, cfg, nblk, dx, part, dy, x, w, C, S, strips, nblk, eps, 1.0f / (float)C, variant,
+                (const uint16_t *)nullptr, (uint16_t *)nullptr, 0.f);
     LAUNCH_OK("rmsnorm_bwd_bf16");
+    if (mi355_dw_submit(dw, part, nblk, C)) return -1;
+    return mi355_dw_op_end();
+}
+
+// The two fusions of the RMSNorm with the residual around it, for bfloat16 storage: the clustered kernels of
+// norm_cluster.h with the storage policy StoreBf16 where the shape clusters, otherwise the composition (forward) or
+// the single-workgroup tile with the residual riding along (backward).
+MI355_API int mi355_residual_rmsnorm_fwd_bf16_dev(uint16_t *y, uint16_t *yn, const uint16_t *a, const uint16_t *b,
+                                                  float alpha, const float *w, int C, int S, int batch, float eps) {
+    if (!mi355_ready("residual_rmsnorm_fwd_bf16")) return -1;
+    if (!y || !yn || !a || !b || !w) return mi355_fail("residual_rmsnorm_fwd_bf16: NULL pointer");
+    if (C <= 0 || S <= 0 || batch <= 0)
+        return mi355_fail("residual_rmsnorm_fwd_bf16: bad shape C=%d S=%d batch=%d", C, S, batch);
+    if (yn == y || yn == a || yn == b) return mi355_fail("residual_rmsnorm_fwd_bf16: yn must not alias y, a or b");
+    const bool vec_ok = S % 8 == 0 && aligned16(y) && aligned16(yn) && aligned16(a) && aligned16(b);
+    const ClusterPlan cp = (y == a || y == b) ? NO_CLUSTER : plan_cluster_bf(C, S, batch, vec_ok);
+    if (cp.csplit) {
+        if (!mi355_exchange(&g_bf_cluster_ws)) return -1;
+#define BF_CLUSTER_RES_FWD(RPT, EXACT)                                                                               \
+    hipLaunchKernelGGL((rms_fwd_cluster_kernel<StoreBf16, RPT, 1024, true, EXACT>), dim3(cp.nblk), dim3(1024), 0,    \
+                       g_ctx.stream, yn, y, a, b, alpha, w, C, S, cp.strips, cp.nblk, cp.csplit, cp.rows_pm, eps,    \
+                       1.0f / (float)C, g_bf_cluster_ws, mi355_exchange_spin_ticks())
+        if (cp.rpt == 2 && cp.exact) BF_CLUSTER_RES_FWD(2, true);
+        else if (cp.rpt == 2) BF_CLUSTER_RES_FWD(2, false);
+        else if (cp.exact) BF_CLUSTER_RES_FWD(4, true);
+        else BF_CLUSTER_RES_FWD(4, false);
+#undef BF_CLUSTER_RES_FWD
+        LAUNCH_OK("residual_rmsnorm_fwd_bf16");
+        return 0;
+    }
+    // two launches: y is rounded to bfloat16 either way and the norm is taken of the rounded values, as above
+    if (mi355_axpby_bf16_dev(y, a, b, alpha, (size_t)batch * C * S, 0)) return -1;
+    return mi355_rmsnorm_fwd_bf16_dev(yn, y, w, C, S, batch, eps);
+}
+
+MI355_API int mi355_rmsnorm_bwd_residual_bf16_dev(uint16_t *dx, uint16_t *dx_scaled, float *dw, const uint16_t *dy,
+                                                  const uint16_t *x, const float *w, const uint16_t *res, float alpha,
+                                                  int C, int S, int batch, float eps, int variant) {
+    if (!mi355_ready("rmsnorm_bwd_residual_bf16")) return -1;
+    if (!dx || !dw || !dy || !x || !w || !res) return mi355_fail("rmsnorm_bwd_residual_bf16: NULL pointer");
+    if (C <= 0 || S <= 0 || batch <= 0)
+        return mi355_fail("rmsnorm_bwd_residual_bf16: bad shape C=%d S=%d batch=%d", C, S, batch);
+    if (variant != 0 && variant != 1) return mi355_fail("rmsnorm_bwd_residual_bf16: variant must be 0 or 1");
+    if (dx_scaled && (dx_scaled == dx || dx_scaled == dy || dx_scaled == x || dx_scaled == res))
+        return mi355_fail("rmsnorm_bwd_residual_bf16: dx_scaled must not alias another operand");
+    if (dx == x) return mi355_fail("rmsnorm_bwd_residual_bf16: dx must not alias x (dx may alias res or dy)");
+    const bool vec_ok = S % 8 == 0 && aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(res) &&
+                        (!dx_scaled || aligned16(dx_scaled));
+    const ClusterPlan cp = dx == dy ? NO_CLUSTER : plan_cluster_bf(C, S, batch, vec_ok);
+    if (cp.csplit) {
+        if (!mi355_exchange(&g_bf_cluster_ws)) return -1;
+        const int nrows = cp.nblk / cp.csplit;
+        float *part = mi355_dw_partials((size_t)nrows * C, dw, nullptr);
+        if (!part) return -1;
+#define BF_CLUSTER_RES_BWD(RPT)                                                                                      \
+    hipLaunchKernelGGL((rms_bwd_cluster_kernel<StoreBf16, RPT, 1024, true, false>), dim3(cp.nblk), dim3(1024), 0,    \
+                       g_ctx.stream, dx, part, dy, x, w, C, S, cp.strips, cp.nblk, cp.csplit, cp.rows_pm, eps,       \
+                       1.0f / (float)C, variant, res, dx_scaled, alpha, g_bf_cluster_ws, mi355_exchange_spin_ticks())
+        if (cp.rpt == 2) BF_CLUSTER_RES_BWD(2);
+        else BF_CLUSTER_RES_BWD(4);
+#undef BF_CLUSTER_RES_BWD
+        LAUNCH_OK("rmsnorm_bwd_residual_bf16");
+        if (mi355_dw_submit(dw, part, nrows, C)) return -1;
+        return mi355_dw_op_end();
+    }
+    const BfCfg cfg = pick_bf(C, vec_ok, S, batch);
+    const int strips = (int)ceil_div((size_t)S, (size_t)cfg.lpr * cfg.vec);
+    const int nblk = strips * batch;
+    float *part = mi355_dw_partials((size_t)nblk * C, dw, nullptr);
+    if (!part) return -1;
+    BF_DISPATCH(rms_bwd_bf16_kernel, cfg, nblk, dx, part, dy, x, w, C, S, strips, nblk, eps, 1.0f / (float)C, variant, res,
+                dx_scaled, alpha);
+    LAUNCH_OK("rmsnorm_bwd_residual_bf16");
     if (mi355_dw_submit(dw, part, nblk, C)) return -1;
     return mi355_dw_op_end();
 }

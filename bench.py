@@ -90,7 +90,7 @@ class Bf16Lib:
     """Routes the ops that have a bfloat16-storage variant to it (mi355_X_dev -> mi355_X_bf16_dev)."""
     HAVE = {"mi355_rmsnorm_fwd_dev", "mi355_rmsnorm_bwd_dev", "mi355_swiglu_fwd_dev", "mi355_swiglu_bwd_dev",
             "mi355_axpby_dev", "mi355_rope_dev", "mi355_qknorm_rope_fwd_dev", "mi355_qknorm_rope_bwd_dev",
-            "mi355_softmax_ce_dev"}
+            "mi355_softmax_ce_dev", "mi355_residual_rmsnorm_fwd_dev", "mi355_rmsnorm_bwd_residual_dev"}
 
     # fp32 entry points that the sweep may still call in bf16 mode: they never see an activation buffer
     FP32_OK = {"mi355_dw_flush", "mi355_int8_scale_dev", "mi355_int8_quant_dev", "mi355_int8_dequant_dev"}
@@ -304,10 +304,7 @@ def per_op_table(br, wl, reps):
              "residual1": "residual", "res_rms1": "residual_rmsnorm_fwd", "rms_bwd_res": "rmsnorm_bwd_residual",
              "scale_copy": "scale_copy", "copy_c": "copy, bytes of rmsnorm_fwd"}
     table = []
-    if wl.bf16:
-        del names["res_rms1"]          # the fused residual + RMSNorm ops exist for fp32 storage only
-        del names["rms_bwd_res"]
-    elif wl.cfg["qk_norm"]:
+    if not wl.bf16 and wl.cfg["qk_norm"]:
         # the fused QK-norm + RoPE again as its unfused composition (three launches, priced at the fused op's bytes);
         # run last: it overwrites q_rot/k_rot with intermediates
         names["qk_unfused_fwd"] = "qknorm_rope_fwd (unfused: 3 launches)"
@@ -773,8 +770,6 @@ def main():
     if args.layers <= 0:
         args.layers = cfg["layers"]
     bf16 = args.storage == "bf16"
-    if bf16 and args.fuse:
-        raise SystemExit("bench.py: the fused residual + RMSNorm has no bf16-storage variant; drop --fuse")
     wl = Workload(br, cfg, args.layers, fuse=args.fuse, bf16=bf16, share=args.share_buffers)
     br.check(br.lib.mi355_dw_defer(0 if args.immediate_dw else 1))
 

@@ -110,6 +110,15 @@ int mi355_cvt_bf16_f32_dev(float *dst, size_t dst_ld, const uint16_t *src, size_
 int mi355_rmsnorm_fwd_bf16_dev(uint16_t *y, const uint16_t *x, const float *w, int C, int S, int batch, float eps);
 int mi355_rmsnorm_bwd_bf16_dev(uint16_t *dx, float *dw, const uint16_t *dy, const uint16_t *x, const float *w, int C,
                                int S, int batch, float eps, int variant);
+/* bf16-storage twins of mi355_residual_rmsnorm_fwd_dev and mi355_rmsnorm_bwd_residual_dev (the residual add and the
+ * RMSNorm after it, training/training_dynamic/train.m:460-461; the RMSNorm backward with the backward residual and the
+ * scaled copy, train.m:586-595, :714-721).  y, dx and dx_scaled are each rounded once, from fp32 values; yn is the norm
+ * of the rounded y.  Aliasing as for the fp32 entry points. */
+int mi355_residual_rmsnorm_fwd_bf16_dev(uint16_t *y, uint16_t *yn, const uint16_t *a, const uint16_t *b, float alpha,
+                                        const float *w, int C, int S, int batch, float eps);
+int mi355_rmsnorm_bwd_residual_bf16_dev(uint16_t *dx, uint16_t *dx_scaled, float *dw, const uint16_t *dy,
+                                        const uint16_t *x, const float *w, const uint16_t *res, float alpha, int C,
+                                        int S, int batch, float eps, int variant);
 int mi355_swiglu_fwd_bf16_dev(uint16_t *out, const uint16_t *h1, const uint16_t *h3, size_t n);
 int mi355_swiglu_bwd_bf16_dev(uint16_t *dh1, uint16_t *dh3, const uint16_t *dsilu, const uint16_t *h1,
                               const uint16_t *h3, size_t n);

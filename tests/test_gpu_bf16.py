@@ -82,6 +82,76 @@ def test_rmsnorm_bf16(br, B, C, S):
         assert H.rel_err(dwd.numpy(), rdw) <= 1e-5                      # fp32 in, fp32 sums, fp32 out
 
 
+@pytest.mark.parametrize("B,C,S", [(16, 1024, 256), (1, 768, 256), (2, 1000, 200), (3, 520, 136), (1, 2048, 8), (2, 100, 37),
+                                   (3, 48, 24), (2, 5000, 64), (40, 1024, 256)])
+def test_rmsnorm_residual_fusions_bf16(br, B, C, S):
+    """The residual add fused with the RMSNorm after it (training/training_dynamic/train.m:460-461) and the RMSNorm
+    backward with the backward residual and the scaled copy riding along (train.m:586-595), bf16 storage: within 5e-3
+    of the fp32 oracle run on the same bf16-representable inputs; y itself equals the rounded oracle sum to the bit;
+    the clustered kernels give the same bits whichever way their exchange goes; in place (y over a, dx over res, dx
+    over dy) the same values."""
+    print("[case] bf16 residual+rmsnorm fusions B=%d C=%d S=%d" % (B, C, S), flush=True)
+    (ab, a), (bb, b) = bf(H.normal(260, (B, C, S))), bf(H.normal(261, (B, C, S)))
+    (dyb, dy), (rb, res) = bf(H.normal(262, (B, C, S))), bf(H.normal(263, (B, C, S)))
+    w = H.normal(264, C, 1.0, 0.02); dw0 = H.normal(265, C)
+    alpha = np.float32(1 / np.sqrt(2 * 28))
+    ad, bd, dyd, rd, wd = (dev(br, v) for v in (ab, bb, dyb, rb, w))
+    ysum = O.axpby(a, b, alpha, 0)
+    yb_ref, y_ref = bf(ysum)                                             # the stored y: the fp32 sum rounded once
+    yn_ref = O.rmsnorm(y_ref, w)
+    rdx, rdw = O.rmsnorm_bwd(dy, a, w, dw=dw0)
+    dx_ref = O.axpby(rdx, res, 0.0, 2)
+    dxs_ref = O.axpby(dx_ref, None, alpha, 1)
+
+    def run_all(in_place=0):
+        y, yn = br.DevArray(a.shape, np.uint16), br.DevArray(a.shape, np.uint16)
+        dx, dxs = br.DevArray(a.shape, np.uint16), br.DevArray(a.shape, np.uint16)
+        dwd = dev(br, dw0)
+        a2 = dev(br, ab) if in_place else ad
+        r2 = dev(br, rb) if in_place == 1 else rd
+        g2 = dev(br, dyb) if in_place == 2 else dyd
+        yo = a2 if in_place else y
+        dxo = r2 if in_place == 1 else g2 if in_place == 2 else dx
+        br.check(br.lib.mi355_residual_rmsnorm_fwd_bf16_dev(yo.ptr, yn.ptr, a2.ptr, bd.ptr, alpha, wd.ptr, C, S, B, 1e-5))
+        br.check(br.lib.mi355_rmsnorm_bwd_residual_bf16_dev(dxo.ptr, dxs.ptr, dwd.ptr, g2.ptr, ad.ptr, wd.ptr, r2.ptr, alpha,
+                                                           C, S, B, 1e-5, 0))
+        return [v.numpy() for v in (yo, yn, dxo, dxs, dwd)]
+
+    def check(out, what):
+        y, yn, dx, dxs, dwv = out
+        assert np.array_equal(y, yb_ref), what
+        assert H.rel_err(O.cvt_bf16_f32(yn), yn_ref) <= TOL16, what
+        assert H.rel_err(O.cvt_bf16_f32(dx), dx_ref) <= TOL16 and H.rel_err(O.cvt_bf16_f32(dxs), dxs_ref) <= TOL16, what
+        assert H.rel_err(dwv, rdw) <= 1e-5, what
+
+    try:
+        got = run_all()
+        check(got, "out of place")
+        expired = br.exchange_fallbacks()[0]
+        again = run_all()
+        assert all(u.tobytes() == v.tobytes() for u, v in zip(got, again))
+        assert br.exchange_fallbacks()[0] == expired
+        br.tune("xch_take_nothing", 1)                                   # every workgroup computes its partners' sums itself
+        refused = run_all()
+        assert all(u.tobytes() == v.tobytes() for u, v in zip(got, refused))
+        if (B, C, S) == (16, 1024, 256):
+            assert br.exchange_fallbacks()[0] > expired                  # (the named shape runs clustered)
+        br.tune("xch_take_nothing", 0)
+        for mode in (1, 2):
+            check(run_all(mode), "in place %d" % mode)
+        dwd = dev(br, dw0); dx = br.DevArray(a.shape, np.uint16)         # no scaled copy asked for
+        br.check(br.lib.mi355_rmsnorm_bwd_residual_bf16_dev(dx.ptr, None, dwd.ptr, dyd.ptr, ad.ptr, wd.ptr, rd.ptr, alpha, C, S,
+                                                           B, 1e-5, 1))
+        rdx1, _ = O.rmsnorm_bwd(dy, a, w, variant=1, dw=dw0)
+        assert H.rel_err(back(dx), O.axpby(rdx1, res, 0.0, 2)) <= TOL16
+    finally:
+        br.tune("xch_take_nothing", 0)
+    assert br.lib.mi355_rmsnorm_bwd_residual_bf16_dev(ad.ptr, None, wd.ptr, dyd.ptr, ad.ptr, wd.ptr, rd.ptr, alpha, C, S, B,
+                                                      1e-5, 0) == -1      # dx over x
+    y = br.DevArray(a.shape, np.uint16)
+    assert br.lib.mi355_residual_rmsnorm_fwd_bf16_dev(y.ptr, y.ptr, ad.ptr, bd.ptr, alpha, wd.ptr, C, S, B, 1e-5) == -1
+
+
 @pytest.mark.parametrize("B,C,S", [(16, 1024, 256), (1, 768, 256), (2, 1000, 200), (3, 520, 136), (1, 2048, 8)])
 def test_rmsnorm_bf16_clustered_every_split_and_the_expired_wait(br, B, C, S):
     """The bf16-storage norm with the channel axis split over 2, 4 or 8 cooperating workgroups (and the library's own
