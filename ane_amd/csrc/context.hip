@@ -150,7 +150,9 @@ MI355_API int mi355_device_info(char *name, size_t name_len, double *peak_hbm_gb
     hipDeviceProp_t prop;
     HIP_OK(hipGetDeviceProperties(&prop, g_ctx.device));
     if (name && name_len) {
-        snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+        // (some driver stacks leave the marketing name empty: the architecture string then stands alone)
+        if (prop.name[0]) snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+        else snprintf(name, name_len, "%s", prop.gcnArchName);
     }
     if (peak_hbm_gbs) {
         // memoryClockRate is in kHz, bus width in bits; HBM transfers twice per clock.

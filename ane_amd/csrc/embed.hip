@@ -269,7 +269,7 @@ __global__ __launch_bounds__(1024) void rank_transpose_kernel(float *__restrict_
     const int n0 = blockIdx.x * TT;
     const int tq4 = t >> 8, ltq = t & 15, lr0 = (t & 255) >> 4;        // quarter; lane along positions; row group
     const int n4 = n0 + 4 * ltq;
-    const bool vec_ld = (S & 3) == 0 && n4 + 3 < N;
+    const bool vec_ld = (S & 3) == 0 && n4 + 3 < N && ((uintptr_t)dx & 15u) == 0;
     const int b4 = n4 / S, t4 = n4 - b4 * S;
     v4f pre0[4], pre1[4], pre2[4];
     {
@@ -458,7 +458,7 @@ __global__ __launch_bounds__(256) void transpose_sorted_kernel(float *__restrict
     const int d0 = blockIdx.y * TD;
     const int tid = threadIdx.x;
     if (tid < TT) dst_row[tid] = (t0 + tid < S) ? rank[(size_t)b * S + t0 + tid] : -1;
-    const bool s_vec = (S & 3) == 0;
+    const bool s_vec = (S & 3) == 0 && ((uintptr_t)dx & 15u) == 0;
     {   // lanes along t
         const int tq = tid & 15, r0 = tid >> 4;
         const int t = t0 + 4 * tq;
@@ -844,12 +844,14 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     if (V <= 0 || D <= 0 || S <= 0 || batch <= 0)
         return mi355_fail("embed_scatter_add: bad shape V=%d D=%d S=%d batch=%d", V, D, S, batch);
     if ((size_t)batch * S > (size_t)1 << 30) return mi355_fail("embed_scatter_add: more than 2^30 positions");
-    if (!aligned16(dx) || !aligned16(dE)) return mi355_fail("embed_scatter_add: pointers must be 16-byte aligned");
+    // (any 4-byte alignment of dx and dE: a dx that is not 16-byte aligned is read four bytes at a time by the row form,
+    // a dE that is not is read and written so)
     const int N = batch * S;
     // Two forms with the same bits (embed_cols.h says what each costs).  Columns of dE owned by workgroups: dx is
     // read where it lies, nothing is copied; chosen where one round of workgroups covers D and the positions are few
     // enough that the small accesses to dE (one per token and workgroup) do not outweigh the copy.
-    if (!g_ctx.scatter_tree && g_ctx.scatter_cols >= 0 && (S % 4 == 0 || N <= COL_SMALL) && V < (1 << (32 - CB_BITS))) {
+    if (!g_ctx.scatter_tree && g_ctx.scatter_cols >= 0 && ((S % 4 == 0 && aligned16(dx)) || N <= COL_SMALL) &&
+        V < (1 << (32 - CB_BITS))) {
         const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
         // (also while a graph is recorded, for inputs whose row form would call the library sort, which cannot be)
         const bool rows_recordable = N <= SMALL_N && key_bits(V) + POS_BITS <= 32;
@@ -863,7 +865,7 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
         !mi355_outside_capture("embed_scatter_add beyond 16384 positions or a vocabulary of 2^18 (its library sort may "
                                "record memset nodes)"))
         return -1;
-    const bool vec = (D % 4 == 0);          // rows and dE are 16-byte aligned, so every row start is too
+    const bool vec = (D % 4 == 0) && aligned16(dE);     // the token-major copy is 16-byte aligned: every row start is too
     const int nchunk = (int)ceil_div((size_t)D, vec ? 256 : 64), nchunk_long = (int)ceil_div((size_t)D, LCH);
     const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
     // Every workgroup of the segment-sum launch reserves 64 KiB of LDS, so two fit on a compute unit and the grid is

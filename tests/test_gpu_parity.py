@@ -608,6 +608,29 @@ def test_embed_scatter_add_tree_order_is_deterministic_and_close(br):
     assert not np.array_equal(outs[0][~short], ref[~short])           # the long ones are rounded differently
 
 
+@pytest.mark.parametrize("V,D,B,S", [(32000, 768, 8, 256), (500, 96, 3, 40), (1000, 64, 80, 256), (300, 7, 2, 256)])
+@pytest.mark.parametrize("off_dx,off_dE", [(1, 0), (0, 1), (3, 2)])
+def test_embed_scatter_add_unaligned_pointers(br, V, D, B, S, off_dx, off_dE):
+    """dx and dE at addresses that are multiples of 4 bytes only (the reference takes any float pointer): every form,
+    same bytes as the reference loop."""
+    say("scatter_add unaligned V=%d D=%d B=%d S=%d +%d/+%d floats" % (V, D, B, S, off_dx, off_dE))
+    _, ids = _embed_case(160, V, D, B, S, 1)
+    dx = H.normal(163, (B, D, S)); dE0 = H.normal(164, (V, D), 0, 0.5)
+    ref = O.embed_backward(dE0, dx, ids)
+    idd = dev(br, ids)
+    dxd = dev(br, np.concatenate([np.zeros(off_dx, np.float32), dx.ravel()]))
+    for form in (0, -1, 1):
+        br.tune("scatter_cols", form)
+        try:
+            dEd = dev(br, np.concatenate([np.full(off_dE, 7.0, np.float32), dE0.ravel(), np.full(4, 9.0, np.float32)]))
+            br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr + 4 * off_dE, dxd.ptr + 4 * off_dx, idd.ptr, V, D, S, B))
+        finally:
+            br.tune("scatter_cols", 0)
+        out = dEd.numpy()
+        assert out[off_dE:off_dE + V * D].tobytes() == ref.tobytes(), form
+        assert (out[:off_dE] == 7.0).all() and (out[off_dE + V * D:] == 9.0).all(), form      # nothing written outside
+
+
 def test_embed_scatter_add_no_valid_id(br):
     """Every id out of range: nothing is added (ids outside [0,V) are skipped, as the oracle's loop does)."""
     V, D, B, S = 100, 20, 2, 50
