@@ -70,6 +70,23 @@ void host_written(const void *p, size_t bytes) {
     }
 }
 
+// A drop-in has written the host range [p, p+bytes) and its device staging buffer `dev_src` holds the same bytes: a
+// resident table that contains the whole range takes them from there (a copy on the device, in stream order) and
+// stays current; one that only overlaps it is stale.  The embedding table that adam_update steps every iteration
+// (training/training_dynamic/train.m:869) is then not uploaded again by the vocab_compact_embed that follows (:871).
+void host_written_from(const void *p, const void *dev_src, size_t bytes) {
+    const char *lo = (const char *)p, *hi = lo + bytes;
+    for (int i = 0; i < g_tab_n; i++) {
+        const char *tlo = (const char *)g_tab[i].host;
+        const char *thi = tlo + (size_t)g_tab[i].V * g_tab[i].D * sizeof(float);
+        if (!(lo < thi && tlo < hi)) continue;
+        if (!g_tab[i].dirty && tlo <= lo && hi <= thi &&
+            hipMemcpyAsync((char *)g_tab[i].dev + (lo - tlo), dev_src, bytes, hipMemcpyDeviceToDevice, g_ctx.stream) == hipSuccess)
+            continue;
+        g_tab[i].dirty = true;
+    }
+}
+
 // The device copy of the host table `embed` [vocab][dim], uploaded if new or stale.  NULL on failure.
 Table *resident_table(const char *who, const float *embed, int vocab, int dim) {
     Table *tb = nullptr;
@@ -283,7 +300,7 @@ MI355_API void mi355_adam_update(float *w, const float *g, float *m, float *v, s
     if (!d2h(v, vd, nb)) return;
     memcpy(w, w2.data(), nb);
     memcpy(m, m2.data(), nb);
-    host_written(w, nb);      // a resident embedding table that lives in w is stale now
+    host_written_from(w, wd_, nb);      // a resident embedding table that lives in w follows on the device
 }
 
 // ---- vocabulary compaction on host arrays: training/training_dynamic/cpu_ops.h:96-148 ----

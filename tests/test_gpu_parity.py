@@ -1355,6 +1355,20 @@ def test_host_vocab_dropins_and_table_coherence(br):
     assert xo.tobytes() == O.embed_lookup(E, tok.astype(np.int32))[0][0].tobytes()      # not the rows of before
     br.lib.mi355_vocab_compact_embed(_p(ce), _p(E), _p(c2f), cv, V, D)
     assert ce.tobytes() == O.vocab_compact_embed(E, rc2f).tobytes()
+    # ... also a step on some rows only (the resident copy takes them on the device), and one on a range that runs
+    # past the table's end (the copy is uploaded again)
+    rows = slice(100, 1200)
+    n_sub = E[rows].size
+    br.lib.mi355_adam_update(_p(E[rows]), _p(g[rows]), _p(m[rows]), _p(v[rows]), n_sub, 2, 1e-2, 0.9, 0.95, 1e-8, 0.1)
+    br.lib.mi355_embed_lookup(_p(xo), _p(E), _p(tok), V, D, S)
+    assert xo.tobytes() == O.embed_lookup(E, tok.astype(np.int32))[0][0].tobytes()
+    big = np.concatenate([E.ravel(), np.zeros(D, np.float32)]); E2 = big[:V * D].reshape(V, D)
+    br.lib.mi355_embed_lookup(_p(xo), _p(E2), _p(tok), V, D, S)                         # a second resident table
+    tail = big[(V - 3) * D:]; zt = np.zeros_like(tail)
+    br.lib.mi355_adam_update(_p(tail), _p(np.ones_like(tail)), _p(zt), _p(zt.copy()), tail.size, 1, 1e-2, 0.9, 0.95, 1e-8, 0.0)
+    tok2 = np.full(S, V - 1, np.uint16)
+    br.lib.mi355_embed_lookup(_p(xo), _p(E2), _p(tok2), V, D, S)
+    assert xo.tobytes() == O.embed_lookup(E2, tok2.astype(np.int32))[0][0].tobytes()
     # update_full writes the host rows and keeps the resident copy current
     new = (ce * np.float32(0.5)).astype(np.float32); E_in = E.copy()
     br.lib.mi355_vocab_update_full(_p(E), _p(new), _p(c2f), cv, V, D)
