@@ -119,6 +119,7 @@ def test_graph_capture_refuses_ops_that_allocate(br):
     assert L.mi355_graph_begin() == -1
     assert L.mi355_embed_scatter_add_dev(dE.ptr, dx.ptr, ids.ptr, 1 << 20, 16, 8, 1) == -1    # library-sort path
     assert L.mi355_sgemm_dev(0, 0, 4, 4, 4, 1.0, a.ptr, 4, a.ptr, 4, 0.0, a.ptr, 4) == -1
+    assert L.mi355_exchange_stats(None, None) == -1                     # it waits for the stream and copies to the host
     assert "captured" in br.last_error()
     br.check(L.mi355_axpby_dev(a.ptr, a.ptr, None, 2.0, 64, 1))
     g = L.mi355_graph_end()
