@@ -77,7 +77,19 @@ bool mi355_exchange(Mi355Exchange *out) {
     return true;
 }
 
+// Watch over the cooperating kernels.  Their results do not depend on whether a partner's value arrived in time, so a
+// device on which they keep missing one another (shared with other work, workgroups not resident together) would only
+// show as launches that each take the bounded wait and then read their operands several times.  mi355_sync(), which
+// waits anyway, therefore looks at the two counters after such kernels have run: when they have grown at three checks
+// in a row-to-row unchanged configuration, the cooperating forms are switched off for the rest of the process (the
+// single-workgroup RMSNorm tiles, the two-launch INT8 scale, the three-launch cross-entropy take over) and one line
+// says so.  A change of a tuning knob starts the count afresh, and the test mode that refuses every value is not counted.
+static bool g_coop_launched = false, g_coop_rebase = true;
+static long long g_coop_seen = 0;
+static int g_coop_strikes = 0;
+
 int mi355_exchange_spin_ticks(void) {
+    g_coop_launched = true;
     if (g_ctx.xch_take_nothing > 0) return -1;
     return g_ctx.rms_cluster_spin == 0 ? 200000 : (g_ctx.rms_cluster_spin < 0 ? 0 : g_ctx.rms_cluster_spin);
 }
@@ -173,12 +185,37 @@ MI355_API int mi355_set_stream(void *hip_stream) {
     return 0;
 }
 
+static int coop_check(void) {
+    if (!g_coop_launched) return 0;
+    g_coop_launched = false;
+    int a = 0, c = 0;
+    if (g_xch.fallbacks) HIP_OK(hipMemcpy(&a, g_xch.fallbacks, sizeof(int), hipMemcpyDeviceToHost));
+    if (int *p = mi355_ce_fallbacks_dev()) HIP_OK(hipMemcpy(&c, p, sizeof(int), hipMemcpyDeviceToHost));
+    const long long total = (long long)a + c;
+    if (g_coop_rebase || g_ctx.xch_take_nothing > 0) {
+        g_coop_rebase = false;
+        g_coop_strikes = 0;
+    } else if (total > g_coop_seen) {
+        if (++g_coop_strikes >= 3 && (g_ctx.rms_cluster >= 0 || g_ctx.ce_resident >= 0)) {
+            g_ctx.rms_cluster = -1;
+            g_ctx.ce_resident = -1;
+            fprintf(stderr, "mi355_bridge: workgroups of the cooperating kernels keep giving up their wait for one another "
+                            "(%lld so far): is the GPU shared?  Switched to the non-cooperating forms "
+                            "(mi355_tune_set(\"rms_cluster\", 0) and (\"ce_resident\", 0) switch back)\n", total);
+        }
+    } else {
+        g_coop_strikes = 0;
+    }
+    g_coop_seen = total;
+    return 0;
+}
+
 MI355_API int mi355_sync(void) {
     if (!mi355_ready("sync")) return -1;
     if (!mi355_outside_capture("sync")) return -1;
     if (mi355_dw_flush()) return -1;
     HIP_OK(hipStreamSynchronize(g_ctx.stream));
-    return 0;
+    return coop_check();
 }
 
 MI355_API int mi355_workspace_reserve(size_t bytes) {
@@ -199,7 +236,7 @@ MI355_API int mi355_tune_set(const char *key, int value) {
         {"ce_resident", &g_ctx.ce_resident}, {"xch_take_nothing", &g_ctx.xch_take_nothing},
     };
     for (auto &t : tab)
-        if (strcmp(t.k, key) == 0) { *t.v = value; return 0; }
+        if (strcmp(t.k, key) == 0) { *t.v = value; g_coop_rebase = true; return 0; }
     return -1;
 }
 

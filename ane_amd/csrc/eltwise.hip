@@ -715,6 +715,18 @@ MI355_API int mi355_int8_scale_dev(float *scale_dev, const float *x, size_t n) {
     if (n == 0) return mi355_fail("int8_scale: empty tensor");
     const bool vec = aligned16(x);
     const size_t n4 = vec ? n / 4 : 0;
+    if (g_ctx.rms_cluster < 0) {
+        // the cooperating forms are switched off ("rms_cluster" = -1, by hand or by the watch in mi355_sync): per-workgroup
+        // maxima, then one workgroup folds them (the maximum is exact in any order: the same bits)
+        size_t nb = ceil_div(vec ? (n4 ? n4 : 1) : n, (size_t)EW_THREADS * 4);
+        if (nb > 1024) nb = 1024;
+        float *part = (float *)mi355_ws(nb * sizeof(float));
+        if (!part) return -1;
+        hipLaunchKernelGGL(absmax_kernel, dim3((unsigned)nb), dim3(EW_THREADS), 0, g_ctx.stream, part, x, n, n4, vec);
+        hipLaunchKernelGGL(scale_from_partials_kernel, dim3(1), dim3(1024), 0, g_ctx.stream, scale_dev, part, (int)nb);
+        LAUNCH_OK("int8_scale (two launches)");
+        return 0;
+    }
     // one workgroup of 1024 threads per compute unit, fewer for small tensors (at least 4 accesses per thread)
     const size_t per_block = (size_t)1024 * 4;
     size_t blocks = ceil_div(vec ? (n4 ? n4 : 1) : n, per_block);

@@ -63,7 +63,8 @@ size_t mi355_workspace_size(void);
  * of the gradient table and reads its rows of dx in place: 1 = for any number of positions, -1 = never),
  * "buf_phase" (where mi355_buf_alloc starts buffers of 1 MiB and more within a 1 KiB group:
  * 0 = a multiple of 128 bytes that rotates from one allocation to the next, 1..8 = always (value-1)*128),
- * "rms_cluster" (channel split of the RMSNorm over cooperating workgroups: -1 = never, 2/4/8 = forced),
+ * "rms_cluster" (channel split of the RMSNorm over cooperating workgroups: -1 = never, and mi355_int8_scale_dev then
+ * runs as two launches; 2/4/8 = forced),
  * "ce_resident" (one-launch softmax-CE: 1 = for any V, -1 = never), "rms_cluster_spin" (how long a workgroup of those
  * kernels and of mi355_int8_scale_dev waits for a partner's partial result before it computes it itself, in ticks
  * of 10 ns: 0 = 2 ms; -1 = do not wait), "xch_take_nothing" (1: those kernels take no partner's value at
@@ -78,7 +79,9 @@ int mi355_tune_set(const char *key, int value);
  * (training/stories_cpu_ops.h:6-53, bridge/ane_bridge.m:346-353).  The results are identical to the bit whichever way
  * a value was obtained, so these counts are the only sign that the cooperating workgroups do not run together (a GPU
  * shared with other work): every expiry costs the wait ("rms_cluster_spin") plus the recomputation.  A caller that
- * sees them grow can switch the cooperating forms off with mi355_tune_set("rms_cluster", -1) and ("ce_resident", -1).
+ * sees them grow can switch the cooperating forms off with mi355_tune_set("rms_cluster", -1) and ("ce_resident", -1);
+ * mi355_sync() does so by itself (one stderr line) when the counts have grown at three of its calls in a row with no
+ * knob changed in between, and setting the two knobs back to 0 switches the forms on again.
  * Waits for the stream and copies two words to the host: not possible during a graph capture.  0 / -1. */
 int mi355_exchange_stats(long long *shared_area, long long *softmax_ce);
 

@@ -732,6 +732,50 @@ def test_int8_scale_single_launch_and_its_expired_wait(br, n):
     assert sd.numpy()[0] == 1.0
 
 
+def test_cooperating_kernels_are_switched_off_after_repeated_expiries(br):
+    """A device on which the cooperating workgroups keep missing one another: forced here from the host with a wait of
+    one clock tick.  mi355_sync looks at the expired-wait counters; when they have grown at three syncs in a row the
+    library takes the non-cooperating forms by itself (same results), and setting the knobs back switches them on."""
+    B, Cc, S, V = 16, 1024, 256, 32000
+    x = H.normal(150, (B, Cc, S)); w = H.normal(151, Cc, 1.0, 0.02)
+    logits = H.normal(152, (V, S), 0, 2.0); tgt = np.random.default_rng(153).integers(0, V, S).astype(np.int32)
+    x8 = H.normal(154, 1024 * 4096)
+    xd, wd, ld, td, x8d = dev(br, x), dev(br, w), dev(br, logits), dev(br, tgt), dev(br, x8)
+    ry = O.rmsnorm(x, w); rl, rd = O.cross_entropy(logits, tgt); rs = np.float32(O.int8_scale(x8))
+    plan = (C.c_int * 5)()
+
+    def run():
+        y = br.DevArray(x.shape); dl = br.DevArray(logits.shape); lossd = br.DevArray(1); sd = br.DevArray(1)
+        br.check(br.lib.mi355_rmsnorm_fwd_dev(y.ptr, xd.ptr, wd.ptr, Cc, S, B, 1e-5))
+        br.check(br.lib.mi355_softmax_ce_dev(dl.ptr, lossd.ptr, ld.ptr, td.ptr, V, S, 1.0))
+        br.check(br.lib.mi355_int8_scale_dev(sd.ptr, x8d.ptr, x8.size))
+        br.sync()
+        assert H.err_elem(y.numpy(), ry) <= TOL and H.err_std(dl.numpy(), rd) <= TOL and sd.numpy()[0] == rs
+        assert abs(float(lossd.numpy()[0]) - rl) <= TOL * abs(rl)
+
+    try:
+        br.tune("rms_cluster_spin", 1)                # 10 ns: a value that is not there at the first look is given up
+        for i in range(4):                            # the first sync after a knob change only takes the counters' level
+            br.check(br.lib.mi355_rmsnorm_tile(0, Cc, S, B, 1, plan))
+            assert plan[4] > 0, i                     # still clustered
+            run()
+        br.check(br.lib.mi355_rmsnorm_tile(0, Cc, S, B, 1, plan))
+        assert plan[4] == 0                           # switched off by the library
+        before = br.exchange_fallbacks()
+        run()                                         # single-workgroup tiles, three-launch cross-entropy, two-launch scale
+        assert br.exchange_fallbacks() == before
+    finally:
+        br.tune("rms_cluster_spin", 0); br.tune("rms_cluster", 0); br.tune("ce_resident", 0)
+    br.check(br.lib.mi355_rmsnorm_tile(0, Cc, S, B, 1, plan))
+    assert plan[4] > 0
+    before = br.exchange_fallbacks()
+    for i in range(4):                                # the normal configuration: nothing expires, nothing is switched off
+        run()
+    assert br.exchange_fallbacks() == before
+    br.check(br.lib.mi355_rmsnorm_tile(0, Cc, S, B, 1, plan))
+    assert plan[4] > 0
+
+
 @pytest.mark.parametrize("n", [1024 * 4096, 2048 * 256 * 16, 13, 1, 4099])
 def test_minmax_exact(br, n):
     say("minmax n=%d" % n)
