@@ -532,6 +532,9 @@ __device__ __forceinline__ void cr_member_partial(const CrGeo<typename ST::T> &g
         }
 #pragma unroll
         for (int c = 0; c < K_REG / CR_SUB; c++) {
+            // (a member with fewer row steps than registers for them: the groups past its last step hold nothing,
+            // and folding nothing leaves (max, sum) as they are: skipped, for the exponentials' sake)
+            if (kR + c * CR_SUB >= g.K) continue;
             Raw t[CR_SUB];
 #pragma unroll
             for (int u = 0; u < CR_SUB; u++) t[u] = xr[c * CR_SUB + u];
