@@ -23,13 +23,23 @@ import glob
 import json
 import os
 import re
+import shlex
 import statistics
+import sys
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PROFILES = os.path.join(ROOT, "profiles")
 TRAFFIC_JSON = os.path.join(PROFILES, "traffic.json")
 COPY_KERNEL = "axpby_kernel<1, 1>"
 PRELUDE = "Command (run from the repo root on the MI355X box, after `cd /tmp && export TMPDIR=/tmp`):"
+
+
+def made_by():
+    """The line of a summary that says which command wrote it from the CSV files."""
+    if len(sys.argv) > 1 and sys.argv[1] in ("stats", "pmc"):
+        return "Written from the CSV files of that run by `python3 -m ane_amd.profile_summary %s`." % " ".join(
+            shlex.quote(a) for a in sys.argv[1:])
+    return "Written from the CSV files of that run by `ane_amd/profile_summary.py`."
 
 
 def short(name):
@@ -53,7 +63,7 @@ def find_csv(directory, suffix):
 
 def write_stats(directory, out_md, cmd, title, note):
     rows = list(csv.DictReader(open(find_csv(directory, "kernel_stats.csv"))))
-    lines = ["# rocprofv3 kernel-trace summary: " + title, "", PRELUDE, "", "    " + cmd, ""]
+    lines = ["# rocprofv3 kernel-trace summary: " + title, "", PRELUDE, "", "    " + cmd, "", made_by(), ""]
     if note:
         lines += [note, ""]
     lines += ["| kernel | calls | avg us | min us | max us | % of GPU time |", "|---|---:|---:|---:|---:|---:|"]
@@ -85,7 +95,7 @@ def write_pmc(fetch_dir, write_dir, out_md, key, cmd_fetch, cmd_write, known_kib
     wf = known_kib / max(w[COPY_KERNEL])          # the largest dispatch is the copy of known size
     lines = ["# rocprofv3 PMC: HBM-side traffic per dispatch (FETCH_SIZE, WRITE_SIZE)", "",
              "Two runs, one counter each (run from the repo root on the MI355X box, after `cd /tmp && export TMPDIR=/tmp`):",
-             "", "    " + cmd_fetch, "    " + cmd_write, "",
+             "", "    " + cmd_fetch, "    " + cmd_write, "", made_by(), "",
              "Calibration: `%s` (y = alpha*a over %s fp32) reads and writes exactly %.0f KiB;" % (COPY_KERNEL, shape, known_kib),
              "the counters report %.1f / %.1f KiB for it, so FETCH_SIZE is scaled by %.4f and WRITE_SIZE by %.4f." % (
                  max(f[COPY_KERNEL]), max(w[COPY_KERNEL]), ff, wf),
