@@ -626,12 +626,20 @@ struct RopeCache {
     float theta;
     float *cos_d, *sin_d;
 };
-static RopeCache g_rope[64];
-static int g_rope_n = 0;
+// Tables stay where they are until shutdown (callers keep the pointers), so the cache only grows: up to ROPE_MAX_TABLES
+// entries and ROPE_MAX_BYTES of device memory, far beyond what a training job asks for (one or two sequence lengths).
+constexpr int ROPE_MAX_TABLES = 1024;
+constexpr size_t ROPE_MAX_BYTES = (size_t)256 << 20;
+static RopeCache *g_rope = nullptr;
+static int g_rope_n = 0, g_rope_cap = 0;
+static size_t g_rope_bytes = 0;
 
 void mi355_free_rope_cache(void) {
     for (int i = 0; i < g_rope_n; i++) (void)hipFree(g_rope[i].cos_d);   // one allocation holds both
-    g_rope_n = 0;
+    free(g_rope);
+    g_rope = nullptr;
+    g_rope_n = g_rope_cap = 0;
+    g_rope_bytes = 0;
 }
 
 MI355_API int mi355_rope_tables_dev(const float **cos_dev, const float **sin_dev, int S, int hd, float theta) {
@@ -644,9 +652,18 @@ MI355_API int mi355_rope_tables_dev(const float **cos_dev, const float **sin_dev
             return 0;
         }
     if (!mi355_outside_capture("rope_tables_dev (first use of this S, head size and theta)")) return -1;
-    if (g_rope_n == 64) return mi355_fail("rope_tables_dev: table cache full (64 distinct (S,hd,theta))");
     if (S <= 0 || hd <= 0 || (hd & 1) || !(theta > 0.f)) return mi355_fail("rope_tables_dev: bad S/hd/theta");
     const size_t n = (size_t)(hd / 2) * S;
+    if (g_rope_n == ROPE_MAX_TABLES || g_rope_bytes + 2 * n * sizeof(float) > ROPE_MAX_BYTES)
+        return mi355_fail("rope_tables_dev: table cache full (%d tables, %zu MiB; the limits are %d and %zu MiB until shutdown)",
+                          g_rope_n, g_rope_bytes >> 20, ROPE_MAX_TABLES, ROPE_MAX_BYTES >> 20);
+    if (g_rope_n == g_rope_cap) {
+        const int cap = g_rope_cap ? 2 * g_rope_cap : 16;
+        RopeCache *grown = (RopeCache *)realloc(g_rope, (size_t)cap * sizeof(RopeCache));
+        if (!grown) return mi355_fail("rope_tables_dev: out of host memory");
+        g_rope = grown;
+        g_rope_cap = cap;
+    }
     float *host = (float *)malloc(2 * n * sizeof(float));
     if (!host) return mi355_fail("rope_tables_dev: out of host memory");
     mi355_rope_tables(host, host + n, S, hd, theta);
@@ -659,6 +676,7 @@ MI355_API int mi355_rope_tables_dev(const float **cos_dev, const float **sin_dev
         return mi355_fail("rope_tables_dev: %s", hipGetErrorString(e));
     }
     g_rope[g_rope_n++] = RopeCache{S, hd, theta, dev, dev + n};
+    g_rope_bytes += 2 * n * sizeof(float);
     *cos_dev = dev;
     *sin_dev = dev + n;
     return 0;

@@ -234,7 +234,8 @@ int mi355_swiglu_bwd_dev(float *dh1, float *dh3, const float *dsilu, const float
  * angle = p * (1/powf(theta, 2i/hd)) — the expression of training/training_dynamic/cpu_ops.h:172-175
  * (theta is 10000 there).  Host pointers. */
 int mi355_rope_tables(float *cos_host, float *sin_host, int S, int hd, float theta);
-/* The same tables resident on the device, cached per (S, hd, theta). */
+/* The same tables resident on the device, cached per (S, hd, theta).  The pointers stay valid until mi355_shutdown; the
+ * cache holds up to 1024 tables and 256 MiB and the call fails beyond that. */
 int mi355_rope_tables_dev(const float **cos_dev, const float **sin_dev, int S, int hd, float theta);
 
 /* RoPE on Q [batch][heads*hd][S] and K [batch][kv_heads*hd][S], interleaved row pairs (2i,2i+1).
