@@ -209,3 +209,126 @@ def test_embed_gather_scatter_random_shapes(br, case, kind, V, D, B, S, seed):
         chain = np.max(np.abs(ref - exact), axis=1)
         assert np.max((np.max(np.abs(got.astype(np.float64) - ref), axis=1) - chain) / scale) <= TOL
         assert np.array_equal(got[cnt <= 96], ref[cnt <= 96])          # short segments keep the reference order
+
+
+def _stream_cases():
+    """Lengths on both sides of the 128-bit path's tail and of one workgroup's share, with pointers 0-3 elements off a
+    16-byte boundary (the inputs and the outputs separately), for the element-wise and reduction kernels."""
+    rng = np.random.default_rng(901 + SEED)
+    out = []
+    for _ in range(12 * MORE):
+        n = int(rng.choice([rng.integers(1, 300), rng.integers(300, 70000), rng.integers(70000, 3_000_000)]))
+        out.append((n, int(rng.integers(0, 4)), int(rng.integers(0, 4)), int(rng.integers(1 << 30))))
+    return out
+
+
+class _Off:
+    """A device array of n elements that starts `off` elements into its allocation."""
+
+    def __init__(self, br, n, off, dtype=np.float32, data=None):
+        self.n, self.off, self.dtype = n, off, np.dtype(dtype)
+        host = np.zeros(n + off, dtype)
+        if data is not None:
+            host[off:] = data
+        self.d = br.DevArray.from_numpy(host)
+        self.ptr = self.d.ptr + off * self.dtype.itemsize
+
+    def numpy(self):
+        return self.d.numpy()[self.off:]
+
+
+@pytest.mark.parametrize("n,oi,oo,seed", _stream_cases())
+def test_streaming_ops_random_lengths_and_offsets(br, n, oi, oo, seed):
+    print("[case] streaming n=%d offsets in=%d out=%d seed=%d" % (n, oi, oo, seed), flush=True)
+    a = H.normal(seed, n); b = H.normal(seed + 1, n); d = H.normal(seed + 2, n)
+    ad, bd, dd = (_Off(br, n, oi, data=v) for v in (a, b, d))
+    o1, o2 = _Off(br, n, oo), _Off(br, n, oo)
+    # SwiGLU (within 1e-5 of the oracle; the gate's gradient against the tensor's scale, where its factor cancels)
+    br.check(br.lib.mi355_swiglu_fwd_dev(o1.ptr, ad.ptr, bd.ptr, n))
+    assert H.err_elem(o1.numpy(), O.swiglu_fwd(a, b)) <= TOL
+    br.check(br.lib.mi355_swiglu_bwd_dev(o1.ptr, o2.ptr, dd.ptr, ad.ptr, bd.ptr, n))
+    r1, r3 = O.swiglu_bwd(d, a, b)
+    assert H.rel_err(o1.numpy(), r1) <= TOL and H.err_elem(o2.numpy(), r3) <= TOL
+    # the residual family: bit for bit
+    al = np.float32(1 / np.sqrt(2 * 28))
+    for mode, second in ((0, bd), (1, None), (2, bd)):
+        br.check(br.lib.mi355_axpby_dev(o1.ptr, ad.ptr, second.ptr if second else None, al, n, mode))
+        assert np.array_equal(o1.numpy(), O.axpby(a, b if second else None, al, mode))
+    # INT8: scale, both roundings, dequantize, and the fused scale+quantize — bit for bit
+    x3 = a * np.float32(3.0)
+    xd = _Off(br, n, oi, data=x3)
+    sd, s2 = br.DevArray(1), br.DevArray(1)
+    br.check(br.lib.mi355_int8_scale_dev(sd.ptr, xd.ptr, n))
+    scale = sd.numpy()[0]
+    assert scale == np.float32(O.int8_scale(x3))
+    for rounding in (0, 1):
+        q, q2 = _Off(br, n, oo, np.int8), _Off(br, n, oo, np.int8)
+        br.check(br.lib.mi355_int8_quant_dev(q.ptr, xd.ptr, sd.ptr, n, rounding))
+        want = O.int8_quant(x3, scale, rounding)
+        assert np.array_equal(q.numpy(), want)
+        br.check(br.lib.mi355_int8_quantize_dynamic_dev(q2.ptr, s2.ptr, xd.ptr, n, rounding))
+        assert s2.numpy()[0] == scale and np.array_equal(q2.numpy(), want)
+        br.check(br.lib.mi355_int8_dequant_dev(o1.ptr, q.ptr, sd.ptr, n))
+        assert np.array_equal(o1.numpy(), O.int8_dequant(want, scale))
+    # range diagnostics: exact
+    mm = br.DevArray(3)
+    br.check(br.lib.mi355_minmax_dev(mm.ptr, xd.ptr, n))
+    assert mm.numpy().tobytes() == O.minmax(x3).tobytes()
+    # optimizer tail: sum of squares, then AdamW with the clip scale read on the device
+    w = H.normal(seed + 3, n, 0, 0.05); m = H.normal(seed + 4, n, 0, 0.01); v = np.abs(H.normal(seed + 5, n, 0, 0.01))
+    g = a * np.float32(40.0)
+    wd_, gd, md, vd = (_Off(br, n, o, data=t) for o, t in ((oo, w), (oi, g), (oo, m), (oi, v)))
+    ss = dev(br, np.zeros(1, np.float32)); cs = br.DevArray(1)
+    gsc = np.float32(1.0 / 256.0)
+    br.check(br.lib.mi355_sumsq_accum_dev(ss.ptr, gd.ptr, n, gsc))
+    t64 = float(np.sum((g * gsc).astype(np.float64) ** 2))
+    assert abs(ss.numpy()[0] - t64) <= TOL * t64
+    br.check(br.lib.mi355_clip_scale_dev(cs.ptr, ss.ptr, np.float32(1e-3)))
+    r_cs = O.clip_scale(float(ss.numpy()[0]), np.float32(1e-3))
+    assert cs.numpy()[0] == np.float32(r_cs)
+    br.check(br.lib.mi355_adam_update_dev(wd_.ptr, gd.ptr, md.ptr, vd.ptr, n, 3, 3e-4, 0.9, 0.95, 1e-8, 0.1, gsc, cs.ptr, 1))
+    rw, rm, rv = O.adam_update(w, (g * gsc) * np.float32(r_cs), m, v, 3, 3e-4, 0.9, 0.95, 1e-8, 0.1)
+    assert H.rel_err(md.numpy(), rm) <= TOL and H.rel_err(vd.numpy(), rv) <= TOL and H.rel_err(wd_.numpy(), rw) <= TOL
+    assert not gd.numpy().any()
+
+
+def _bf16_shapes():
+    rng = np.random.default_rng(333 + SEED)
+    out = []
+    for _ in range(6 * MORE):
+        C = int(rng.choice([rng.integers(1, 64), rng.integers(64, 600), rng.integers(600, 2200), rng.integers(2200, 5200)]))
+        S = int(rng.choice([rng.integers(1, 40), 8 * rng.integers(1, 40), 256]))
+        out.append((int(rng.integers(1, 5)), C, S))
+    return out
+
+
+@pytest.mark.parametrize("B,C,S", _bf16_shapes())
+def test_bf16_norms_random_shapes(br, B, C, S):
+    """The bfloat16-storage RMSNorm kernels and their residual fusions on random shapes: the checks of the named shapes
+    (within 5e-3 of the fp32 oracle on the same bf16-representable inputs, y and the exchange-free rerun to the bit)."""
+    import test_gpu_bf16 as BF
+    BF.test_rmsnorm_bf16(br, B, C, S)
+    BF.test_rmsnorm_residual_fusions_bf16(br, B, C, S)
+
+
+def _bf16_qk_shapes():
+    rng = np.random.default_rng(444 + SEED)
+    out = []
+    for _ in range(4 * MORE):
+        hd = int(rng.choice([16, 32, 64, 96, 128, 256]))
+        kvh = int(rng.integers(1, 4)); heads = kvh * int(rng.integers(1, 4))
+        S = int(rng.choice([8 * rng.integers(1, 40), rng.integers(1, 30)]))
+        out.append((int(rng.integers(1, 4)), heads, kvh, hd, S))
+    return out
+
+
+@pytest.mark.parametrize("B,heads,kvh,hd,S", _bf16_qk_shapes())
+def test_bf16_rope_random_shapes(br, B, heads, kvh, hd, S):
+    import test_gpu_bf16 as BF
+    BF.test_rope_and_qknorm_rope_bf16(br, B, heads, kvh, hd, S)
+
+
+@pytest.mark.parametrize("V,S", [(v, s) for v, s in _ce_shapes()[:4 * MORE]])
+def test_bf16_softmax_ce_random_shapes(br, V, S):
+    import test_gpu_bf16 as BF
+    BF.test_softmax_ce_bf16(br, V, S)
