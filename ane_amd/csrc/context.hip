@@ -81,9 +81,10 @@ bool mi355_exchange(Mi355Exchange *out) {
 // device on which they keep missing one another (shared with other work, workgroups not resident together) would only
 // show as launches that each take the bounded wait and then read their operands several times.  mi355_sync(), which
 // waits anyway, therefore looks at the two counters after such kernels have run: when they have grown at three checks
-// in a row-to-row unchanged configuration, the cooperating forms are switched off for the rest of the process (the
-// single-workgroup RMSNorm tiles, the two-launch INT8 scale, the three-launch cross-entropy take over) and one line
-// says so.  A change of a tuning knob starts the count afresh, and the test mode that refuses every value is not counted.
+// in a row with no tuning knob changed in between, the cooperating forms are switched off for the rest of the process
+// (the single-workgroup RMSNorm tiles, the two-launch INT8 scale, the three-launch cross-entropy take over) and one
+// line says so.  A change of a tuning knob starts the count afresh, and the test mode that refuses every value is not
+// counted.
 static bool g_coop_launched = false, g_coop_rebase = true;
 static long long g_coop_seen = 0;
 static int g_coop_strikes = 0;
@@ -151,6 +152,9 @@ MI355_API void mi355_shutdown(void) {
     mi355_graph_shutdown();
     if (g_xch.slots) (void)hipFree(g_xch.slots);
     g_xch = Mi355Exchange{nullptr, nullptr, nullptr};
+    g_coop_launched = false;                // (the shared area's counter starts from zero again after the next init)
+    g_coop_rebase = true;
+    g_coop_strikes = 0;
     if (g_ctx.ws) (void)hipFree(g_ctx.ws);
     g_ctx = Mi355Ctx{};
 }
