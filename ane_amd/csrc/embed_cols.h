@@ -19,7 +19,8 @@
 //   3. col_sum_kernel<K>: per block, every thread writes its values of dx (fetched into registers while the previous
 //      block was summed) to LDS at their ranks, so that a run is a contiguous piece of an LDS column.  Waves 0..K-1
 //      take the long runs of one column each (128-bit LDS reads issued sixteen adds ahead); the other waves take the
-//      short runs, K columns to a lane.  A long run's result also stays in LDS under its token, so the run of the
+//      short runs, K columns to a lane, the old sums of a lane's runs asked for before the block's values are put in
+//      their places.  A long run's result also stays in LDS under its token, so the run of the
 //      same token in the next block starts from there and not from a load of dE: the chain of the most frequent
 //      token, which bounds the whole operation, goes on from block to block without a trip to memory.
 #pragma once
@@ -207,28 +208,36 @@ __device__ __forceinline__ float long_chain(float acc, const float *xc, int star
 template <int K>
 struct __attribute__((packed, aligned(4))) ColVec { float f[K]; };
 
-template <int K>
+template <int K, bool FULL>                                     // FULL: D is a multiple of K, every workgroup has K columns
 __global__ __launch_bounds__(1024) void col_sum_kernel(float *dE, const float *__restrict__ dx,
                                                        const v2u *__restrict__ tasks,
                                                        const unsigned long long *__restrict__ cnt,
                                                        const uint16_t *__restrict__ rk, int N, int D, int S, int nblk) {
     constexpr int XP = CB + 48;                                 // a column in LDS, with room for the reads issued ahead
     constexpr int NSL = (16 - K) * 64;                          // lanes that take short runs
+    constexpr int RPL = 4;                                      // runs of a block whose old sums a lane asks for in one go
     __shared__ __attribute__((aligned(16))) float xs[K][XP];
     __shared__ unsigned long long carry[2][K][COL_CARRY];       // {token, bits of the sum} of the long runs of a block
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int d0 = xcd_remap(blockIdx.x, gridDim.x) * K;        // neighbouring columns on one XCD: they share lines of dE
-    const int kv = min(K, D - d0);                              // columns of this workgroup that exist
+    const int kv = FULL ? K : min(K, D - d0);                   // columns of this workgroup that exist
     const bool hot = wave < K;                                  // wave d < K: the long runs of column d0 + d
     const int sl = (wave - K) * 64 + lane;                      // the other lanes: short runs, all K columns each
 
-    // what a thread fetches ahead for a block: its positions' values of dx and ranks, the numbers of runs, and the
-    // first two runs it will take
-    v4f px[K][COL_PPT / 4];
-    unsigned prk[COL_PPT / 2];
-    unsigned long long pc;
-    v2u pd0, pd1;
-    auto fetch = [&](int blk) {
+    // What a thread fetches ahead for a block: its positions' values of dx and ranks, the numbers of runs, and the
+    // first runs it will take.
+    struct Pre {
+        v4f px[K][COL_PPT / 4];
+        unsigned prk[COL_PPT / 2];
+        unsigned long long pc;
+        v2u pd[RPL];
+    };
+    Pre o;
+    auto fetch = [&](Pre &o, int blk) __attribute__((always_inline)) {
+        const v2u *tb = tasks + (size_t)blk * CB;
+        o.pc = cnt[blk];
+#pragma unroll
+        for (int i = 0; i < RPL; i++) o.pd[i] = tb[hot ? lane + 64 * i : CB - 1 - (sl + NSL * i)];
         const int p0 = blk * CB + COL_PPT * t;
 #pragma unroll
         for (int q = 0; q < COL_PPT / 4; q++) {
@@ -236,113 +245,140 @@ __global__ __launch_bounds__(1024) void col_sum_kernel(float *dE, const float *_
             const int b = p / S, s = p - b * S;
 #pragma unroll
             for (int d = 0; d < K; d++)
-                px[d][q] = ld4_nt(dx + ((size_t)b * D + d0 + (d < kv ? d : 0)) * S + s);
+                o.px[d][q] = ld4_nt(dx + ((size_t)b * D + d0 + (d < kv ? d : 0)) * S + s);
         }
         const unsigned *rp = reinterpret_cast<const unsigned *>(rk + (size_t)blk * CB + COL_PPT * t);
 #pragma unroll
-        for (int q = 0; q < COL_PPT / 2; q++) prk[q] = rp[q];
-        pc = cnt[blk];
-        const v2u *tb = tasks + (size_t)blk * CB;
-        pd0 = tb[hot ? lane : CB - 1 - sl];
-        pd1 = tb[hot ? lane + 64 : CB - 1 - (sl + NSL)];
+        for (int q = 0; q < COL_PPT / 2; q++) o.prk[q] = rp[q];
     };
-    fetch(0);
+    float *dcol = dE + d0 + (hot ? wave : 0);
+    const float *xc = &xs[hot ? wave : 0][0];
+    const bool col_ok = wave < kv;
+
+    fetch(o, 0);
     for (int blk = 0; blk < nblk; blk++) {
-        const bool more = blk + 1 < nblk;
-        __syncthreads();                                        // the previous block's runs are summed and stored
+        const int n_long = (int)(o.pc & 0xffffffffu), n_short = (int)(o.pc >> 32);
+        const v2u *tb = tasks + (size_t)blk * CB;
+        v2u dsc_[RPL];
+#pragma unroll
+        for (int i = 0; i < RPL; i++) dsc_[i] = o.pd[i];
+        __syncthreads();                                    // the previous block's runs are summed and stored
+        // the old sums are asked for first: they travel while the block's values are put in their places
+        // (every wave issues the same loads, a row that is not needed read as row 0: the wait for the values of
+        // dx below then counts these loads exactly and does not include them)
+        float acc[RPL][K];
+        bool valid[RPL];
+        unsigned row[RPL];
+        bool hvalid = false, hcarried = false;
+        float hacc = 0.f;
+#pragma unroll
+        for (int i = 0; i < RPL; i++) {
+            valid[i] = !hot && sl + NSL * i < n_short;
+            row[i] = valid[i] ? dsc_[i].x : 0u;
+        }
+        if (hot) {
+            hvalid = col_ok && lane < n_long;
+            const unsigned tok = hvalid ? dsc_[0].x : 0u;
+            if (hvalid && blk > 0) {
+                const unsigned long long e = carry[(blk - 1) & 1][wave][tok & (COL_CARRY - 1)];
+                if ((unsigned)e == tok) {
+                    hacc = __uint_as_float((unsigned)(e >> 32));
+                    hcarried = true;
+                }
+            }
+            row[0] = hvalid && !hcarried ? tok : 0u;
+        }
+#pragma unroll
+        for (int i = 0; i < RPL; i++) {
+            const float *src = dE + (size_t)row[i] * D + d0;
+            if (FULL || kv == K) {                                  // one request for the K columns
+                const ColVec<K> v = *reinterpret_cast<const ColVec<K> *>(src);
+#pragma unroll
+                for (int d = 0; d < K; d++) acc[i][d] = v.f[d];
+            } else {
+#pragma unroll
+                for (int d = 0; d < K; d++) acc[i][d] = src[d < kv ? d : 0];
+            }
+        }
 #pragma unroll
         for (int q = 0; q < COL_PPT; q++) {
-            const int r = (prk[q / 2] >> (16 * (q & 1))) & 0xffff;
+            const int r = (o.prk[q / 2] >> (16 * (q & 1))) & 0xffff;
             if (blk * CB + COL_PPT * t + q < N) {
 #pragma unroll
-                for (int d = 0; d < K; d++) xs[d][r] = px[d][q / 4][q & 3];
+                for (int d = 0; d < K; d++) xs[d][r] = o.px[d][q / 4][q & 3];
             }
         }
         if (t < K * COL_CARRY) carry[blk & 1][t / COL_CARRY][t % COL_CARRY] = ~0ull;
-        const int n_long = (int)(pc & 0xffffffffu), n_short = (int)(pc >> 32);
-        const v2u *tb = tasks + (size_t)blk * CB;
-        const v2u d0_ = pd0, d1_ = pd1;
         __syncthreads();
+        if (blk + 1 < nblk) fetch(o, blk + 1);              // (behind the loads of the old sums: those arrive first)
         if (hot) {
             __builtin_amdgcn_s_setprio(3);
-            float *dcol = dE + d0 + wave;
-            const float *xc = &xs[wave][0];
-            const bool col_ok = wave < kv;
-            for (int r = 0; r * 64 < n_long; r++) {
+            if (hvalid) {
+                const unsigned tok = dsc_[0].x;
+                if (!hcarried) {
+#pragma unroll
+                    for (int d = 0; d < K; d++)
+                        if (d == wave) hacc = acc[0][d];
+                }
+                hacc = long_chain(hacc, xc, (int)(dsc_[0].y & 0xffffu), (int)(dsc_[0].y >> 16));
+                dcol[(size_t)tok * D] = hacc;
+                carry[blk & 1][wave][tok & (COL_CARRY - 1)] = ((unsigned long long)__float_as_uint(hacc) << 32) | tok;
+            }
+            for (int r = 1; r * 64 < n_long; r++) {          // more than 64 long runs in the block
                 const int a = lane + 64 * r;
-                const bool valid = col_ok && a < n_long;
-                v2u dsc = r == 0 ? d0_ : d1_;
-                if (r >= 2) dsc = tb[min(a, CB - 1)];
-                const unsigned tok = valid ? dsc.x : 0u;
-                const int start = (int)(dsc.y & 0xffffu), len = valid ? (int)(dsc.y >> 16) : 0;
-                float acc = 0.f;
-                bool need = valid;
-                if (valid && blk > 0) {
+                const bool val = col_ok && a < n_long;
+                const v2u dsc = tb[min(a, CB - 1)];
+                const unsigned tok = val ? dsc.x : 0u;
+                float ac = 0.f;
+                bool need = val;
+                if (val && blk > 0) {
                     const unsigned long long e = carry[(blk - 1) & 1][wave][tok & (COL_CARRY - 1)];
                     if ((unsigned)e == tok) {
-                        acc = __uint_as_float((unsigned)(e >> 32));
+                        ac = __uint_as_float((unsigned)(e >> 32));
                         need = false;
                     }
                 }
-                if (__builtin_amdgcn_ballot_w64(need)) {         // some run of this wave starts from dE itself
-                    float v = 0.f;
-                    if (need) v = dcol[(size_t)tok * D];
-                    acc = need ? v : acc;
-                }
-                if (r == 0 && more) fetch(blk + 1);
-                if (valid) {
-                    acc = long_chain(acc, xc, start, len);
-                    dcol[(size_t)tok * D] = acc;
-                    carry[blk & 1][wave][tok & (COL_CARRY - 1)] =
-                        ((unsigned long long)__float_as_uint(acc) << 32) | tok;
+                if (need) ac = dcol[(size_t)tok * D];
+                if (val) {
+                    ac = long_chain(ac, xc, (int)(dsc.y & 0xffffu), (int)(dsc.y >> 16));
+                    dcol[(size_t)tok * D] = ac;
+                    carry[blk & 1][wave][tok & (COL_CARRY - 1)] = ((unsigned long long)__float_as_uint(ac) << 32) | tok;
                 }
             }
-            if (n_long == 0 && more) fetch(blk + 1);
             __builtin_amdgcn_s_setprio(0);
         } else {
-            for (int r0 = 0; r0 * NSL < n_short; r0 += 2) {
-                v2u dsc[2] = {d0_, d1_};
-                float acc[2][K];
-                bool valid[2];
-#pragma unroll
-                for (int i = 0; i < 2; i++) {
-                    const int s = sl + (r0 + i) * NSL;
-                    valid[i] = s < n_short;
-                    if (r0 > 0) dsc[i] = tb[CB - 1 - min(s, CB - 1)];
-                                        const float *src = dE + (size_t)(valid[i] ? dsc[i].x : 0u) * D + d0;
-                    if (kv == K) {                              // one request for the K columns
-                        const ColVec<K> v = *reinterpret_cast<const ColVec<K> *>(src);
-#pragma unroll
-                        for (int d = 0; d < K; d++) acc[i][d] = v.f[d];
-                    } else {
-#pragma unroll
-                        for (int d = 0; d < K; d++) acc[i][d] = src[d < kv ? d : 0];
-                    }
-                }
-                if (r0 == 0 && more) fetch(blk + 1);
-#pragma unroll
-                for (int i = 0; i < 2; i++) {
-                    if (!valid[i]) continue;
-                    const int start = (int)(dsc[i].y & 0xffffu), len = (int)(dsc[i].y >> 16);
+            auto finish = [&](const v2u dsc, float (&ac)[K]) {
+                const int start = (int)(dsc.y & 0xffffu), len = (int)(dsc.y >> 16);
 #pragma unroll 4
-                    for (int j = 0; j < len; j++) {
+                for (int jj = 0; jj < len; jj++) {
 #pragma unroll
-                        for (int d = 0; d < K; d++) acc[i][d] += xs[d][start + j];
-                    }
-                    float *dst = dE + (size_t)dsc[i].x * D + d0;
-                    if (kv == K) {
-                        ColVec<K> v;
-#pragma unroll
-                        for (int d = 0; d < K; d++) v.f[d] = acc[i][d];
-                        *reinterpret_cast<ColVec<K> *>(dst) = v;
-                    } else {
-#pragma unroll
-                        for (int d = 0; d < K; d++)
-                            if (d < kv) dst[d] = acc[i][d];
-                    }
+                    for (int d = 0; d < K; d++) ac[d] += xs[d][start + jj];
                 }
+                float *dst = dE + (size_t)dsc.x * D + d0;
+                if (FULL || kv == K) {
+                    ColVec<K> v;
+#pragma unroll
+                    for (int d = 0; d < K; d++) v.f[d] = ac[d];
+                    *reinterpret_cast<ColVec<K> *>(dst) = v;
+                } else {
+#pragma unroll
+                    for (int d = 0; d < K; d++)
+                        if (d < kv) dst[d] = ac[d];
+                }
+            };
+#pragma unroll
+            for (int i = 0; i < RPL; i++)
+                if (valid[i]) finish(dsc_[i], acc[i]);
+            for (int r0 = RPL; r0 * NSL < n_short; r0++) {   // more short runs than RPL per lane: one at a time
+                const int s = sl + r0 * NSL;
+                if (s >= n_short) continue;
+                const v2u dsc = tb[CB - 1 - s];
+                const float *src = dE + (size_t)dsc.x * D + d0;
+                float ac[K];
+#pragma unroll
+                for (int d = 0; d < K; d++) ac[d] = src[d < kv ? d : 0];
+                finish(dsc, ac);
             }
-            if (n_short == 0 && more) fetch(blk + 1);
         }
     }
 }
@@ -475,7 +511,12 @@ int scatter_add_cols(float *dE, const float *dx, const int32_t *ids, int V, int 
     LAUNCH_OK("embed_scatter_add plan");
 #define COL_LAUNCH(KK)                                                                                              \
     case KK:                                                                                                        \
-        hipLaunchKernelGGL(col_sum_kernel<KK>, grid, dim3(1024), 0, g_ctx.stream, dE, dx, tasks, cnt, rk, N, D, S, nblk); \
+        if (D % KK == 0)                                                                                            \
+            hipLaunchKernelGGL((col_sum_kernel<KK, true>), grid, dim3(1024), 0, g_ctx.stream, dE, dx, tasks, cnt, rk, N, D, \
+                               S, nblk);                                                                            \
+        else                                                                                                        \
+            hipLaunchKernelGGL((col_sum_kernel<KK, false>), grid, dim3(1024), 0, g_ctx.stream, dE, dx, tasks, cnt, rk, N, D, \
+                               S, nblk);                                                                            \
         break;
     switch (K) {
         COL_LAUNCH(1) COL_LAUNCH(2) COL_LAUNCH(3)
