@@ -53,7 +53,7 @@ OP_KERNELS = {
 # BASELINE.json config 2: the three launches of the ordered scatter-add in its column form and in its row form, and
 # the gather
 EMBED_KERNELS = {
-    "scatter_cols": [("chunk_sort_blk_kernel", 1.0), ("block_rank_kernel", 1.0), ("col_sum_kernel<3>", 1.0)],
+    "scatter_cols": [("chunk_sort_blk_kernel", 1.0), ("block_rank_kernel", 1.0), ("col_sum_kernel<3, true>", 1.0)],
     "scatter_rows": [("chunk_sort_kernel", 1.0), ("rank_transpose_kernel", 1.0), ("seg_sum_kernel<false>", 1.0)],
     "gather": [("gather_kernel<true>", 1.0)],
 }
