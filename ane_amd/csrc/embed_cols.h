@@ -233,11 +233,13 @@ __global__ __launch_bounds__(1024) void col_sum_kernel(float *dE, const float *_
         v2u pd[RPL];
     };
     Pre o;
-    auto fetch = [&](Pre &o, int blk) __attribute__((always_inline)) {
+    auto fetch_runs = [&](Pre &o, int blk) __attribute__((always_inline)) {
         const v2u *tb = tasks + (size_t)blk * CB;
         o.pc = cnt[blk];
 #pragma unroll
         for (int i = 0; i < RPL; i++) o.pd[i] = tb[hot ? lane + 64 * i : CB - 1 - (sl + NSL * i)];
+    };
+    auto fetch_values = [&](Pre &o, int blk) __attribute__((always_inline)) {
         const int p0 = blk * CB + COL_PPT * t;
 #pragma unroll
         for (int q = 0; q < COL_PPT / 4; q++) {
@@ -255,7 +257,18 @@ __global__ __launch_bounds__(1024) void col_sum_kernel(float *dE, const float *_
     const float *xc = &xs[hot ? wave : 0][0];
     const bool col_ok = wave < kv;
 
-    fetch(o, 0);
+    // The long runs of the first block start from dE itself, and the chain of the most frequent token is what the
+    // launch waits for.  The waves that take them are the first of the workgroup to issue anything, so their piece of
+    // the run list is back within half a microsecond; they ask for their old sums then, ahead of every value of dx,
+    // and have them when the block is in its place (asked for with everybody else's, behind 25 MB of dx, they come
+    // 2.4 us after that for the median workgroup and 4.8 us for the slowest).
+    fetch_runs(o, 0);
+    float h0 = 0.f;
+    if (hot) {
+        const bool hv = col_ok && lane < (int)(o.pc & 0xffffffffu);
+        h0 = dcol[(size_t)(hv ? o.pd[0].x : 0u) * D];
+    }
+    fetch_values(o, 0);
     for (int blk = 0; blk < nblk; blk++) {
         const int n_long = (int)(o.pc & 0xffffffffu), n_short = (int)(o.pc >> 32);
         const v2u *tb = tasks + (size_t)blk * CB;
@@ -286,6 +299,10 @@ __global__ __launch_bounds__(1024) void col_sum_kernel(float *dE, const float *_
                     hcarried = true;
                 }
             }
+            if (blk == 0) {
+                hacc = h0;
+                hcarried = true;
+            }
             row[0] = hvalid && !hcarried ? tok : 0u;
         }
 #pragma unroll
@@ -310,7 +327,10 @@ __global__ __launch_bounds__(1024) void col_sum_kernel(float *dE, const float *_
         }
         if (t < K * COL_CARRY) carry[blk & 1][t / COL_CARRY][t % COL_CARRY] = ~0ull;
         __syncthreads();
-        if (blk + 1 < nblk) fetch(o, blk + 1);              // (behind the loads of the old sums: those arrive first)
+        if (blk + 1 < nblk) {                               // (behind the loads of the old sums: those arrive first)
+            fetch_runs(o, blk + 1);
+            fetch_values(o, blk + 1);
+        }
         if (hot) {
             __builtin_amdgcn_s_setprio(3);
             if (hvalid) {
