@@ -81,6 +81,7 @@ SIGNATURES = {
     "mi355_axpby_dev": (_i, [_p, _p, _p, _f, _z, _i]),
     "mi355_embed_gather_dev": (_i, [_p, _p, _p, _i, _i, _i, _i]),
     "mi355_embed_scatter_add_dev": (_i, [_p, _p, _p, _i, _i, _i, _i]),
+    "mi355_embed_scatter_add_form": (_i, [_i, _i, _i, _i, _i]),
     "mi355_softmax_ce_dev": (_i, [_p, _p, _p, _p, _i, _i, _f]),
     "mi355_minmax_dev": (_i, [_p, _p, _z]),
     "mi355_int8_scale_dev": (_i, [_p, _p, _z]),

@@ -219,6 +219,13 @@ __global__ __launch_bounds__(PLAN_T) void plan_write_kernel(int *__restrict__ se
 //      the rows just found (the transpose of the large path, fused in: the slab's loads are issued before the
 //      searches and land meanwhile).
 constexpr int SMALL_N = 16384, POS_BITS = 14, CHUNK = 256, CHUNK_PITCH = CHUNK + 1;
+
+// The word the last kernel of a scatter-add leaves for the host: how many runs (form 1, columns: (token, block)
+// pairs; form 2, rows: distinct tokens) the input of N positions and row width D had.
+__host__ __device__ inline unsigned long long scatter_report(int runs, int N, int D, int form) {
+    return ((unsigned long long)(unsigned)form << 60) | ((unsigned long long)((unsigned)D & 0xfffffu) << 40) |
+           ((unsigned long long)((unsigned)N & 0xfffffu) << 20) | ((unsigned)runs & 0xfffffu);
+}
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ unsigned pack_word(const int32_t *__restrict__ ids, int i, int N, int V) {
@@ -520,7 +527,8 @@ __global__ __launch_bounds__(1024, 8) void seg_sum_kernel(float *__restrict__ dE
                                                        const v4i *__restrict__ seg_list,
                                                        const int *__restrict__ meta, const v4i *__restrict__ long_list,
                                                        int D, int nchunk, int nchunk_long,
-                                                       int long_x, int short_blocks, bool vec) {
+                                                       int long_x, int short_blocks, bool vec,
+                                                       unsigned long long *report, int N) {
     __shared__ float stage[2][STAGE_ROWS][LCH];
     __shared__ v4i ent[MAX_ORDERED];
     __shared__ short order[MAX_ORDERED];
@@ -528,6 +536,8 @@ __global__ __launch_bounds__(1024, 8) void seg_sum_kernel(float *__restrict__ dE
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nseg = meta[0];
     const int long_blocks = long_x * nchunk_long;
+    // what the host looks at before it picks a form for the next call of this shape (one 8-byte store to host memory)
+    if (report && blockIdx.x == 0 && threadIdx.x == 0) *report = scatter_report(nseg, N, D, 2);
     if ((int)blockIdx.x < long_blocks) {
         const int ch = blockIdx.x % nchunk_long, x0 = blockIdx.x / nchunk_long;
         const int col = lane & (LCH - 1), sub = lane / LCH;      // a load instruction covers rows r and r+1
@@ -837,6 +847,78 @@ MI355_API int mi355_embed_gather_dev(float *x, const float *E, const int32_t *id
     return 0;
 }
 
+// Which form takes an input of N positions and row width D.  Both forms give the same bits, so the choice is only a
+// matter of time, and what decides it is how the ids repeat: the column form pays one small access to dE per
+// (token, block of 8192 positions) and workgroup, the row form a token-major copy of dx whatever the ids are.  Ids of
+// text repeat (config 2: 4621 pairs in 16384 positions) and the column form is the default; for ids that hardly
+// repeat (drawn uniformly from a large vocabulary) it is up to twice as slow.  The ids are on the device, so the
+// library learns from the previous call: the last kernel of either form leaves its number of runs in a word of
+// pinned host memory, and the next call of the same N and D compares it with the number at which the two forms
+// cost the same (fitted to measurements: column form 10 + 2.5 per block + 4.9 ns per pair, row form
+// 24 + 1.4e-6 N D, in us).  The row form reports distinct tokens, not pairs; how many pairs a token makes is taken
+// from the last time both forms saw this shape (1.2, config 2's figure, until then), so that a steady input settles
+// on one form instead of alternating.
+namespace {
+unsigned long long *g_report = nullptr;        // pinned, written by the device
+unsigned long long *g_report_dev = nullptr;
+int g_cols_runs = 0, g_cols_N = 0, g_cols_D = 0;   // the column form's last report
+double g_pairs_per_token = 1.2;
+
+unsigned long long *scatter_report_word(void) {
+    if (!g_report && !g_ctx.capturing) {
+        void *h = nullptr, *d = nullptr;
+        if (hipHostMalloc(&h, 64, hipHostMallocMapped) == hipSuccess && hipHostGetDevicePointer(&d, h, 0) == hipSuccess) {
+            g_report = (unsigned long long *)h;
+            g_report_dev = (unsigned long long *)d;
+            *(volatile unsigned long long *)g_report = 0ull;
+        } else {
+            if (h) (void)hipHostFree(h);
+            (void)hipGetLastError();
+        }
+    }
+    return g_report_dev;
+}
+
+// 1: columns of dE owned by workgroups, -1: token-major copy and row sums.  `cols_ok`: the column form can take the call.
+int scatter_form(int N, int D, bool cols_ok, bool rows_recordable) {
+    if (!cols_ok) return -1;
+    if (g_ctx.scatter_cols > 0) return 1;
+    if (g_ctx.capturing && !rows_recordable) return 1;
+    const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
+    if (N > SMALL_N || (int)ceil_div((size_t)D, cols_per_workgroup(D)) > cu) return -1;
+    if (N <= COL_SMALL || !g_report) return 1;
+    const unsigned long long w = *(volatile unsigned long long *)g_report;
+    const int form = (int)(w >> 60), rD = (int)((w >> 40) & 0xfffffu), rN = (int)((w >> 20) & 0xfffffu);
+    const int runs = (int)(w & 0xfffffu);
+    if (form == 0 || rN != N || rD != D) return 1;
+    const int nblk = (int)ceil_div((size_t)N, CB);
+    const double even = std::max((14.0 - 2.5 * nblk + 1.4e-6 * (double)N * D) / 4.9e-3, 0.30 * N);
+    if (form == 1) {
+        g_cols_runs = runs; g_cols_N = N; g_cols_D = D;
+        return runs <= 1.08 * even ? 1 : -1;
+    }
+    if (g_cols_N == N && g_cols_D == D && runs > 0) {       // both forms have seen this shape: pairs per distinct token
+        g_pairs_per_token = std::min(std::max((double)g_cols_runs / runs, 1.0), (double)nblk);
+        g_cols_N = 0;                                       // (used once: the next column report refreshes it)
+    }
+    return runs * std::min(g_pairs_per_token, (double)nblk) <= even ? 1 : -1;
+}
+}   // namespace
+
+void mi355_free_scatter_report(void) {
+    if (g_report) (void)hipHostFree(g_report);
+    g_report = g_report_dev = nullptr;
+}
+
+MI355_API int mi355_embed_scatter_add_form(int V, int D, int S, int batch, int aligned) {
+    if (!mi355_ready("embed_scatter_add_form")) return 0;
+    if (V <= 0 || D <= 0 || S <= 0 || batch <= 0 || (size_t)batch * S > (size_t)1 << 30) return 0;
+    const int N = batch * S;
+    const bool cols_ok = !g_ctx.scatter_tree && g_ctx.scatter_cols >= 0 && ((S % 4 == 0 && aligned) || N <= COL_SMALL) &&
+                         V < (1 << (32 - CB_BITS));
+    return scatter_form(N, D, cols_ok, N <= SMALL_N && key_bits(V) + POS_BITS <= 32);
+}
+
 MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, int V, int D, int S,
                                           int batch) {
     if (!mi355_ready("embed_scatter_add")) return -1;
@@ -850,15 +932,12 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     // Two forms with the same bits (embed_cols.h says what each costs).  Columns of dE owned by workgroups: dx is
     // read where it lies, nothing is copied; chosen where one round of workgroups covers D and the positions are few
     // enough that the small accesses to dE (one per token and workgroup) do not outweigh the copy.
-    if (!g_ctx.scatter_tree && g_ctx.scatter_cols >= 0 && ((S % 4 == 0 && aligned16(dx)) || N <= COL_SMALL) &&
-        V < (1 << (32 - CB_BITS))) {
-        const int cu = g_ctx.num_cu > 0 ? g_ctx.num_cu : 256;
-        // (also while a graph is recorded, for inputs whose row form would call the library sort, which cannot be)
-        const bool rows_recordable = N <= SMALL_N && key_bits(V) + POS_BITS <= 32;
-        if (g_ctx.scatter_cols > 0 || (N <= SMALL_N && (int)ceil_div((size_t)D, cols_per_workgroup(D)) <= cu) ||
-            (g_ctx.capturing && !rows_recordable))
-            return scatter_add_cols(dE, dx, ids, V, D, S, N);
-    }
+    const bool cols_ok = !g_ctx.scatter_tree && g_ctx.scatter_cols >= 0 &&
+                         ((S % 4 == 0 && aligned16(dx)) || N <= COL_SMALL) && V < (1 << (32 - CB_BITS));
+    // (the column form also while a graph is recorded, for inputs whose row form would call the library sort, which cannot be)
+    unsigned long long *report = scatter_report_word();
+    if (scatter_form(N, D, cols_ok, N <= SMALL_N && key_bits(V) + POS_BITS <= 32) > 0)
+        return scatter_add_cols(dE, dx, ids, V, D, S, N, report);
     const int bits = key_bits(V);
     const bool small = N <= SMALL_N && bits + POS_BITS <= 32;
     if (!small &&
@@ -936,10 +1015,10 @@ MI355_API int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int3
     const dim3 sgrid((unsigned)((size_t)long_x * nchunk_long + short_blocks));
     if (g_ctx.scatter_tree)
         hipLaunchKernelGGL(seg_sum_kernel<true>, sgrid, dim3(1024), 0, g_ctx.stream, dE, rows, seg_list, meta,
-                           long_list, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec);
+                           long_list, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec, report, N);
     else
         hipLaunchKernelGGL(seg_sum_kernel<false>, sgrid, dim3(1024), 0, g_ctx.stream, dE, rows, seg_list, meta,
-                           long_list, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec);
+                           long_list, D, nchunk, nchunk_long, long_x, (int)short_blocks, vec, report, N);
     LAUNCH_OK("embed_scatter_add segment sums");
     return 0;
 }

@@ -212,7 +212,8 @@ template <int K, bool FULL>                                     // FULL: D is a 
 __global__ __launch_bounds__(1024) void col_sum_kernel(float *dE, const float *__restrict__ dx,
                                                        const v2u *__restrict__ tasks,
                                                        const unsigned long long *__restrict__ cnt,
-                                                       const uint16_t *__restrict__ rk, int N, int D, int S, int nblk) {
+                                                       const uint16_t *__restrict__ rk, int N, int D, int S, int nblk,
+                                                       unsigned long long *report) {
     constexpr int XP = CB + 48;                                 // a column in LDS, with room for the reads issued ahead
     constexpr int NSL = (16 - K) * 64;                          // lanes that take short runs
     constexpr int RPL = 4;                                      // runs of a block whose old sums a lane asks for in one go
@@ -269,8 +270,10 @@ __global__ __launch_bounds__(1024) void col_sum_kernel(float *dE, const float *_
         h0 = dcol[(size_t)(hv ? o.pd[0].x : 0u) * D];
     }
     fetch_values(o, 0);
+    int runs = 0;
     for (int blk = 0; blk < nblk; blk++) {
         const int n_long = (int)(o.pc & 0xffffffffu), n_short = (int)(o.pc >> 32);
+        runs += n_long + n_short;
         const v2u *tb = tasks + (size_t)blk * CB;
         v2u dsc_[RPL];
 #pragma unroll
@@ -401,6 +404,8 @@ __global__ __launch_bounds__(1024) void col_sum_kernel(float *dE, const float *_
             }
         }
     }
+    // what the host looks at before it picks a form for the next call of this shape (one 8-byte store to host memory)
+    if (report && blockIdx.x == 0 && t == 0) *report = scatter_report(runs, N, D, 1);
 }
 
 // Up to COL_SMALL positions (one sequence of the reference's loops): plan and sums in ONE launch.  Every workgroup
@@ -489,12 +494,14 @@ __global__ __launch_bounds__(1024) void col_sum_small_kernel(float *dE, const fl
     }
 }
 
-// Columns of dE per workgroup: three from D = 513 on (256 workgroups at D = 768).
-int cols_per_workgroup(int D) { return D > 512 ? 3 : D > 256 ? 2 : 1; }
+// Columns of dE per workgroup: three from D = 513 on (256 workgroups at D = 768), four from 769 (256 at D = 1024:
+// 148 KB of LDS, the most a workgroup can hold of a block of 8192 positions).
+int cols_per_workgroup(int D) { return D > 768 ? 4 : D > 512 ? 3 : D > 256 ? 2 : 1; }
 
 // Launches the kernels of the column form.  The caller has checked: V < 2^(32 - CB_BITS) and, beyond COL_SMALL
 // positions, S a multiple of 4 and dx 16-byte aligned.
-int scatter_add_cols(float *dE, const float *dx, const int32_t *ids, int V, int D, int S, int N) {
+int scatter_add_cols(float *dE, const float *dx, const int32_t *ids, int V, int D, int S, int N,
+                     unsigned long long *report) {
     const int K = cols_per_workgroup(D);
     const dim3 grid((unsigned)ceil_div((size_t)D, K));
     if (N <= COL_SMALL) {
@@ -502,7 +509,7 @@ int scatter_add_cols(float *dE, const float *dx, const int32_t *ids, int V, int 
     case KK:                                                                                                        \
         hipLaunchKernelGGL(col_sum_small_kernel<KK>, grid, dim3(1024), 0, g_ctx.stream, dE, dx, ids, N, V, D, S);   \
         break;
-        switch (K) { COL_LAUNCH(1) COL_LAUNCH(2) COL_LAUNCH(3) }
+        switch (K) { COL_LAUNCH(1) COL_LAUNCH(2) COL_LAUNCH(3) COL_LAUNCH(4) }
 #undef COL_LAUNCH
         LAUNCH_OK("embed_scatter_add column sums");
         return 0;
@@ -533,13 +540,13 @@ int scatter_add_cols(float *dE, const float *dx, const int32_t *ids, int V, int 
     case KK:                                                                                                        \
         if (D % KK == 0)                                                                                            \
             hipLaunchKernelGGL((col_sum_kernel<KK, true>), grid, dim3(1024), 0, g_ctx.stream, dE, dx, tasks, cnt, rk, N, D, \
-                               S, nblk);                                                                            \
+                               S, nblk, report);                                                                    \
         else                                                                                                        \
             hipLaunchKernelGGL((col_sum_kernel<KK, false>), grid, dim3(1024), 0, g_ctx.stream, dE, dx, tasks, cnt, rk, N, D, \
-                               S, nblk);                                                                            \
+                               S, nblk, report);                                                                    \
         break;
     switch (K) {
-        COL_LAUNCH(1) COL_LAUNCH(2) COL_LAUNCH(3)
+        COL_LAUNCH(1) COL_LAUNCH(2) COL_LAUNCH(3) COL_LAUNCH(4)
     default: return mi355_fail("embed_scatter_add: no kernel for %d columns per workgroup", K);
     }
 #undef COL_LAUNCH

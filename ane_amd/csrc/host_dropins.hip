@@ -111,12 +111,14 @@ Table *resident_table(const char *who, const float *embed, int vocab, int dim) {
 }   // namespace
 
 void mi355_free_rope_cache(void);
+void mi355_free_scatter_report(void);
 
 void mi355_free_caches(void) {
     for (auto &s : g_slot) { if (s.dev) (void)hipFree(s.dev); s = Slot{}; }
     for (int i = 0; i < g_tab_n; i++) if (g_tab[i].dev) (void)hipFree(g_tab[i].dev);
     g_tab_n = 0;
     mi355_free_rope_cache();
+    mi355_free_scatter_report();
 }
 
 MI355_API void mi355_rmsnorm(float *out, const float *x, const float *w, int d, int S) {

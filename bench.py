@@ -560,6 +560,31 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
                      traffic_source="profiles/traffic.json (embed_config2)")
         return r
     tr_g, tr_s, tr_r = (traffic_bytes("embed_config2", EMBED_KERNELS[k]) for k in ("gather", "scatter_cols", "scatter_rows"))
+
+    # the same ids (drawn over its vocabulary) into the embedding table of the headline model, Qwen3-0.6B [151936,1024]
+    Vq, Dq = 151936, 1024
+    idq = zipf_ids(0, N, Vq).reshape(B, S)
+    Uq = int(np.unique(idq).size)
+    idqd = br.DevArray.from_numpy(idq)
+    gq = [br.DevArray((B, Dq, S)) for _ in range(3)]
+    dEq = [br.DevArray((Vq, Dq)) for _ in range(3)]
+    for i, g in enumerate(gq):
+        br.check(br.lib.mi355_fill_normal_dev(g.ptr, g.size, 30 + i, 0.0, 1.0))
+    for d in dEq:
+        d.zero()
+
+    def scatter_q():
+        for g, dE in zip(gq, dEq):
+            br.check(br.lib.mi355_embed_scatter_add_dev(dE.ptr, g.ptr, idqd.ptr, Vq, Dq, S, B))
+    scatter_q(); scatter_q()
+    t_q = time_region(br, scatter_q, steps) / 3
+    br.tune("scatter_cols", -1)
+    scatter_q()
+    t_q_rows = time_region(br, scatter_q, steps) / 3
+    br.tune("scatter_cols", 0)
+    b_q = 4 * Dq * N + 8 * Dq * Uq + 4 * N
+    for a in gq + dEq + [idqd]:
+        a.free()
     out = {"metric": "embedding gather + ordered scatter-add (BASELINE.json config 2)", "value": N / ((t_g + t_s) / 1e3),
            "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": t_g + t_s,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32+i32", "data": "synthetic",
@@ -574,6 +599,8 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
                    row("embed_scatter_add (scatter_cols=-1, scatter_tree=1)", t_s_tree, b_s),
                    row("embed_scatter_add, one sequence of 256 ids", t_s1, b_s1),
                    row("embed_scatter_add, one sequence of 256 ids (scatter_cols=-1)", t_s1_rows, b_s1),
+                   row("embed_scatter_add into [151936,1024] (Qwen3-0.6B's table), 64x256 Zipf ids", t_q, b_q),
+                   row("embed_scatter_add into [151936,1024] (scatter_cols=-1)", t_q_rows, b_q),
                    row("copy of one activation slab", t_c, 8 * D * N)],
            "roofline": dict(bound="hbm", kernel="embed_scatter_add (3 launches: chunk sort, ranks, column sums)", achieved=b_s / t_s / 1e6, peak=PEAK_HBM_GBS,
                             unit="GB/s", frac=b_s / t_s / 1e6 / PEAK_HBM_GBS,

@@ -279,10 +279,18 @@ int mi355_embed_gather_dev(float *x, const float *E, const int32_t *ids, int V, 
  * bit-identical to the reference loop and run-to-run deterministic.  Ids outside [0,V) are skipped.
  * Two forms give the same bits: up to 16384 positions (S a multiple of 4, V < 2^19, D within one round of workgroups)
  * every workgroup owns a few columns of dE and reads its rows of dx in place; otherwise dx is first copied
- * token-major and summed row by row (the "scatter_cols" knob names a form).  While a graph is recorded, inputs beyond
- * 16384 positions take the first form too (the library sort of the second cannot be recorded). */
+ * token-major and summed row by row (the "scatter_cols" knob names a form).  The first form costs by the number of
+ * distinct (token, block of 8192 positions) pairs and is the default; every call leaves that number in a word of
+ * pinned host memory, and the next call with the same number of positions and D takes the second form if the ids
+ * repeated too little for the first (and returns when they repeat again): same bits, only the time differs.
+ * While a graph is recorded, inputs beyond 16384 positions take the first form too (the library sort of the second
+ * cannot be recorded). */
 int mi355_embed_scatter_add_dev(float *dE, const float *dx, const int32_t *ids, int V, int D,
                                 int S, int batch);
+/* Which form the next mi355_embed_scatter_add_dev call of this shape would take under the current knobs and the last
+ * call's report: 1 = columns of dE owned by workgroups, -1 = token-major copy and row sums, 0 = bad shape.  `aligned`:
+ * dx is 16-byte aligned.  No counterpart in the reference (its op is one loop); for tests and tuning. */
+int mi355_embed_scatter_add_form(int V, int D, int S, int batch, int aligned);
 
 /* Fused softmax + cross-entropy forward/backward on logits [V][S].  Replaces cross_entropy_loss —
  * training/training_dynamic/cpu_ops.h:68-93, training/stories_cpu_ops.h:71-108 — and the loss-scale

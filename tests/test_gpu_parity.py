@@ -567,6 +567,9 @@ def test_embed_gather_bit_exact(br, V, D, B, S, oob):
     (524287, 6, 3, 3000, 2),      # the largest vocabulary of the column form; a partial second block of positions
     (2000, 770, 5, 4096, 0),      # 20480 positions, 257 workgroups of three columns, the last with two
     (40, 515, 1, 8192, 0),        # exactly one block; one column left over for the last workgroup
+    (32000, 1024, 64, 256, 2),    # the width of Qwen3-0.6B: four columns per workgroup, 256 workgroups
+    (700, 1000, 3, 1000, 0),      # four columns, 250 workgroups, three runs of ~4 per token and block
+    (90, 1022, 2, 2052, 1),       # four columns, the last workgroup with two
     (100, 7, 2, 256, 0),          # 512 positions: the most the single-launch column kernel takes
     (100, 7, 4, 129, 1),          # 516: one more (S not a multiple of 4: row form)
     (3000, 770, 1, 511, 3),       # single launch, S odd, 257 workgroups, the last with two columns
@@ -593,6 +596,48 @@ def test_embed_scatter_add_bit_exact_and_deterministic(br, V, D, B, S, oob):
             br.tune("scatter_cols", 0)
         assert outs[0].tobytes() == outs[1].tobytes(), form            # run-to-run deterministic
         assert outs[0].tobytes() == ref.tobytes(), form                # the ordered fp32 sum of the reference loop
+
+
+def test_embed_scatter_add_form_follows_how_the_ids_repeat(br):
+    """Left to itself the library takes the column form, whose cost goes by the distinct (token, block) pairs, learns
+    from each call's report how the ids repeated, and moves an input that hardly repeats to the row form (and back).
+    Same bytes whichever form runs."""
+    V, D, B, S = 32000, 768, 64, 256
+    say("scatter_add form choice V=%d D=%d B=%d S=%d" % (V, D, B, S))
+    zipf = H.zipf_ids(3, B * S, V).astype(np.int32).reshape(B, S)
+    flat = np.random.default_rng(4).integers(0, V, (B, S)).astype(np.int32)
+    dx = H.normal(65, (B, D, S)); dE0 = H.normal(66, (V, D), 0, 0.5)
+    dxd = dev(br, dx)
+    form = lambda: br.lib.mi355_embed_scatter_add_form(V, D, S, B, 1)
+
+    def call(ids):
+        dEd = dev(br, dE0)
+        br.check(br.lib.mi355_embed_scatter_add_dev(dEd.ptr, dxd.ptr, dev(br, ids).ptr, V, D, S, B))
+        br.sync()                                  # the report of this call is in host memory now
+        return dEd.numpy().tobytes()
+
+    try:
+        br.tune("scatter_cols", 1)
+        ref_zipf = call(zipf)                      # a column-form report of this shape: a known starting point
+        br.tune("scatter_cols", 0)
+        assert ref_zipf == O.embed_backward(dE0, dx, zipf).tobytes()
+        assert form() == 1
+        ref_flat = O.embed_backward(dE0, dx, flat).tobytes()
+        assert call(flat) == ref_flat              # (ran in the column form)
+        assert form() == -1                        # ~12800 distinct ids in 16384 positions: the row form next
+        assert call(flat) == ref_flat and form() == -1      # ... and it stays there
+        assert call(zipf) == ref_zipf              # (ran in the row form)
+        assert form() == 1                         # ids that repeat: back to the columns
+        assert call(zipf) == ref_zipf and form() == 1
+        br.tune("scatter_cols", -1)
+        assert form() == -1 and call(zipf) == ref_zipf
+        br.tune("scatter_cols", 0)
+        assert form() == 1                         # a forced call of the other form leaves a report too
+        assert br.lib.mi355_embed_scatter_add_form(0, D, S, B, 1) == 0
+        assert br.lib.mi355_embed_scatter_add_form(V, D, 255, B, 1) == -1      # S not a multiple of 4: rows only
+        assert br.lib.mi355_embed_scatter_add_form(V, D, S, 100, 1) == -1      # 25600 positions: rows only
+    finally:
+        br.tune("scatter_cols", 0)
 
 
 def test_embed_scatter_add_tree_order_is_deterministic_and_close(br):
