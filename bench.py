@@ -496,7 +496,7 @@ def zipf_ids(seed, n, vocab, s=1.1):
     return np.minimum(np.searchsorted(cdf, u, side="right"), vocab - 1).astype(np.int32)
 
 
-def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
+def measure_embed(br, steps, warmup, with_cpu, nbuf=6, other_tables=True):
     """BASELINE.json config 2: vocab 32000 x dim 768 table, 64 sequences x 256 Zipf(1.1) ids; gather + ordered
     scatter-add.  Returns the JSON object of that workload."""
     V, D, B, S = 32000, 768, 64, 256
@@ -562,29 +562,34 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
     tr_g, tr_s, tr_r = (traffic_bytes("embed_config2", EMBED_KERNELS[k]) for k in ("gather", "scatter_cols", "scatter_rows"))
 
     # the same ids (drawn over its vocabulary) into the embedding table of the headline model, Qwen3-0.6B [151936,1024]
-    Vq, Dq = 151936, 1024
-    idq = zipf_ids(0, N, Vq).reshape(B, S)
-    Uq = int(np.unique(idq).size)
-    idqd = br.DevArray.from_numpy(idq)
-    gq = [br.DevArray((B, Dq, S)) for _ in range(3)]
-    dEq = [br.DevArray((Vq, Dq)) for _ in range(3)]
-    for i, g in enumerate(gq):
-        br.check(br.lib.mi355_fill_normal_dev(g.ptr, g.size, 30 + i, 0.0, 1.0))
-    for d in dEq:
-        d.zero()
+    # (left out of the profiled runs, whose per-kernel figures are config 2's)
+    extra = []
+    if other_tables:
+        Vq, Dq = 151936, 1024
+        idq = zipf_ids(0, N, Vq).reshape(B, S)
+        Uq = int(np.unique(idq).size)
+        idqd = br.DevArray.from_numpy(idq)
+        gq = [br.DevArray((B, Dq, S)) for _ in range(3)]
+        dEq = [br.DevArray((Vq, Dq)) for _ in range(3)]
+        for i, g in enumerate(gq):
+            br.check(br.lib.mi355_fill_normal_dev(g.ptr, g.size, 30 + i, 0.0, 1.0))
+        for d in dEq:
+            d.zero()
 
-    def scatter_q():
-        for g, dE in zip(gq, dEq):
-            br.check(br.lib.mi355_embed_scatter_add_dev(dE.ptr, g.ptr, idqd.ptr, Vq, Dq, S, B))
-    scatter_q(); scatter_q()
-    t_q = time_region(br, scatter_q, steps) / 3
-    br.tune("scatter_cols", -1)
-    scatter_q()
-    t_q_rows = time_region(br, scatter_q, steps) / 3
-    br.tune("scatter_cols", 0)
-    b_q = 4 * Dq * N + 8 * Dq * Uq + 4 * N
-    for a in gq + dEq + [idqd]:
-        a.free()
+        def scatter_q():
+            for g, dE in zip(gq, dEq):
+                br.check(br.lib.mi355_embed_scatter_add_dev(dE.ptr, g.ptr, idqd.ptr, Vq, Dq, S, B))
+        scatter_q(); scatter_q()
+        t_q = time_region(br, scatter_q, steps) / 3
+        br.tune("scatter_cols", -1)
+        scatter_q()
+        t_q_rows = time_region(br, scatter_q, steps) / 3
+        br.tune("scatter_cols", 0)
+        b_q = 4 * Dq * N + 8 * Dq * Uq + 4 * N
+        for a in gq + dEq + [idqd]:
+            a.free()
+        extra = [("embed_scatter_add into [151936,1024] (Qwen3-0.6B's table), 64x256 Zipf ids", t_q, b_q),
+                 ("embed_scatter_add into [151936,1024] (scatter_cols=-1)", t_q_rows, b_q)]
     out = {"metric": "embedding gather + ordered scatter-add (BASELINE.json config 2)", "value": N / ((t_g + t_s) / 1e3),
            "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": t_g + t_s,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32+i32", "data": "synthetic",
@@ -599,8 +604,7 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
                    row("embed_scatter_add (scatter_cols=-1, scatter_tree=1)", t_s_tree, b_s),
                    row("embed_scatter_add, one sequence of 256 ids", t_s1, b_s1),
                    row("embed_scatter_add, one sequence of 256 ids (scatter_cols=-1)", t_s1_rows, b_s1),
-                   row("embed_scatter_add into [151936,1024] (Qwen3-0.6B's table), 64x256 Zipf ids", t_q, b_q),
-                   row("embed_scatter_add into [151936,1024] (scatter_cols=-1)", t_q_rows, b_q),
+                   *[row(*e) for e in extra],
                    row("copy of one activation slab", t_c, 8 * D * N)],
            "roofline": dict(bound="hbm", kernel="embed_scatter_add (3 launches: chunk sort, ranks, column sums)", achieved=b_s / t_s / 1e6, peak=PEAK_HBM_GBS,
                             unit="GB/s", frac=b_s / t_s / 1e6 / PEAK_HBM_GBS,
@@ -622,7 +626,7 @@ def measure_embed(br, steps, warmup, with_cpu, nbuf=6):
 
 
 def bench_embed(br, args):
-    print(json.dumps(measure_embed(br, args.steps, args.warmup, args.cpu_layers > 0)))
+    print(json.dumps(measure_embed(br, args.steps, args.warmup, args.cpu_layers > 0, other_tables=not args.config2_only)))
 
 
 def measure_optimizer(br, steps, warmup, nset=8):
@@ -846,6 +850,8 @@ def main():
                          "(BASELINE.json configs 0/1: one [C,256] sequence per op, 12 layers, RoPE without QK-norm); "
                          "embed = BASELINE.json config 2; optimizer = the Adam tail (each prints its own JSON line)")
     ap.add_argument("--batch", type=int, default=0, help="sequences per op (default: 16 for qwen3, 1 for stories110m)")
+    ap.add_argument("--config2-only", action="store_true",
+                    help="--workload embed: BASELINE.json config 2 alone, without the rows for other tables (for profiles)")
     ap.add_argument("--headline-only", action="store_true",
                     help="default workload only: skip the other BASELINE.json configurations (embedding config 2, the "
                          "Stories110M shapes of configs 0/1, the optimizer tail) that a default run appends to its line")
