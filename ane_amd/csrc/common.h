@@ -48,7 +48,7 @@ bool mi355_outside_capture(const char *who);
 // Workspace of at least `bytes` (256-byte aligned), NULL on failure.
 void *mi355_ws(size_t bytes);
 // Exchange area for kernels whose workgroups pass values to one another inside one launch (the clustered
-// RMSNorm, the single-launch INT8 scale): 8-byte slots {fp32 value, tag}, XCH_SLOT_STRIDE per workgroup number, and
+// RMSNorm, the single-launch INT8 scale and scale + quantize): 8-byte slots {fp32 value, tag}, XCH_SLOT_STRIDE per workgroup number, and
 // one launch counter per workgroup number; norm_cluster.h describes the protocol.  Allocated and zeroed on first
 // use (not possible during a graph capture); false with the error recorded on failure.
 constexpr int XCH_SLOT_STRIDE = 256;

@@ -82,8 +82,8 @@ bool mi355_exchange(Mi355Exchange *out) {
 // show as launches that each take the bounded wait and then read their operands several times.  mi355_sync(), which
 // waits anyway, therefore looks at the two counters after such kernels have run: when they have grown at three checks
 // in a row with no tuning knob changed in between, the cooperating forms are switched off for the rest of the process
-// (the single-workgroup RMSNorm tiles, the two-launch INT8 scale, the three-launch cross-entropy take over) and one
-// line says so.  A change of a tuning knob starts the count afresh, and the test mode that refuses every value is not
+// (the single-workgroup RMSNorm tiles, the two-launch INT8 scale and quantizer, the three-launch cross-entropy take
+// over) and one line says so.  A change of a tuning knob starts the count afresh, and the test mode that refuses every value is not
 // counted.
 static bool g_coop_launched = false, g_coop_rebase = true;
 static long long g_coop_seen = 0;

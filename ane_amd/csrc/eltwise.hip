@@ -433,6 +433,96 @@ __global__ __launch_bounds__(EW_THREADS) void quant_dyn_kernel(int *__restrict__
         }
     }
 }
+
+// The reference's quantizer as it is written (bridge/ane_bridge.m:346-365: the maximum of |x|, then the rounding) in
+// ONE launch that reads x once: a workgroup keeps its share of the tensor in registers (PER groups of four per
+// thread), publishes the maximum of it as absmax_scale_kernel does, gathers every workgroup's, and quantizes what
+// it holds.  The maximum is exact in any order, so every workgroup computes the same scale and the bytes are those of
+// the two separate steps.  A workgroup whose wait for another's maximum expires takes the maximum of the whole tensor
+// itself.  (A workgroup raises its launch counter only after it has gathered everyone's maximum, that is after every
+// other workgroup has started and read that counter: nobody can be taken for absent because it was too fast.)
+template <int PER>
+__global__ __launch_bounds__(1024) void quant_dyn_one_kernel(int *__restrict__ q4, float *__restrict__ scale_out,
+                                                             const float *__restrict__ x, size_t n, size_t n4,
+                                                             int rounding, Mi355Exchange ws, int spin_ticks) {
+    __shared__ float red[16];
+    __shared__ int failed;
+    const int nblk = (int)gridDim.x, blk = (int)blockIdx.x, t = (int)threadIdx.x;
+    if (t == 0) failed = 0;
+    unsigned want = 0;
+    if (t < nblk) want = ws.cnt[t] + 1u;
+    const unsigned my_tag = ws.cnt[blk] + 1u;
+    v4f a[PER];
+#pragma unroll
+    for (int u = 0; u < PER; u++) {
+        const size_t i = ((size_t)u * nblk + blk) * 1024 + t;
+        const v4f zero = {0.f, 0.f, 0.f, 0.f};
+        a[u] = i < n4 ? ld4_nt(x + 4 * i) : zero;
+    }
+    auto block_max = [&](float m) {          // maximum over the workgroup, in every thread
+        m = wave_max(m);
+        __syncthreads();
+        if ((t & 63) == 0) red[t >> 6] = m;
+        __syncthreads();
+        float r = red[0];
+#pragma unroll
+        for (int k = 1; k < 16; k++) r = fmaxf(r, red[k]);
+        return r;
+    };
+    float m = 0.f;
+    if (blk == 0 && n4 * 4 + t < n) m = fabsf(x[n4 * 4 + t]);       // the few elements behind the last whole group
+#pragma unroll
+    for (int u = 0; u < PER; u++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) m = fmaxf(m, fabsf(a[u][j]));
+    m = block_max(m);
+    if (t == 0)
+        __hip_atomic_store(&ws.slots[(size_t)blk * XCH_SLOT_STRIDE], ((unsigned long long)my_tag << 32) | __float_as_uint(m),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    float g = 0.f;
+    if (t < nblk) {
+        const unsigned long long *sp = &ws.slots[(size_t)t * XCH_SLOT_STRIDE];
+        const long long t0 = wall_clock64();
+        unsigned long long pk;
+        bool ok = false;
+        for (;;) {
+            pk = __hip_atomic_load(sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (spin_ticks < 0) break;                            // test mode: whatever the slot holds is refused
+            if ((unsigned)(pk >> 32) == want) { ok = true; break; }
+            if (wall_clock64() - t0 >= (long long)spin_ticks) break;
+            __builtin_amdgcn_s_sleep(2);
+        }
+        if (!ok) failed = 1;
+        g = __uint_as_float((unsigned)pk);
+    }
+    g = block_max(g);
+    if (failed) {                                                 // (block-uniform: read after the barriers above)
+        if (t == 0) atomicAdd(ws.fallbacks, 1);
+        float w = 0.f;
+        for (size_t i = t; i < n4; i += 1024) {
+            const v4f v = ld4(x + 4 * i);
+#pragma unroll
+            for (int j = 0; j < 4; j++) w = fmaxf(w, fabsf(v[j]));
+        }
+        for (size_t i = n4 * 4 + t; i < n; i += 1024) w = fmaxf(w, fabsf(x[i]));
+        g = block_max(w);
+    }
+    float scale = g / 127.0f;
+    if (scale == 0.0f) scale = 1.0f;
+    if (blk == 0 && t == 0) *scale_out = scale;
+#pragma unroll
+    for (int u = 0; u < PER; u++) {
+        const size_t i = ((size_t)u * nblk + blk) * 1024 + t;
+        if (i < n4) {
+            unsigned int pk = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) pk |= ((unsigned int)(quant1(a[u][j], scale, rounding) & 0xFF)) << (8 * j);
+            q4[i] = (int)pk;
+        }
+    }
+    if (t == 0) ws.cnt[blk] = my_tag;
+}
+
 template <int UNROLL>
 __global__ __launch_bounds__(EW_THREADS) void dequant_kernel(float *__restrict__ x, const int *__restrict__ q4,
                                                              const float *__restrict__ scale_p, size_t n4) {
@@ -789,6 +879,30 @@ MI355_API int mi355_int8_quantize_dynamic_dev(int8_t *q, float *scale_dev, const
     if (n4 == 0) {      // no vector body: the two separate steps
         if (mi355_int8_scale_dev(scale_dev, x, n)) return -1;
         return mi355_int8_quant_dev(q, x, scale_dev, n, rounding);
+    }
+    {
+        // one launch while a workgroup per compute unit can hold the tensor in registers (up to 8 groups of four per
+        // thread: 8.4 M floats on 256 compute units); "rms_cluster" = -1 switches the cooperating forms off
+        const size_t cus = g_ctx.num_cu > 0 ? (size_t)g_ctx.num_cu : 256;
+        size_t nb = std::min(std::min(ceil_div(n4, (size_t)1024), cus), (size_t)XCH_MAX_BLOCKS);
+        const size_t per = ceil_div(n4, nb * 1024);
+        if (g_ctx.rms_cluster >= 0 && per <= 8) {
+            Mi355Exchange xch;
+            if (!mi355_exchange(&xch)) return -1;
+            const int spin = mi355_exchange_spin_ticks();
+#define QDYN(P)                                                                                                        \
+    hipLaunchKernelGGL(quant_dyn_one_kernel<P>, dim3((unsigned)nb), dim3(1024), 0, g_ctx.stream, (int *)q, scale_dev, x, n, \
+                       n4, rounding, xch, spin)
+            if (per <= 1) QDYN(1); else if (per <= 2) QDYN(2); else if (per <= 4) QDYN(4); else QDYN(8);
+#undef QDYN
+            LAUNCH_OK("int8_quantize_dynamic");
+            if (lo < n) {
+                hipLaunchKernelGGL(quant_scalar, dim3((unsigned)ceil_div(n - lo, 256)), dim3(256), 0, g_ctx.stream, q, x,
+                                   scale_dev, lo, n, rounding);
+                LAUNCH_OK("int8_quantize_dynamic tail");
+            }
+            return 0;
+        }
     }
     size_t blocks = ceil_div(n4, (size_t)EW_THREADS);
     if (blocks > 256) blocks = 256;         // one workgroup per compute unit; few maxima for the quantizer to fold

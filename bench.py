@@ -49,6 +49,7 @@ OP_KERNELS = {
     "int8_scale": [("absmax_scale_kernel", 1.0)],
     "int8_quant": [("quant_kernel<1>", 1.0)],
     "int8_dequant": [("dequant_kernel<1>", 1.0)],
+    "int8_quantize_dynamic": [("quant_dyn_one_kernel<4>", 1.0)],
 }
 # BASELINE.json config 2: the three launches of the ordered scatter-add in its column form and in its row form, and
 # the gather
@@ -103,7 +104,7 @@ def alg_bytes(cfg, a=4):
         "int8_scale": 4 * n8,
         "int8_quant": 5 * n8,
         "int8_dequant": 5 * n8,
-        "int8_quantize_dynamic": 9 * n8,     # the scale's read and the quantizer's read + write in two launches
+        "int8_quantize_dynamic": 5 * n8,     # one launch that reads x once (the tensor stays in registers) and writes q
     }
 
 

@@ -63,8 +63,8 @@ size_t mi355_workspace_size(void);
  * of the gradient table and reads its rows of dx in place: 1 = for any number of positions, -1 = never),
  * "buf_phase" (where mi355_buf_alloc starts buffers of 1 MiB and more within a 1 KiB group:
  * 0 = a multiple of 128 bytes that rotates from one allocation to the next, 1..8 = always (value-1)*128),
- * "rms_cluster" (channel split of the RMSNorm over cooperating workgroups: -1 = never, and mi355_int8_scale_dev then
- * runs as two launches; 2/4/8 = forced),
+ * "rms_cluster" (channel split of the RMSNorm over cooperating workgroups: -1 = never, and mi355_int8_scale_dev and
+ * mi355_int8_quantize_dynamic_dev then run as two launches each; 2/4/8 = forced),
  * "ce_resident" (one-launch softmax-CE: 1 = for any V, -1 = never), "rms_cluster_spin" (how long a workgroup of those
  * kernels and of mi355_int8_scale_dev waits for a partner's partial result before it computes it itself, in ticks
  * of 10 ns: 0 = 2 ms; -1 = do not wait), "xch_take_nothing" (1: those kernels take no partner's value at
@@ -341,8 +341,9 @@ int mi355_minmax_dev(float *out3_dev, const float *x, size_t n);
  * half-to-even (rounding 0) or half away from zero (rounding 1, the reference's); x^ = q*scale. */
 int mi355_int8_scale_dev(float *scale_dev, const float *x, size_t n);
 int mi355_int8_quant_dev(int8_t *q, const float *x, const float *scale_dev, size_t n, int rounding);
-/* The activation path of W8A8 in one call: scale = max|x|/127 (written to scale_dev) and q = quantize(x, scale),
- * two launches instead of the three of mi355_int8_scale_dev + mi355_int8_quant_dev; same bytes out. */
+/* The quantizer of bridge/ane_bridge.m:346-365 as one call (the activation path of W8A8): scale = max|x|/127 (written
+ * to scale_dev) and q = quantize(x, scale); one launch that reads x once up to 8.4 M floats, two beyond; the same
+ * bytes out as mi355_int8_scale_dev + mi355_int8_quant_dev. */
 int mi355_int8_quantize_dynamic_dev(int8_t *q, float *scale_dev, const float *x, size_t n, int rounding);
 int mi355_int8_dequant_dev(float *x, const int8_t *q, const float *scale_dev, size_t n);
 

@@ -749,18 +749,37 @@ def test_embed_scatter_add_column_form_runs_that_change_length(br):
     assert dEd.numpy().tobytes() == O.embed_backward(dE0, dx, ids).tobytes()
 
 
-@pytest.mark.parametrize("n", [1024 * 4096, 13, 4099, 3, 1024 * 1024 * 5 + 2])
+@pytest.mark.parametrize("n", [1024 * 4096, 13, 4099, 3, 1024 * 1024 * 5 + 2, 9 * 1024 * 1024 + 4])
 @pytest.mark.parametrize("rounding", [0, 1])
 def test_int8_quantize_dynamic_equals_scale_then_quant(br, n, rounding):
+    """The reference's quantizer (maximum, then rounding) in one call: up to 8.4 M floats one launch whose workgroups
+    keep the tensor in registers and hand one another their maxima; the same bytes as the two separate steps and the
+    oracle, also when every wait is made to expire or every maximum is refused, and the counter says which it was."""
     x = H.normal(72, n) * np.float32(3.0)
     if n > 8: x[5] = np.float32(-11.0)
+    if n > 4096: x[n - 2] = np.float32(12.5)            # the maximum among the last elements (n % 4 != 0: in the tail)
     xd = dev(br, x)
     s1 = br.DevArray(1); q1 = br.DevArray(n, np.int8)
     br.check(br.lib.mi355_int8_scale_dev(s1.ptr, xd.ptr, n))
     br.check(br.lib.mi355_int8_quant_dev(q1.ptr, xd.ptr, s1.ptr, n, rounding))
     s2 = br.DevArray(1); q2 = br.DevArray(n, np.int8)
-    br.check(br.lib.mi355_int8_quantize_dynamic_dev(q2.ptr, s2.ptr, xd.ptr, n, rounding))
-    assert s2.numpy().tobytes() == s1.numpy().tobytes() and q2.numpy().tobytes() == q1.numpy().tobytes()
+    one_launch = 4 <= n <= 8 * 1024 * 1024
+    # workgroups that wait for one another: those of the one launch; below four elements the scale kernel's one
+    blocks = min(-(-(n // 4) // 1024), br.device_info()[2]) if one_launch else (1 if n < 4 else 0)
+    try:
+        for spin, refuse in ((0, 0), (-1, 0), (0, 1)):
+            br.tune("rms_cluster_spin", spin); br.tune("xch_take_nothing", refuse)
+            s2.upload(np.zeros(1, np.float32)); q2.upload(np.zeros(n, np.int8))
+            expired = br.exchange_fallbacks()[0]
+            br.check(br.lib.mi355_int8_quantize_dynamic_dev(q2.ptr, s2.ptr, xd.ptr, n, rounding))
+            assert s2.numpy().tobytes() == s1.numpy().tobytes() and q2.numpy().tobytes() == q1.numpy().tobytes(), (spin, refuse)
+            if spin == 0:       # handed over in the normal run; every workgroup on its own when it refuses the others' maxima
+                assert br.exchange_fallbacks()[0] - expired == blocks * refuse, (refuse, blocks)
+        br.tune("rms_cluster", -1)                       # the cooperating forms switched off: two launches
+        br.check(br.lib.mi355_int8_quantize_dynamic_dev(q2.ptr, s2.ptr, xd.ptr, n, rounding))
+        assert s2.numpy().tobytes() == s1.numpy().tobytes() and q2.numpy().tobytes() == q1.numpy().tobytes()
+    finally:
+        br.tune("rms_cluster_spin", 0); br.tune("xch_take_nothing", 0); br.tune("rms_cluster", 0)
     sc = O.int8_scale(x)
     assert np.float32(sc) == s2.numpy()[0] and np.array_equal(q2.numpy(), O.int8_quant(x, sc, rounding))
     z = dev(br, np.zeros(64, np.float32))               # all zeros: scale 1
