@@ -332,3 +332,30 @@ def test_bf16_rope_random_shapes(br, B, heads, kvh, hd, S):
 def test_bf16_softmax_ce_random_shapes(br, V, S):
     import test_gpu_bf16 as BF
     BF.test_softmax_ce_bf16(br, V, S)
+
+
+def _helper_cases():
+    """Random shapes for the helpers either side of the path (bit-exact ops): GQA tile / reduce, fp16 rectangle converts
+    with pitches, vocabulary compaction rows, the map build and the one-pass attention-gradient finish."""
+    rng = np.random.default_rng(555 + SEED)
+    out = []
+    for _ in range(5 * MORE):
+        kvh = int(rng.integers(1, 5)); ratio = int(rng.integers(1, 5))
+        hd = int(rng.choice([2, 4, 6, 8, 16, 64, 128])); S = int(rng.choice([rng.integers(1, 40), 4 * rng.integers(1, 70)]))
+        rows = int(rng.integers(1, 300)); cols = int(rng.integers(1, 600))
+        out.append((int(rng.integers(1, 4)), kvh, ratio, hd, S, rows, cols, cols + int(rng.integers(0, 40)),
+                    cols + int(rng.integers(0, 40)), int(rng.choice([5, 300, 1031, 32000])),
+                    int(rng.choice([1, 6, 64, 250, 1024])), int(rng.integers(1, 5000)), int(rng.integers(0, 2))))
+    return out
+
+
+@pytest.mark.parametrize("B,kvh,ratio,hd,S,rows,cols,dst_ld,src_ld,V,D,ntok,in_f16", _helper_cases())
+def test_helper_ops_random_shapes(br, B, kvh, ratio, hd, S, rows, cols, dst_ld, src_ld, V, D, ntok, in_f16):
+    print("[case] helpers B=%d kvh=%d ratio=%d hd=%d S=%d | cvt %dx%d ld %d/%d | vocab V=%d D=%d ntok=%d | f16 in %d"
+          % (B, kvh, ratio, hd, S, rows, cols, dst_ld, src_ld, V, D, ntok, in_f16), flush=True)
+    import test_gpu_parity as P
+    P.test_gqa_tile_reduce(br, B, kvh, ratio, hd, S)
+    P.test_cvt_rectangles(br, rows, cols, dst_ld, src_ld)
+    P.test_vocab_compaction_bit_exact(br, V, D, ntok)
+    P.test_vocab_map_build_and_remap_exact(br, V, ntok)
+    P.test_attn_grads_finish_equals_separate_steps(br, B, kvh * ratio, kvh, hd, S, in_f16)
