@@ -3,10 +3,10 @@
 //
 // embed_backward (training/stories_cpu_ops.h:123-131, training/training_dynamic/cpu_ops.h:158-164) adds dx[:,t] into
 // dE[tok_t] for t ascending: every (row, d) sum has one fixed fp32 order, and the columns d are independent of one
-// another.  Here a workgroup owns K adjacent columns of dE (K = 3 for D = 768 on 256 compute units) and sees every
-// position: its part of dx is K whole rows of every sequence, contiguous in the channel-first layout, so dx is read
-// once, coalesced, by exactly one workgroup, and nothing is copied token-major through memory.  The positions are
-// taken in blocks of CB, in order; within a block they are ranked by (token, position), so a token's positions form
+// another.  Here a workgroup owns K adjacent columns of dE (K = 3 for D = 768, 4 for D = 1024, on 256 compute units)
+// and sees every position: its part of dx is K whole rows of every sequence, contiguous in the channel-first layout,
+// so dx is read once, coalesced, by exactly one workgroup, and nothing is copied token-major through memory.  The
+// positions are taken in blocks of CB, in order; within a block they are ranked by (token, position), so a token's positions form
 // a run of consecutive ranks, and a lane adds a run to dE[token][d] sequentially: acc = dE; acc += x[rank] for the
 // ranks ascending; dE = acc.  Blocks in ascending order and ranks ascending within a run are the order of the
 // reference loop, so the result is that loop's bit for bit.
@@ -20,9 +20,10 @@
 //      block was summed) to LDS at their ranks, so that a run is a contiguous piece of an LDS column.  Waves 0..K-1
 //      take the long runs of one column each (128-bit LDS reads issued sixteen adds ahead); the other waves take the
 //      short runs, K columns to a lane, the old sums of a lane's runs asked for before the block's values are put in
-//      their places.  A long run's result also stays in LDS under its token, so the run of the
-//      same token in the next block starts from there and not from a load of dE: the chain of the most frequent
-//      token, which bounds the whole operation, goes on from block to block without a trip to memory.
+//      their places.  A long run's result also stays in LDS under its token, so the run of the same token in the
+//      next block starts from there and not from a load of dE: the chain of the most frequent token, which bounds
+//      the whole operation, goes on from block to block without a trip to memory.  The last thing the launch does is
+//      to leave the number of runs it saw where the host finds it before the next call (see scatter_form in embed.hip).
 #pragma once
 
 constexpr int CB = 8192, CB_BITS = 13;      // positions per block
