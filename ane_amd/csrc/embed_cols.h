@@ -6,10 +6,10 @@
 // another.  Here a workgroup owns K adjacent columns of dE (K = 3 for D = 768, 4 for D = 1024, on 256 compute units)
 // and sees every position: its part of dx is K whole rows of every sequence, contiguous in the channel-first layout,
 // so dx is read once, coalesced, by exactly one workgroup, and nothing is copied token-major through memory.  The
-// positions are taken in blocks of CB, in order; within a block they are ranked by (token, position), so a token's positions form
-// a run of consecutive ranks, and a lane adds a run to dE[token][d] sequentially: acc = dE; acc += x[rank] for the
-// ranks ascending; dE = acc.  Blocks in ascending order and ranks ascending within a run are the order of the
-// reference loop, so the result is that loop's bit for bit.
+// positions are taken in blocks of CB, in order; within a block they are ranked by (token, position), so a token's
+// positions form a run of consecutive ranks, and a lane adds a run to dE[token][d] sequentially: acc = dE;
+// acc += x[rank] for the ranks ascending; dE = acc.  Blocks in ascending order and ranks ascending within a run are
+// the order of the reference loop, so the result is that loop's bit for bit.
 //
 // Three launches (one, col_sum_small_kernel, up to 512 positions):
 //   1. chunk_sort_blk_kernel: every 256 consecutive (token, position-in-block) words sorted by counting.
